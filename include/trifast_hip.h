@@ -1,0 +1,128 @@
+/*
+ * trifast_hip.h -- C ABI of the MI355X (gfx950) triangle self-attention kernels.
+ *
+ * This is the boundary that replaces the host->device launches of the reference
+ * operator (reference src/trifast/torch.py:48-59 for forward, :111-174 for the
+ * three backward launches): raw device pointers, element strides, sizes, a dtype
+ * code, a tile id and a HIP stream.  No torch types cross it.
+ *
+ * Conventions
+ *   - Every entry point returns 0 on success, a negative TRIFAST_E* code for a
+ *     rejected argument, or a positive hipError_t for a failed launch.  The text
+ *     of the last failure on the calling thread is in trifast_last_error().
+ *   - Tensors are owned by the caller.  The library never allocates or frees
+ *     device memory and keeps no pointer after a call returns; temporary storage
+ *     is a caller-provided workspace whose size trifast_*_workspace_bytes gives.
+ *   - Launches are asynchronous on `stream` (a hipStream_t passed as void*).
+ *   - Layouts (reference src/trifast/torch.py:220-226):
+ *       q, k, v, do : [b, h, n, n, d]  element strides {sb, sh, si, sj, sd}, sd == 1
+ *       bias        : [b, h, n, n]     element strides {sb, sh, sj, sk}, sk == 1
+ *       mask        : [b, n, n] bytes  strides {sb, si, sk}, any; nonzero = key masked OUT
+ *       o, dq, dk, dv : contiguous [b, h, n, n, d];  db : contiguous [b, h, n, n]
+ *       lse         : contiguous float32 [b, h, n, n], natural log, indexed [i, j]
+ *     Vector loads need 16-byte alignment: base pointers of q, k, v, do, o must be
+ *     16-byte aligned and their si/sj/sh/sb strides multiples of 16/sizeof(elem).
+ *     bias may have any row stride (an unaligned row takes an element-wise path).
+ */
+#ifndef TRIFAST_HIP_H
+#define TRIFAST_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TRIFAST_ABI_VERSION 1
+
+/* dtype codes */
+#define TRIFAST_F32 0
+#define TRIFAST_BF16 1
+#define TRIFAST_F16 2
+
+/* kernel ids: one per launch of the reference operator
+ * (reference src/trifast/triton.py:19 _fwd, :274 _bwd_q, :143 _bwd_kv, :394 _bwd_b) */
+#define TRIFAST_KERNEL_FWD 0
+#define TRIFAST_KERNEL_BWD_Q 1
+#define TRIFAST_KERNEL_BWD_KV 2
+#define TRIFAST_KERNEL_BWD_B 3
+#define TRIFAST_NUM_KERNELS 4
+
+/* error codes */
+#define TRIFAST_OK 0
+#define TRIFAST_EINVAL (-1)      /* bad size / null pointer / bad dtype            */
+#define TRIFAST_EUNSUPPORTED (-2) /* head dim or tile not among the compiled ones */
+#define TRIFAST_EALIGN (-3)      /* pointer or stride breaks the alignment rule    */
+#define TRIFAST_EWORKSPACE (-4)  /* workspace missing or too small                 */
+
+int trifast_abi_version(void);
+
+/* Text of the last error on this thread ("" if none). */
+const char* trifast_last_error(void);
+
+/*
+ * Compiled tile instantiations, for the tuner.  Replaces the triton.Config lists
+ * of reference src/trifast/autotune_helpers.py:58-211.
+ *   trifast_num_tiles(kernel)            number of instantiations of that kernel
+ *   trifast_tile_info(kernel, tile, ...) block sizes of one instantiation
+ *   trifast_supports(...)                1 if the instantiation can run the shape
+ *   trifast_default_tile(...)            heuristic pick when nothing is cached
+ */
+int trifast_num_tiles(int kernel);
+int trifast_tile_info(int kernel, int tile, int* block_j, int* block_k, int* num_waves);
+int trifast_supports(int kernel, int tile, int64_t n, int64_t h, int64_t d, int dtype);
+int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype);
+
+/* Bytes of caller-provided workspace (256-byte aligned) each call needs. */
+int64_t trifast_fwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype);
+int64_t trifast_bwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype);
+
+/*
+ * Forward: o, lse = triangle_attention(q, k, v, bias, mask).
+ * Replaces the _fwd launch of reference src/trifast/torch.py:48-59.
+ * tile < 0 selects trifast_default_tile.
+ */
+int trifast_fwd(void* o, float* lse,
+                const void* q, const void* k, const void* v,
+                const void* bias, const uint8_t* mask,
+                int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
+                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                const int64_t* bias_strides, const int64_t* mask_strides,
+                int tile, void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * Backward: dq, dk, dv, db from do and the saved q, k, v, bias, mask, o, lse.
+ * Replaces the _bwd_q, _bwd_kv and _bwd_b launches of reference
+ * src/trifast/torch.py:111-174 (one call, fixed launch order, deterministic).
+ * do may have any strides with sd == 1 or sd == 0 patterns excluded: the caller
+ * materialises a do whose last stride is not 1.  o and lse are the forward's
+ * contiguous outputs.  tiles[3] = {bwd_q, bwd_kv, bwd_b} tile ids (<0: default).
+ */
+int trifast_bwd(void* dq, void* dk, void* dv, void* db,
+                const void* dout, const void* q, const void* k, const void* v,
+                const void* bias, const uint8_t* mask, const void* o, const float* lse,
+                int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
+                const int64_t* do_strides, const int64_t* q_strides, const int64_t* k_strides,
+                const int64_t* v_strides, const int64_t* bias_strides, const int64_t* mask_strides,
+                const int* tiles, void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * The three backward launches one at a time (same arguments as trifast_bwd; each
+ * writes only its own outputs), so a tuner can time them separately.  Order
+ * matters exactly as in the reference (src/trifast/torch.py:110): BWD_Q first --
+ * it also fills the workspace's delta = rowsum(o * do) that the other two read.
+ */
+int trifast_bwd_one(int kernel,
+                    void* dq, void* dk, void* dv, void* db,
+                    const void* dout, const void* q, const void* k, const void* v,
+                    const void* bias, const uint8_t* mask, const void* o, const float* lse,
+                    int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
+                    const int64_t* do_strides, const int64_t* q_strides, const int64_t* k_strides,
+                    const int64_t* v_strides, const int64_t* bias_strides, const int64_t* mask_strides,
+                    int tile, void* workspace, int64_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRIFAST_HIP_H */

@@ -1,0 +1,10 @@
+"""trifast_amd: fused triangle self-attention for AMD Instinct MI355X (gfx950).
+
+Same Python surface as the reference package (src/trifast/__init__.py:1-3).
+"""
+
+from trifast_amd.torch import triangle_attention
+
+__version__ = "0.1.12"
+
+__all__ = ["triangle_attention"]

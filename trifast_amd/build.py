@@ -1,0 +1,81 @@
+"""Build the gfx950 shared library in-tree with hipcc.
+
+``python -m trifast_amd.build`` compiles every ``csrc/*.hip`` translation unit for
+``--offload-arch=gfx950`` (in parallel) and links ``trifast_amd/libtrifast_hip.so``.
+hipcc cross-compiles without a GPU, so this runs anywhere the ROCm toolchain is.
+"""
+
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+PKG_DIR = Path(__file__).resolve().parent
+CSRC = PKG_DIR / "csrc"
+LIB_NAME = "libtrifast_hip.so"
+LIB_PATH = PKG_DIR / LIB_NAME
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-fno-gpu-rdc",
+    # packed fp32 VALU forms are kept out of the generated code on purpose
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found: the ROCm toolchain is required to build trifast_amd")
+    return exe
+
+
+def sources() -> list[Path]:
+    return sorted(CSRC.glob("*.hip"))
+
+
+def _compile(src: Path, obj: Path, verbose: bool) -> None:
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src.name}:\n{res.stdout}\n{res.stderr}")
+    if verbose:
+        # the host pass does not know the packed-fp32 feature name; that warning is noise
+        noise = "packed-fp32-ops"
+        msg = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+        if msg.strip():
+            print(msg, file=sys.stderr)
+
+
+def build(verbose: bool = False, jobs: int | None = None) -> Path:
+    """Compile every translation unit and link the shared library.  Always rebuilds."""
+    build_dir = PKG_DIR / "build"
+    build_dir.mkdir(exist_ok=True)
+    srcs = sources()
+    if not srcs:
+        raise RuntimeError(f"no .hip sources under {CSRC}")
+    objs = [build_dir / (s.stem + ".o") for s in srcs]
+    jobs = jobs or min(len(srcs), int(os.environ.get("MAX_JOBS", "8")))
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        futs = [pool.submit(_compile, s, o, verbose) for s, o in zip(srcs, objs)]
+        for f in futs:
+            f.result()
+    tmp = PKG_DIR / (LIB_NAME + ".tmp")
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    path = build(verbose=True)
+    print(f"built {path}")

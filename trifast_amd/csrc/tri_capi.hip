@@ -1,0 +1,365 @@
+// C ABI of the triangle-attention library (see include/trifast_hip.h):
+// argument checking, workspace carving, the mask pre-pass and the fixed launch
+// order of the backward kernels.  Nothing here allocates device memory.
+#include <hip/hip_runtime.h>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <limits>
+
+#include "../../include/trifast_hip.h"
+#include "tri_common.hpp"
+#include "tri_launch.hpp"
+
+namespace tri {
+
+// ---------------------------------------------------------------------------
+// Mask pre-pass: bytes -> "keep" bit words + fully-masked-row flags.
+// One wave per (batch, row).  A row whose valid keys are all masked follows the
+// additive-mask semantics of reference src/trifast/equiv.py:49,59-62: all logits
+// saturate to the same value, so the row attends uniformly to every key; its
+// keep words are set to "all valid keys" and rowflag tells the kernels to
+// drop the q.k and bias terms.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void mask_prep_kernel(const MaskPrepArgs a) {
+  const int i = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
+  const uint8_t* row = a.mask + b * a.sb + i * a.si;
+  uint32_t* out = a.keep + ((int64_t)b * a.n + i) * a.nwords;
+  bool any_kept = false;
+  for (int w = lane; w < a.nwords; w += 64) {
+    uint32_t bits = 0;
+    for (int t = 0; t < 32; ++t) {
+      const int key = 32 * w + t;
+      if (key < a.n && row[key * a.sk] == 0) bits |= 1u << t;
+    }
+    out[w] = bits;
+    any_kept |= bits != 0;
+  }
+  const bool row_kept = __any(any_kept);
+  if (!row_kept) {
+    for (int w = lane; w < a.nwords; w += 64) {
+      const int rem = a.n - 32 * w;
+      out[w] = rem >= 32 ? 0xffffffffu : ((1u << rem) - 1u);
+    }
+  }
+  if (lane == 0) a.rowflag[(int64_t)b * a.n + i] = row_kept ? 0 : 1;
+}
+
+hipError_t mask_prep_launch(const MaskPrepArgs& a, int b, hipStream_t st) {
+  hipLaunchKernelGGL(mask_prep_kernel, dim3(a.n, b), dim3(64), 0, st, a);
+  return hipGetLastError();
+}
+
+}  // namespace tri
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(e));
+  return (int)e > 0 ? (int)e : 1;
+}
+
+int64_t align256(int64_t x) { return (x + 255) & ~int64_t(255); }
+int elem_size(int dtype) { return dtype == TRIFAST_F32 ? 4 : 2; }
+
+float dtype_min(int dtype) {
+  switch (dtype) {
+    case TRIFAST_BF16: return -3.3895313892515355e38f;
+    case TRIFAST_F16: return -65504.0f;
+    default: return -std::numeric_limits<float>::max();
+  }
+}
+
+struct Workspace {
+  uint32_t* keep;
+  uint8_t* rowflag;
+  float* delta;
+  int nwords;
+};
+
+int64_t ws_mask_bytes(int64_t b, int64_t n) {
+  const int64_t nwords = (n + 31) / 32;
+  return align256(b * n * nwords * 4) + align256(b * n);
+}
+
+Workspace carve(void* ws, int64_t b, int64_t n) {
+  Workspace w;
+  const int64_t nwords = (n + 31) / 32;
+  char* p = static_cast<char*>(ws);
+  w.keep = reinterpret_cast<uint32_t*>(p);
+  p += align256(b * n * nwords * 4);
+  w.rowflag = reinterpret_cast<uint8_t*>(p);
+  p += align256(b * n);
+  w.delta = reinterpret_cast<float*>(p);
+  w.nwords = (int)nwords;
+  return w;
+}
+
+int check_common(int64_t b, int64_t h, int64_t n, int64_t d, int dtype) {
+  if (b < 1 || h < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive (b=%lld h=%lld n=%lld)", (long long)b, (long long)h, (long long)n);
+  if (dtype != TRIFAST_F32 && dtype != TRIFAST_BF16 && dtype != TRIFAST_F16) return fail(TRIFAST_EINVAL, "unknown dtype code %d", dtype);
+  if (!tri::head_dim_ok((int)d)) return fail(TRIFAST_EUNSUPPORTED, "head dim %lld is not one of the compiled ones (16, 32, 64, 128)", (long long)d);
+  if (n > 65535 || b * h > 65535) return fail(TRIFAST_EINVAL, "n and b*h must be at most 65535");
+  return 0;
+}
+
+// q-like tensor: 16-byte aligned base, strides multiples of the vector width, d stride 1
+int check_qlike(const char* name, const void* p, const int64_t* s, int dtype) {
+  if (!p || !s) return fail(TRIFAST_EINVAL, "%s: null pointer", name);
+  const int vec = 16 / elem_size(dtype);
+  if (s[4] != 1) return fail(TRIFAST_EALIGN, "%s: last stride must be 1 (got %lld)", name, (long long)s[4]);
+  if ((reinterpret_cast<uintptr_t>(p) & 15) != 0) return fail(TRIFAST_EALIGN, "%s: base pointer is not 16-byte aligned", name);
+  for (int t = 0; t < 4; ++t)
+    if (s[t] % vec != 0) return fail(TRIFAST_EALIGN, "%s: stride %d (%lld) is not a multiple of %d elements", name, t, (long long)s[t], vec);
+  return 0;
+}
+
+tri::Str5 str5(const int64_t* s) { return tri::Str5{s[0], s[1], s[2], s[3]}; }
+
+int bias_vec_ok(const void* bias, const int64_t* s) {
+  return ((reinterpret_cast<uintptr_t>(bias) & 15) == 0 && s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0) ? 1 : 0;
+}
+
+int run_mask_prep(const uint8_t* mask, const int64_t* ms, const Workspace& w, int64_t b, int64_t n, hipStream_t st) {
+  tri::MaskPrepArgs m;
+  m.mask = mask;
+  m.sb = ms[0]; m.si = ms[1]; m.sk = ms[2];
+  m.keep = w.keep;
+  m.rowflag = w.rowflag;
+  m.n = (int)n;
+  m.nwords = w.nwords;
+  hipError_t e = tri::mask_prep_launch(m, (int)b, st);
+  if (e != hipSuccess) return hip_fail(e, "mask pre-pass launch");
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int trifast_abi_version(void) { return TRIFAST_ABI_VERSION; }
+
+const char* trifast_last_error(void) { return g_err; }
+
+int trifast_num_tiles(int kernel) {
+  switch (kernel) {
+    case TRIFAST_KERNEL_FWD: return tri::fwd_num_tiles();
+    case TRIFAST_KERNEL_BWD_Q: return tri::bwd_q_num_tiles();
+    case TRIFAST_KERNEL_BWD_KV: return tri::bwd_kv_num_tiles();
+    case TRIFAST_KERNEL_BWD_B: return tri::bwd_b_num_tiles();
+  }
+  return fail(TRIFAST_EINVAL, "unknown kernel id %d", kernel);
+}
+
+int trifast_tile_info(int kernel, int tile, int* block_j, int* block_k, int* num_waves) {
+  const int nt = trifast_num_tiles(kernel);
+  if (nt < 0) return nt;
+  if (tile < 0 || tile >= nt) return fail(TRIFAST_EINVAL, "tile %d out of range for kernel %d", tile, kernel);
+  tri::TileInfo t;
+  switch (kernel) {
+    case TRIFAST_KERNEL_FWD: t = tri::fwd_tile_info(tile); break;
+    case TRIFAST_KERNEL_BWD_Q: t = tri::bwd_q_tile_info(tile); break;
+    case TRIFAST_KERNEL_BWD_KV: t = tri::bwd_kv_tile_info(tile); break;
+    default: t = tri::bwd_b_tile_info(tile); break;
+  }
+  if (block_j) *block_j = t.block_j;
+  if (block_k) *block_k = t.block_k;
+  if (num_waves) *num_waves = t.num_waves;
+  return 0;
+}
+
+int trifast_supports(int kernel, int tile, int64_t n, int64_t h, int64_t d, int dtype) {
+  (void)h;
+  if (dtype != TRIFAST_F32 && dtype != TRIFAST_BF16 && dtype != TRIFAST_F16) return 0;
+  switch (kernel) {
+    case TRIFAST_KERNEL_FWD: return tri::fwd_supports(tile, n, (int)d, dtype) ? 1 : 0;
+    case TRIFAST_KERNEL_BWD_Q: return tri::bwd_q_supports(tile, n, (int)d, dtype) ? 1 : 0;
+    case TRIFAST_KERNEL_BWD_KV: return tri::bwd_kv_supports(tile, n, (int)d, dtype) ? 1 : 0;
+    case TRIFAST_KERNEL_BWD_B: return tri::bwd_b_supports(tile, n, (int)d, dtype) ? 1 : 0;
+  }
+  return 0;
+}
+
+int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype) {
+  (void)h;
+  int pick = 0;
+  switch (kernel) {
+    case TRIFAST_KERNEL_FWD:
+      if (n <= 64) pick = 2;
+      else if (n <= 256 || d >= 128 || dtype == TRIFAST_F32) pick = 0;
+      else pick = 1;
+      break;
+    default: pick = 0; break;
+  }
+  if (!trifast_supports(kernel, pick, n, h, d, dtype)) {
+    const int nt = trifast_num_tiles(kernel);
+    for (int t = 0; t < nt; ++t)
+      if (trifast_supports(kernel, t, n, h, d, dtype)) return t;
+    return fail(TRIFAST_EUNSUPPORTED, "no tile of kernel %d supports n=%lld d=%lld dtype=%d", kernel, (long long)n, (long long)d, dtype);
+  }
+  return pick;
+}
+
+int64_t trifast_fwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype) {
+  (void)h; (void)d; (void)dtype;
+  if (b < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
+  return ws_mask_bytes(b, n);
+}
+
+int64_t trifast_bwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype) {
+  (void)d; (void)dtype;
+  if (b < 1 || h < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
+  return ws_mask_bytes(b, n) + align256(b * h * n * n * 4);
+}
+
+int trifast_fwd(void* o, float* lse, const void* q, const void* k, const void* v, const void* bias,
+                const uint8_t* mask, int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
+                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                const int64_t* bias_strides, const int64_t* mask_strides, int tile, void* workspace,
+                int64_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  int rc = check_common(b, h, n, d, dtype);
+  if (rc) return rc;
+  if (!o || !lse || !bias || !mask || !bias_strides || !mask_strides) return fail(TRIFAST_EINVAL, "null pointer argument");
+  if ((rc = check_qlike("q", q, q_strides, dtype))) return rc;
+  if ((rc = check_qlike("k", k, k_strides, dtype))) return rc;
+  if ((rc = check_qlike("v", v, v_strides, dtype))) return rc;
+  if ((reinterpret_cast<uintptr_t>(o) & 15) != 0) return fail(TRIFAST_EALIGN, "o: base pointer is not 16-byte aligned");
+  if (bias_strides[3] != 1) return fail(TRIFAST_EALIGN, "bias: last stride must be 1 (got %lld)", (long long)bias_strides[3]);
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
+      workspace_bytes < trifast_fwd_workspace_bytes(b, h, n, d, dtype))
+    return fail(TRIFAST_EWORKSPACE, "workspace missing, misaligned or smaller than trifast_fwd_workspace_bytes");
+  if (tile < 0) tile = trifast_default_tile(TRIFAST_KERNEL_FWD, n, h, d, dtype);
+  if (tile < 0) return tile;
+  if (!tri::fwd_supports(tile, n, (int)d, dtype)) return fail(TRIFAST_EUNSUPPORTED, "forward tile %d does not support n=%lld d=%lld dtype=%d", tile, (long long)n, (long long)d, dtype);
+
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const Workspace w = carve(workspace, b, n);
+  if ((rc = run_mask_prep(mask, mask_strides, w, b, n, st))) return rc;
+
+  tri::FwdArgs a;
+  a.q = q; a.k = k; a.v = v; a.bias = bias;
+  a.keep = w.keep; a.rowflag = w.rowflag;
+  a.o = o; a.lse = lse;
+  a.sq = str5(q_strides); a.sk = str5(k_strides); a.sv = str5(v_strides);
+  a.sbias = tri::Str4{bias_strides[0], bias_strides[1], bias_strides[2]};
+  a.H = (int)h; a.N = (int)n; a.nwords = w.nwords;
+  a.bias_vec_ok = bias_vec_ok(bias, bias_strides);
+  a.c = (float)(1.4426950408889634 / std::sqrt((double)d));
+  a.sqrt_d = (float)std::sqrt((double)d);
+  a.neg_inf = dtype_min(dtype);
+  hipError_t e = tri::fwd_launch(a, (int)(b * h), (int)d, dtype, tile, st);
+  if (e != hipSuccess) return hip_fail(e, "forward launch");
+  return 0;
+}
+
+static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const void* dout, const void* q,
+                    const void* k, const void* v, const void* bias, const uint8_t* mask, const void* o,
+                    const float* lse, int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
+                    const int64_t* do_strides, const int64_t* q_strides, const int64_t* k_strides,
+                    const int64_t* v_strides, const int64_t* bias_strides, const int64_t* mask_strides,
+                    const int* tiles, void* workspace, int64_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  int rc = check_common(b, h, n, d, dtype);
+  if (rc) return rc;
+  if (!bias || !mask || !o || !lse || !bias_strides || !mask_strides) return fail(TRIFAST_EINVAL, "null pointer argument");
+  if ((rc = check_qlike("do", dout, do_strides, dtype))) return rc;
+  if ((rc = check_qlike("q", q, q_strides, dtype))) return rc;
+  if ((rc = check_qlike("k", k, k_strides, dtype))) return rc;
+  if ((rc = check_qlike("v", v, v_strides, dtype))) return rc;
+  if (bias_strides[3] != 1) return fail(TRIFAST_EALIGN, "bias: last stride must be 1 (got %lld)", (long long)bias_strides[3]);
+  if ((reinterpret_cast<uintptr_t>(o) & 15) != 0) return fail(TRIFAST_EALIGN, "o: base pointer is not 16-byte aligned");
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
+      workspace_bytes < trifast_bwd_workspace_bytes(b, h, n, d, dtype))
+    return fail(TRIFAST_EWORKSPACE, "workspace missing, misaligned or smaller than trifast_bwd_workspace_bytes");
+  const bool all = which < 0;
+  const bool do_q = all || which == TRIFAST_KERNEL_BWD_Q;
+  const bool do_kv = all || which == TRIFAST_KERNEL_BWD_KV;
+  const bool do_b = all || which == TRIFAST_KERNEL_BWD_B;
+  if (!do_q && !do_kv && !do_b) return fail(TRIFAST_EINVAL, "kernel id %d is not a backward kernel", which);
+  if (do_q && (!dq || (reinterpret_cast<uintptr_t>(dq) & 15))) return fail(TRIFAST_EINVAL, "dq: null or misaligned");
+  if (do_kv && (!dk || !dv || (reinterpret_cast<uintptr_t>(dk) & 15) || (reinterpret_cast<uintptr_t>(dv) & 15))) return fail(TRIFAST_EINVAL, "dk/dv: null or misaligned");
+  if (do_b && !db) return fail(TRIFAST_EINVAL, "db: null");
+
+  int tq = tiles ? tiles[0] : -1, tkv = tiles ? tiles[1] : -1, tb = tiles ? tiles[2] : -1;
+  if (tq < 0) tq = trifast_default_tile(TRIFAST_KERNEL_BWD_Q, n, h, d, dtype);
+  if (tkv < 0) tkv = trifast_default_tile(TRIFAST_KERNEL_BWD_KV, n, h, d, dtype);
+  if (tb < 0) tb = trifast_default_tile(TRIFAST_KERNEL_BWD_B, n, h, d, dtype);
+  if (tq < 0 || tkv < 0 || tb < 0) return TRIFAST_EUNSUPPORTED;
+  if (do_q && !tri::bwd_q_supports(tq, n, (int)d, dtype)) return fail(TRIFAST_EUNSUPPORTED, "bwd_q tile %d unsupported for this shape", tq);
+  if (do_kv && !tri::bwd_kv_supports(tkv, n, (int)d, dtype)) return fail(TRIFAST_EUNSUPPORTED, "bwd_kv tile %d unsupported for this shape", tkv);
+  if (do_b && !tri::bwd_b_supports(tb, n, (int)d, dtype)) return fail(TRIFAST_EUNSUPPORTED, "bwd_b tile %d unsupported for this shape", tb);
+
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const Workspace w = carve(workspace, b, n);
+  // The pre-pass is cheap (n^2 bytes) and makes every single-kernel call
+  // self-contained, so it runs whenever the first kernel of a call needs it.
+  if ((rc = run_mask_prep(mask, mask_strides, w, b, n, st))) return rc;
+
+  tri::BwdArgs a;
+  a.q = q; a.k = k; a.v = v; a.bias = bias; a.o = o; a.dout = dout;
+  a.lse = lse;
+  a.keep = w.keep; a.rowflag = w.rowflag; a.delta = w.delta;
+  a.dq = dq; a.dk = dk; a.dv = dv; a.db = db;
+  a.sq = str5(q_strides); a.sk = str5(k_strides); a.sv = str5(v_strides); a.sdo = str5(do_strides);
+  a.sbias = tri::Str4{bias_strides[0], bias_strides[1], bias_strides[2]};
+  a.H = (int)h; a.N = (int)n; a.nwords = w.nwords;
+  a.bias_vec_ok = bias_vec_ok(bias, bias_strides);
+  a.c = (float)(1.4426950408889634 / std::sqrt((double)d));
+  a.sqrt_d = (float)std::sqrt((double)d);
+  a.scale = (float)(1.0 / std::sqrt((double)d));
+  const int bh = (int)(b * h);
+  hipError_t e;
+  if (do_q) {
+    e = tri::bwd_q_launch(a, bh, (int)d, dtype, tq, st);
+    if (e != hipSuccess) return hip_fail(e, "bwd_q launch");
+  }
+  if (do_kv) {
+    e = tri::bwd_kv_launch(a, bh, (int)d, dtype, tkv, st);
+    if (e != hipSuccess) return hip_fail(e, "bwd_kv launch");
+  }
+  if (do_b) {
+    e = tri::bwd_b_launch(a, bh, (int)d, dtype, tb, st);
+    if (e != hipSuccess) return hip_fail(e, "bwd_b launch");
+  }
+  return 0;
+}
+
+int trifast_bwd(void* dq, void* dk, void* dv, void* db, const void* dout, const void* q, const void* k,
+                const void* v, const void* bias, const uint8_t* mask, const void* o, const float* lse,
+                int64_t b, int64_t h, int64_t n, int64_t d, int dtype, const int64_t* do_strides,
+                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                const int64_t* bias_strides, const int64_t* mask_strides, const int* tiles,
+                void* workspace, int64_t workspace_bytes, void* stream) {
+  return bwd_impl(-1, dq, dk, dv, db, dout, q, k, v, bias, mask, o, lse, b, h, n, d, dtype, do_strides,
+                  q_strides, k_strides, v_strides, bias_strides, mask_strides, tiles, workspace,
+                  workspace_bytes, stream);
+}
+
+int trifast_bwd_one(int kernel, void* dq, void* dk, void* dv, void* db, const void* dout, const void* q,
+                    const void* k, const void* v, const void* bias, const uint8_t* mask, const void* o,
+                    const float* lse, int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
+                    const int64_t* do_strides, const int64_t* q_strides, const int64_t* k_strides,
+                    const int64_t* v_strides, const int64_t* bias_strides, const int64_t* mask_strides,
+                    int tile, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (kernel != TRIFAST_KERNEL_BWD_Q && kernel != TRIFAST_KERNEL_BWD_KV && kernel != TRIFAST_KERNEL_BWD_B)
+    return fail(TRIFAST_EINVAL, "kernel id %d is not a backward kernel", kernel);
+  int tiles[3] = {-1, -1, -1};
+  tiles[kernel - TRIFAST_KERNEL_BWD_Q] = tile;
+  return bwd_impl(kernel, dq, dk, dv, db, dout, q, k, v, bias, mask, o, lse, b, h, n, d, dtype, do_strides,
+                  q_strides, k_strides, v_strides, bias_strides, mask_strides, tiles, workspace,
+                  workspace_bytes, stream);
+}
+
+}  // extern "C"

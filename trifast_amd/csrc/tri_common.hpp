@@ -1,0 +1,121 @@
+// Shared device-side pieces of the gfx950 triangle-attention kernels.
+//
+// MFMA register layouts used everywhere (wave64, 32x32 tiles):
+//   A operand (M=32 rows x contraction): lane l supplies row l%32 and the KP
+//     contraction slots owned by lane group g = l/32.
+//   B operand (contraction x N=32 cols): lane l supplies column l%32, same slots.
+//   C/D (32x32 fp32, 16 values per lane): value v of lane l is
+//     row 8*(v/4) + 4*g + v%4, column l%32.
+// A C tile can feed the next MFMA as a B (or A) operand without leaving
+// registers when the contraction runs over its in-lane (row) index: slot
+// (g, v) of the C tile pairs with slot (g, v) of the other operand.  To make the
+// other operand a single 16-byte read, tile rows are assigned to real indices
+// through a permutation: value v of group g stands for real index
+//   idx(v, g) = 16*(v/8) + 8*g + v%8      (8 consecutive indices per 8 values)
+// which means tile row m holds real index perm32(m) = m with bits 2 and 3
+// swapped.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+#define TRI_DEV __device__ __forceinline__
+
+namespace tri {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+// Finite stand-in for "minus infinity" on raw scores: large enough that
+// exp2((NEG - max) * c) is exactly 0, finite so that NEG - NEG is never NaN.
+constexpr float kNeg = -1.0e30f;
+
+TRI_DEV int perm32(int m) {  // swap bits 2 and 3
+  return (m & 0x13) | ((m & 4) << 1) | ((m & 8) >> 1);
+}
+// real index (within a 32-tile) of C value v for lane group g
+TRI_DEV constexpr int cidx(int v, int g) { return 16 * (v / 8) + 8 * g + (v % 8); }
+// output row (within a 32-tile) of C value v for lane group g, no permutation
+TRI_DEV constexpr int crow(int v, int g) { return 8 * (v / 4) + 4 * g + (v % 4); }
+
+template <typename T>
+struct Elem;
+
+template <>
+struct Elem<__bf16> {
+  static constexpr int KP = 8;    // contraction slots per lane per MFMA
+  static constexpr int VEC = 8;   // elements per 16-byte vector
+  typedef bf16x8 frag;
+  typedef bf16x8 vec;
+  typedef bf16x4 vec4;
+  static TRI_DEV f32x16 mfma(frag a, frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static TRI_DEV frag zero() { return (frag){0, 0, 0, 0, 0, 0, 0, 0}; }
+  static TRI_DEV frag pack(const float* x) {
+    frag r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (__bf16)x[e];
+    return r;
+  }
+};
+
+template <>
+struct Elem<_Float16> {
+  static constexpr int KP = 8;
+  static constexpr int VEC = 8;
+  typedef f16x8 frag;
+  typedef f16x8 vec;
+  typedef f16x4 vec4;
+  static TRI_DEV f32x16 mfma(frag a, frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static TRI_DEV frag zero() { return (frag){0, 0, 0, 0, 0, 0, 0, 0}; }
+  static TRI_DEV frag pack(const float* x) {
+    frag r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (_Float16)x[e];
+    return r;
+  }
+};
+
+template <>
+struct Elem<float> {
+  static constexpr int KP = 1;
+  static constexpr int VEC = 4;
+  typedef float frag;
+  typedef f32x4 vec;
+  typedef f32x4 vec4;
+  static TRI_DEV f32x16 mfma(frag a, frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+  }
+  static TRI_DEV frag zero() { return 0.f; }
+  static TRI_DEV frag pack(const float* x) { return x[0]; }
+};
+
+template <typename T>
+TRI_DEV float to_f32(T x) { return (float)x; }
+
+TRI_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+TRI_DEV float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// exchange with the lane that holds the other half of the same column
+TRI_DEV float xhalf(float x) { return __shfl_xor(x, 32, 64); }
+
+TRI_DEV f32x16 zero16() {
+  f32x16 z;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) z[v] = 0.f;
+  return z;
+}
+
+}  // namespace tri

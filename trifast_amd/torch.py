@@ -1,0 +1,231 @@
+"""PyTorch operator boundary of the MI355X triangle attention.
+
+Mirrors the public surface of reference src/trifast/torch.py: two ``torch.library``
+operators, ``trifast::triangle_attention`` (-> o, lse; reference :17-65) and
+``trifast::triangle_attention_backward`` (-> dq, dk, dv, db, dmask; reference
+:68-182), glued by ``register_autograd`` (reference :185-217), and the
+``triangle_attention`` wrapper that drops lse (reference :220-228).  The device
+work is done by hand-written HIP kernels behind the C ABI of
+``libtrifast_hip.so``; PyTorch only owns the memory and the stream.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from trifast_amd import _lib, tuner
+
+_DTYPE_CODE = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise TypeError(f"triangle_attention supports float32, bfloat16 and float16, got {t.dtype}") from None
+
+
+def _check_inputs(q, k, v, b, mask) -> tuple[int, int, int, int]:
+    if q.dim() != 5:
+        raise ValueError(f"q must be [b, h, n, n, d], got shape {tuple(q.shape)}")
+    bs, h, n, n2, d = q.shape
+    if n != n2:
+        raise ValueError(f"q must be square in its pair dims, got shape {tuple(q.shape)}")
+    if k.shape != q.shape or v.shape != q.shape:
+        raise ValueError("q, k, v must have the same shape")
+    if tuple(b.shape) != (bs, h, n, n):
+        raise ValueError(f"bias must be [b, h, n, n] = {(bs, h, n, n)}, got {tuple(b.shape)}")
+    if tuple(mask.shape) != (bs, n, n):
+        raise ValueError(f"mask must be [b, n, n] = {(bs, n, n)}, got {tuple(mask.shape)}")
+    if mask.dtype != torch.bool:
+        raise TypeError(f"mask must be bool, got {mask.dtype}")
+    if not (k.dtype == q.dtype and v.dtype == q.dtype and b.dtype == q.dtype):
+        raise TypeError("q, k, v and bias must share one dtype")
+    for name, t in (("q", q), ("k", k), ("v", v), ("bias", b), ("mask", mask)):
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} is on {t.device}: triangle_attention runs on the GPU only")
+        if t.device != q.device:
+            raise RuntimeError("all inputs must be on the same device")
+    return bs, h, n, d
+
+
+def _strides(t: torch.Tensor) -> list[int]:
+    # the stride of a size-1 dim is never used for addressing; report 0
+    return [0 if sz == 1 else st for sz, st in zip(t.shape, t.stride())]
+
+
+def _vector_ready(t: torch.Tensor) -> torch.Tensor:
+    """q-like tensors are read with 16-byte vector loads along d: the last stride
+    must be 1, the base 16-byte aligned and the other strides multiples of the
+    vector width.  Transposed (i<->j) views qualify and are read in place; anything
+    else is copied, as the reference forward copies every non-contiguous input
+    (src/trifast/torch.py:30-34)."""
+    vec = 16 // t.element_size()
+    st = _strides(t)
+    if st[-1] == 1 and t.data_ptr() % 16 == 0 and all(s % vec == 0 for s in st[:-1]):
+        return t
+    return t.contiguous()
+
+
+def _bias_ready(b: torch.Tensor) -> torch.Tensor:
+    return b if (b.stride(-1) == 1 or b.shape[-1] == 1) else b.contiguous()
+
+
+def _workspace(nbytes: int, device) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def _ptr(t):
+    return t.data_ptr()
+
+
+@torch.library.custom_op("trifast::triangle_attention", mutates_args=())
+def _triangle_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    b: torch.Tensor,
+    mask: torch.Tensor,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    lib = _lib.load()
+    bs, h, n, d = _check_inputs(q, k, v, b, mask)
+    code = _dtype_code(q)
+    q, k, v, b = _vector_ready(q), _vector_ready(k), _vector_ready(v), _bias_ready(b)
+    mask_u8 = mask.view(torch.uint8)
+
+    o = torch.empty((bs, h, n, n, d), dtype=q.dtype, device=q.device)
+    lse = torch.empty((bs, h, n, n), dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        ws_bytes = lib.trifast_fwd_workspace_bytes(bs, h, n, d, code)
+        ws = _workspace(ws_bytes, q.device)
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+
+        def launch(tile: int) -> None:
+            rc = lib.trifast_fwd(
+                _ptr(o), _ptr(lse), _ptr(q), _ptr(k), _ptr(v), _ptr(b), _ptr(mask_u8),
+                bs, h, n, d, code,
+                _lib.i64_array(_strides(q)), _lib.i64_array(_strides(k)), _lib.i64_array(_strides(v)),
+                _lib.i64_array(_strides(b)), _lib.i64_array(_strides(mask_u8)),
+                tile, _ptr(ws), ws.numel(), stream,
+            )
+            _lib.check(rc, "trifast_fwd")
+
+        tile = tuner.pick(_lib.KERNEL_FWD, n, h, d, q.dtype, launch)
+        launch(tile)
+    return o, lse
+
+
+@_triangle_attention.register_fake
+def _(q, k, v, b, mask):
+    bs, h, n, _, d = q.shape
+    o = q.new_empty((bs, h, n, n, d))
+    lse = q.new_empty((bs, h, n, n), dtype=torch.float32)
+    return o, lse
+
+
+@torch.library.custom_op("trifast::triangle_attention_backward", mutates_args=())
+def triangle_attention_bwd(
+    do: torch.Tensor,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    b: torch.Tensor,
+    o: torch.Tensor,
+    l: torch.Tensor,
+    mask: torch.Tensor,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    lib = _lib.load()
+    bs, h, n, d = _check_inputs(q, k, v, b, mask)
+    code = _dtype_code(q)
+    if do.dtype != q.dtype:
+        do = do.to(q.dtype)
+    # the upstream gradient is often an expanded (stride-0) tensor, e.g. from
+    # o.sum().backward(): _vector_ready materialises exactly those
+    do = _vector_ready(do)
+    q, k, v, b = _vector_ready(q), _vector_ready(k), _vector_ready(v), _bias_ready(b)
+    o = o.contiguous()
+    l = l.contiguous()
+    mask_u8 = mask.view(torch.uint8)
+
+    dq = torch.empty((bs, h, n, n, d), dtype=q.dtype, device=q.device)
+    dk = torch.empty_like(dq)
+    dv = torch.empty_like(dq)
+    db = torch.empty((bs, h, n, n), dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        ws_bytes = lib.trifast_bwd_workspace_bytes(bs, h, n, d, code)
+        ws = _workspace(ws_bytes, q.device)
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        strides = [
+            _lib.i64_array(_strides(t)) for t in (do, q, k, v, b, mask_u8)
+        ]
+
+        def launch_one(kernel: int, tile: int) -> None:
+            rc = lib.trifast_bwd_one(
+                kernel, _ptr(dq), _ptr(dk), _ptr(dv), _ptr(db),
+                _ptr(do), _ptr(q), _ptr(k), _ptr(v), _ptr(b), _ptr(mask_u8), _ptr(o), _ptr(l),
+                bs, h, n, d, code, *strides, tile, _ptr(ws), ws.numel(), stream,
+            )
+            _lib.check(rc, "trifast_bwd_one")
+
+        # fixed launch order; _bwd_q also produces delta for the other two
+        # (reference src/trifast/torch.py:110)
+        tiles = []
+        for kernel in (_lib.KERNEL_BWD_Q, _lib.KERNEL_BWD_KV, _lib.KERNEL_BWD_B):
+            tiles.append(tuner.pick(kernel, n, h, d, q.dtype, lambda t, kern=kernel: launch_one(kern, t)))
+        rc = lib.trifast_bwd(
+            _ptr(dq), _ptr(dk), _ptr(dv), _ptr(db),
+            _ptr(do), _ptr(q), _ptr(k), _ptr(v), _ptr(b), _ptr(mask_u8), _ptr(o), _ptr(l),
+            bs, h, n, d, code, *strides,
+            (_lib.c_int * 3)(*tiles), _ptr(ws), ws.numel(), stream,
+        )
+        _lib.check(rc, "trifast_bwd")
+    # the mask takes no gradient; autograd still wants a tensor in this slot
+    # (reference src/trifast/torch.py:102)
+    dmask = torch.zeros_like(mask)
+    return dq, dk, dv, db, dmask
+
+
+@triangle_attention_bwd.register_fake
+def _(do, q, k, v, b, o, l, mask):
+    return (
+        q.new_empty(q.shape),
+        q.new_empty(q.shape),
+        q.new_empty(q.shape),
+        b.new_empty(b.shape),
+        torch.zeros_like(mask),
+    )
+
+
+def backwards(ctx, *grad):
+    # reference src/trifast/torch.py:185-207
+    do = grad[0]
+    q, k, v, b, mask, o, l = ctx.saved_tensors
+    dq, dk, dv, db, _ = triangle_attention_bwd(do, q, k, v, b, o, l, mask)
+    return dq, dk, dv, db, None
+
+
+def setup_context(ctx, inputs, output) -> None:
+    # reference src/trifast/torch.py:210-214
+    q, k, v, b, mask, *_ = inputs
+    o, l = output
+    ctx.save_for_backward(q, k, v, b, mask, o, l)
+
+
+_triangle_attention.register_autograd(backwards, setup_context=setup_context)
+
+
+def triangle_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    b: torch.Tensor,
+    mask: torch.Tensor,
+) -> torch.Tensor:
+    """Fused triangle self-attention (starting node).
+
+    q, k, v: [b, h, n, n, d]; b (bias): [b, h, n, n]; mask: [b, n, n] bool with
+    True = key masked out.  Returns o: [b, h, n, n, d].  Reference
+    src/trifast/torch.py:220-228.
+    """
+    o, _ = _triangle_attention(q, k, v, b, mask)
+    return o
