@@ -1,0 +1,49 @@
+// Runtime (dtype, head dim, tile id) -> compile-time instantiation dispatch,
+// shared by the four kernel families.  A family F provides
+//   static constexpr int kNumTiles;                 (at most 4)
+//   static constexpr int P(int tile, int which);    three ints per tile
+//   template <typename T, int D, int A, int B, int C>
+//   static hipError_t run(const Args&, int bh, hipStream_t, bool dry);
+// run() returns hipErrorInvalidConfiguration when the instantiation does not fit
+// the hardware (LDS), and launches nothing when dry is set.
+#pragma once
+#include <hip/hip_runtime.h>
+#include "tri_launch.hpp"
+
+namespace tri {
+
+template <class F, typename T, int D, class Args>
+hipError_t dispatch_tile(const Args& a, int bh, int tile, hipStream_t st, bool dry) {
+  switch (tile) {
+    case 0: return F::template run<T, D, F::P(0, 0), F::P(0, 1), F::P(0, 2)>(a, bh, st, dry);
+    case 1: if constexpr (F::kNumTiles > 1) return F::template run<T, D, F::P(1, 0), F::P(1, 1), F::P(1, 2)>(a, bh, st, dry); break;
+    case 2: if constexpr (F::kNumTiles > 2) return F::template run<T, D, F::P(2, 0), F::P(2, 1), F::P(2, 2)>(a, bh, st, dry); break;
+    case 3: if constexpr (F::kNumTiles > 3) return F::template run<T, D, F::P(3, 0), F::P(3, 1), F::P(3, 2)>(a, bh, st, dry); break;
+  }
+  return hipErrorInvalidValue;
+}
+
+template <class F, typename T, class Args>
+hipError_t dispatch_d(const Args& a, int bh, int d, int tile, hipStream_t st, bool dry) {
+  switch (d) {
+    case 16: return dispatch_tile<F, T, 16>(a, bh, tile, st, dry);
+    case 32: return dispatch_tile<F, T, 32>(a, bh, tile, st, dry);
+    case 64: return dispatch_tile<F, T, 64>(a, bh, tile, st, dry);
+    case 128: return dispatch_tile<F, T, 128>(a, bh, tile, st, dry);
+  }
+  return hipErrorInvalidValue;
+}
+
+template <class F, class Args>
+hipError_t dispatch(const Args& a, int bh, int d, int dtype, int tile, hipStream_t st, bool dry) {
+  switch (dtype) {
+    case kF32: return dispatch_d<F, float>(a, bh, d, tile, st, dry);
+    case kBF16: return dispatch_d<F, __bf16>(a, bh, d, tile, st, dry);
+    case kF16: return dispatch_d<F, _Float16>(a, bh, d, tile, st, dry);
+  }
+  return hipErrorInvalidValue;
+}
+
+constexpr int kMaxStaticLds = 64 * 1024;
+
+}  // namespace tri
