@@ -1,0 +1,297 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused triangle attention on one MI355X.
+
+A "step" is one forward + one backward pass of ``trifast.triangle_attention`` over
+one batch of synthetic pair tensors that are already resident in HBM.  The default
+workload is the one the headline metric is quoted on: bf16, b=1, h=4, d=32,
+n=1024, all keys attended.  Prints ONE JSON line:
+
+  value        fwd+bwd TFLOP/s, counting 14*b*h*n^3*d FLOP per step
+               (forward 4*b*h*n^3*d: two GEMMs; backward 10*b*h*n^3*d: five GEMMs)
+  roofline     the slowest kernel of the step against the dense bf16 MFMA peak,
+               its launch duration measured here with events on the launch stream
+  cpu_baseline the PyTorch restatement of the reference's pure-PyTorch triangle
+               attention, forward + autograd backward, on the host cores, on a
+               bounded sample of rows of the same workload
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload M|C2|C3|C4a|C4b|C5]
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA
+PEAK_F32_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+# name -> (dtype, b, n, h, d, description)
+WORKLOADS = {
+    "C1": (torch.float32, 1, 32, 4, 32, "fp32 b1 n32 h4 d32, 10% random mask"),
+    "C2": (torch.bfloat16, 1, 256, 4, 32, "bf16 b1 n256 h4 d32, no mask"),
+    "C3": (torch.bfloat16, 1, 512, 4, 32, "bf16 b1 n512 h4 d32, padding mask"),
+    "C4a": (torch.float16, 1, 768, 8, 64, "fp16 b1 n768 h8 d64, transposed views"),
+    "C4b": (torch.float16, 2, 384, 8, 64, "fp16 b2 n384 h8 d64, transposed views"),
+    "C5": (torch.bfloat16, 1, 2048, 4, 32, "bf16 b1 n2048 h4 d32, bias outliers, 5% random mask"),
+    "M": (torch.bfloat16, 1, 1024, 4, 32, "bf16 b1 n1024 h4 d32, no mask"),
+}
+
+
+def make_workload(name: str, device, seed: int = 1337):
+    """Seeded synthetic inputs q, k, v, bias, mask, do of one benchmark config.
+
+    Drawn in fp32 in the order q, k, v, bias, mask, do and then cast.  Small
+    configs draw from a CPU generator; above 2**27 elements per tensor the draw
+    moves to the device's generator (same seed) to keep set-up time bounded.
+    """
+    dtype, b, n, h, d, _ = WORKLOADS[name]
+    numel = b * h * n * n * d
+    gdev = torch.device(device) if numel > 2**27 else torch.device("cpu")
+    g = torch.Generator(device=gdev).manual_seed(seed)
+
+    def randn(*shape):
+        return torch.randn(*shape, generator=g, device=gdev)
+
+    def rand(*shape):
+        return torch.rand(*shape, generator=g, device=gdev)
+
+    std = d**-0.5
+    if name in ("C4a", "C4b"):
+        q, k, v = randn(b, h, n, n, d), randn(b, h, n, n, d), randn(b, h, n, n, d)
+    else:
+        q, k, v = randn(b, h, n, n, d) * std, randn(b, h, n, n, d) * std, randn(b, h, n, n, d) * std
+    bias = randn(b, h, n, n)
+    if name == "C1":
+        bias = bias * std
+        mask = rand(b, n, n) < 0.1
+        full = mask.all(dim=-1)  # leave at least one attended key per row
+        mask[..., 0] &= ~full
+    elif name == "C3":
+        # per batch element a valid length L in [n/2, n]; everything >= L is padding
+        L = torch.randint(n // 2, n + 1, (b,), generator=g, device=gdev)
+        idx = torch.arange(n, device=gdev)
+        pad = idx[None, :] >= L[:, None]
+        mask = pad[:, :, None] | pad[:, None, :]
+    elif name in ("C4a", "C4b"):
+        mask = rand(b, n, n) < 0.5
+    elif name == "C5":
+        u = rand(b, h, n, n)
+        bias = torch.where(u < 0.025, torch.full_like(bias, 8.0), bias)
+        bias = torch.where(u > 0.975, torch.full_like(bias, -8.0), bias)
+        mask = rand(b, n, n) < 0.05
+    else:
+        mask = torch.zeros(b, n, n, dtype=torch.bool, device=gdev)
+    do = randn(b, h, n, n, d)
+    q, k, v, bias, do = (t.to(device=device, dtype=dtype) for t in (q, k, v, bias, do))
+    mask = mask.to(device)
+    if name in ("C4a", "C4b"):
+        # ending-node variant: every input is an i<->j transposed, non-contiguous view
+        q, k, v, do = (t.transpose(2, 3) for t in (q, k, v, do))
+        bias = bias.transpose(-1, -2)
+        mask = mask.transpose(-1, -2)
+    return q, k, v, bias, mask, do
+
+
+def flops(b, h, n, d):
+    unit = b * h * n**3 * d
+    return 4 * unit, 10 * unit  # forward, backward
+
+
+def _event_ms(fn, reps):
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        fn()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) / reps
+
+
+def kernel_breakdown(q, k, v, bias, mask, do, reps):
+    """Average launch duration (ms) of the four kernels, each timed with events on the
+    stream it is launched on (torch's current stream), through the C ABI."""
+    from trifast_amd import _lib, tuner
+    from trifast_amd import torch as tt
+
+    lib = _lib.load()
+    b, h, n, _, d = q.shape
+    code = tt._DTYPE_CODE[q.dtype]
+    qv, kv, vv, dov = (tt._vector_ready(t) for t in (q, k, v, do))
+    bv = tt._bias_ready(bias)
+    mu8 = mask.view(torch.uint8)
+    o, lse = tt._triangle_attention(q, k, v, bias, mask)
+    dq, dk, dv = (torch.empty_like(o) for _ in range(3))
+    db = torch.empty(bias.shape, dtype=bias.dtype, device=bias.device)
+    ws = torch.empty(lib.trifast_bwd_workspace_bytes(b, h, n, d, code), dtype=torch.uint8, device=q.device)
+    stream = torch.cuda.current_stream().cuda_stream
+    S = lambda t: _lib.i64_array(tt._strides(t))
+    out = {}
+
+    def fwd(tile):
+        rc = lib.trifast_fwd(o.data_ptr(), lse.data_ptr(), qv.data_ptr(), kv.data_ptr(), vv.data_ptr(), bv.data_ptr(), mu8.data_ptr(),
+                             b, h, n, d, code, S(qv), S(kv), S(vv), S(bv), S(mu8), tile, ws.data_ptr(), ws.numel(), stream)
+        _lib.check(rc, "trifast_fwd")
+
+    def bwd_one(kernel, tile):
+        rc = lib.trifast_bwd_one(kernel, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), db.data_ptr(), dov.data_ptr(), qv.data_ptr(), kv.data_ptr(),
+                                 vv.data_ptr(), bv.data_ptr(), mu8.data_ptr(), o.data_ptr(), lse.data_ptr(), b, h, n, d, code,
+                                 S(dov), S(qv), S(kv), S(vv), S(bv), S(mu8), tile, ws.data_ptr(), ws.numel(), stream)
+        _lib.check(rc, "trifast_bwd_one")
+
+    for kernel in (_lib.KERNEL_FWD, _lib.KERNEL_BWD_Q, _lib.KERNEL_BWD_KV, _lib.KERNEL_BWD_B):
+        launch = fwd if kernel == _lib.KERNEL_FWD else (lambda t, kern=kernel: bwd_one(kern, t))
+        tile = tuner.pick(kernel, n, h, d, q.dtype, launch)
+        launch(tile)
+        torch.cuda.synchronize()
+        out[_lib.KERNEL_NAMES[kernel]] = {"ms": _event_ms(lambda: launch(tile), reps), "tile": _lib.tile_info(kernel, tile)}
+    return out
+
+
+def cpu_baseline(name: str, budget_s: float = 20.0):
+    """Forward + autograd backward of the oracle restatement on the host cores, on the
+    first rows of the same workload (rows are independent; the b*h*n^3 logits of the
+    full job would not fit).  Returns the JSON object for the bench line."""
+    from oracle import triangle_oracle as orc
+
+    dtype, b, n, h, d, _ = WORKLOADS[name]
+    # the host share of a one-GPU box is 16 cores, whatever the machine reports
+    cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(1337)
+    rows = min(n, 8)
+    # time a few rows, then size the sample for the budget
+    def run(rows):
+        q, k, v, do = (torch.randn(b, h, rows, n, d, generator=g) * d**-0.5 for _ in range(4))
+        bias = torch.randn(b, h, n, n, generator=g)
+        mask = torch.zeros(b, rows, n, dtype=torch.bool)
+        t0 = time.perf_counter()
+        for i0 in range(0, rows, 8):
+            sl = slice(i0, min(rows, i0 + 8))
+            qc, kc, vc = (t[:, :, sl].clone().requires_grad_(True) for t in (q, k, v))
+            bc = bias.clone().requires_grad_(True)
+            orc.attention_reference(qc, kc, vc, bc, mask[:, sl]).backward(do[:, :, sl])
+        return time.perf_counter() - t0
+
+    run(rows)  # warm-up
+    t_probe = run(rows)
+    sample = int(max(rows, min(n, rows * budget_s / max(t_probe, 1e-6)) // 8 * 8))
+    t = run(sample)
+    fl = sum(flops(b, h, n, d)) * sample / n
+    return {
+        "value": fl / t / 1e12,
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{sample} of {n} pair rows of the same workload, fp32, fwd + autograd bwd in {t:.1f} s "
+                  f"(full job extrapolates to {t * n / sample:.0f} s)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="M", choices=[w for w in WORKLOADS if w != "C1"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-budget", type=float, default=20.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU: the operator has no CPU path", file=sys.stderr)
+        sys.exit(2)
+
+    import trifast_amd
+    from trifast_amd import tuner
+
+    dev = torch.device("cuda:0")
+    dtype, b, n, h, d, desc = WORKLOADS[args.workload]
+    q, k, v, bias, mask, do = make_workload(args.workload, dev)
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True), bias.requires_grad_(True)
+
+    def step():
+        o = trifast_amd.triangle_attention(q, k, v, bias, mask)
+        o.backward(do)
+        q.grad = k.grad = v.grad = bias.grad = None
+
+    def fwd_only():
+        with torch.no_grad():
+            trifast_amd.triangle_attention(q, k, v, bias, mask)
+
+    for _ in range(args.warmup):  # also warms the tile cache
+        step()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base_mem = torch.cuda.memory_allocated()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    peak_extra = torch.cuda.max_memory_allocated() - base_mem
+
+    fwd_only()
+    torch.cuda.synchronize()
+    ms_fwd = _event_ms(fwd_only, args.steps)
+
+    f_fwd, f_bwd = flops(b, h, n, d)
+    peak = PEAK_F32_TFLOPS if dtype == torch.float32 else PEAK_BF16_TFLOPS
+    tf_step = (f_fwd + f_bwd) / ms_step / 1e9
+    tf_fwd = f_fwd / ms_fwd / 1e9
+
+    kern = kernel_breakdown(q.detach(), k.detach(), v.detach(), bias.detach(), mask, do, max(3, args.steps // 2))
+    # GEMMs each kernel needs for its own outputs (S and dP are recomputed per kernel)
+    gemms = {"_fwd": 2, "_bwd_q": 3, "_bwd_kv": 4, "_bwd_b": 2}
+    for name, rec in kern.items():
+        rec["tflops"] = gemms[name] * 2 * b * h * n**3 * d / rec["ms"] / 1e9
+    dom = max(kern, key=lambda key: kern[key]["ms"])
+    roofline = {
+        "kernel": dom,
+        "bound": "mfma",
+        "achieved": kern[dom]["tflops"],
+        "peak": peak,
+        "unit": "TFLOP/s",
+        "frac": kern[dom]["tflops"] / peak,
+        "traffic": None,
+        "launch_ms": kern[dom]["ms"],
+        "flop_per_launch": gemms[dom] * 2 * b * h * n**3 * d,
+    }
+
+    line = {
+        "metric": "fwd+bwd TFLOP/s & % bf16 MFMA peak, bf16 h=4 d=32 n=1024, 1xMI355X",
+        "value": tf_step,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype],
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {desc}", "b": b, "h": h, "n": n, "d": d},
+        "frac_of_peak": tf_step / peak,
+        "fwd_ms": ms_fwd,
+        "fwd_tflops": tf_fwd,
+        "fwd_frac_of_peak": tf_fwd / peak,
+        "peak_extra_mem_mib": peak_extra / 2**20,
+        "kernels": {name: {"ms": round(rec["ms"], 4), "tflops": round(rec["tflops"], 1), "tile": rec["tile"]} for name, rec in kern.items()},
+        "roofline": roofline,
+        "autotune": tuner.autotune_enabled(),
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(args.workload, args.cpu_budget)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

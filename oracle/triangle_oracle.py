@@ -116,7 +116,7 @@ def forward_backward_chunked(q, k, v, bias, mask, do, chunk: int = 32, want_grad
     dq = torch.empty_like(q) if want_grads else None
     dk = torch.empty_like(k) if want_grads else None
     dv = torch.empty_like(v) if want_grads else None
-    db = torch.zeros(bias.shape, dtype=torch.float32) if want_grads else None
+    db = torch.zeros(bias.shape, dtype=torch.float32, device=bias.device) if want_grads else None
     for i0 in range(0, n, chunk):
         sl = slice(i0, min(n, i0 + chunk))
         qc, kc, vc = (t[:, :, sl].detach().clone().requires_grad_(want_grads) for t in (q, k, v))

@@ -1,0 +1,106 @@
+"""The C-ABI library loads and exports what include/trifast_hip.h declares.
+
+No kernel is launched here: the checks stop at argument validation and the
+host-side tile tables, none of which touch the GPU.
+"""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from trifast_amd import _lib
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "trifast_hip.h"
+
+
+def declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(trifast_\w+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    lib = _lib.load()
+    names = declared_functions()
+    assert len(names) >= 11
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature"
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_abi_version_matches_header():
+    want = int(re.search(r"#define TRIFAST_ABI_VERSION (\d+)", HEADER.read_text()).group(1))
+    assert _lib.load().trifast_abi_version() == want == _lib.ABI_VERSION
+
+
+def test_tile_tables():
+    lib = _lib.load()
+    for kernel in range(4):
+        nt = lib.trifast_num_tiles(kernel)
+        assert 1 <= nt <= 8
+        for t in range(nt):
+            info = _lib.tile_info(kernel, t)
+            assert info["BLOCK_J"] % 32 == 0 and info["BLOCK_K"] % 32 == 0 and info["num_waves"] in (1, 2, 4, 8)
+        with pytest.raises(ValueError):
+            _lib.tile_info(kernel, nt)
+    assert lib.trifast_num_tiles(99) < 0
+
+
+@pytest.mark.parametrize("dtype", [_lib.F32, _lib.BF16, _lib.F16])
+@pytest.mark.parametrize("d", [16, 32, 64, 128])
+def test_every_shape_has_a_default_tile(dtype, d):
+    lib = _lib.load()
+    for kernel in range(4):
+        for n in (1, 17, 256, 2048):
+            t = lib.trifast_default_tile(kernel, n, 4, d, dtype)
+            assert t >= 0, _lib.last_error()
+            assert lib.trifast_supports(kernel, t, n, 4, d, dtype) == 1
+
+
+def test_unsupported_head_dim_and_dtype():
+    lib = _lib.load()
+    assert lib.trifast_supports(0, 0, 64, 4, 48, _lib.BF16) == 0
+    assert lib.trifast_supports(0, 0, 64, 4, 32, 7) == 0
+    assert lib.trifast_default_tile(0, 64, 4, 48, _lib.BF16) < 0
+
+
+def test_workspace_sizes_are_quadratic_in_n():
+    lib = _lib.load()
+    f1 = lib.trifast_fwd_workspace_bytes(1, 4, 1024, 32, _lib.BF16)
+    b1 = lib.trifast_bwd_workspace_bytes(1, 4, 1024, 32, _lib.BF16)
+    b2 = lib.trifast_bwd_workspace_bytes(1, 4, 2048, 32, _lib.BF16)
+    assert 0 < f1 < 1 << 20
+    assert 4 * 1024 * 1024 * 4 <= b1 <= 4 * 1024 * 1024 * 4 + (1 << 20)
+    assert 3.9 < b2 / b1 < 4.1
+    assert lib.trifast_fwd_workspace_bytes(0, 4, 16, 32, _lib.BF16) < 0
+
+
+def test_argument_errors_come_back_as_codes_not_crashes():
+    lib = _lib.load()
+    st5 = _lib.i64_array([0, 0, 0, 32, 1])
+    st4 = _lib.i64_array([0, 0, 8, 1])
+    st3 = _lib.i64_array([0, 8, 1])
+    args = lambda d, q: (0x1000, 0x1000, q, 0x1000, 0x1000, 0x1000, 0x1000, 1, 1, 8, d, _lib.BF16, st5, st5, st5, st4, st3, -1, None, 0, None)
+    rc = lib.trifast_fwd(*args(48, 0x1000))
+    assert rc == -2 and "head dim" in _lib.last_error()
+    rc = lib.trifast_fwd(*args(32, 0x1008))
+    assert rc == -3 and "aligned" in _lib.last_error()
+    rc = lib.trifast_fwd(*args(32, 0x1000))  # passes the pointer checks, has no workspace
+    assert rc == -4 and "workspace" in _lib.last_error()
+    with pytest.raises(ValueError):
+        _lib.check(rc, "trifast_fwd")
+    bad_stride = _lib.i64_array([0, 0, 0, 32, 2])
+    rc = lib.trifast_fwd(0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 1, 1, 8, 32, _lib.BF16, bad_stride, st5, st5, st4, st3, -1, None, 0, None)
+    assert rc == -3 and "last stride" in _lib.last_error()
+    rc = lib.trifast_bwd_one(0, *([0x1000] * 12), 1, 1, 8, 32, _lib.BF16, st5, st5, st5, st5, st4, st3, -1, None, 0, None)
+    assert rc == -1 and "backward kernel" in _lib.last_error()
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libtrifast_hip.so")
+    with pytest.raises(ImportError, match="no fallback"):
+        _lib.load()

@@ -1,0 +1,146 @@
+"""Host-side logic that needs no GPU: operator schema and fake kernels, input
+validation, stride handling, the tile cache and the tune CLI."""
+
+import json
+
+import pytest
+import torch
+
+import trifast
+import trifast_amd
+from trifast_amd import _lib, tune, tuner
+from trifast_amd import torch as tt
+
+
+def meta_inputs(b=1, h=2, n=8, d=16, dtype=torch.bfloat16):
+    q = torch.empty(b, h, n, n, d, device="meta", dtype=dtype)
+    bias = torch.empty(b, h, n, n, device="meta", dtype=dtype)
+    mask = torch.empty(b, n, n, device="meta", dtype=torch.bool)
+    return q, q, q, bias, mask
+
+
+def test_public_surface_matches_reference_names():
+    # reference src/trifast/__init__.py:1-3, src/trifast/torch.py:17,68,185,210,220
+    assert trifast.triangle_attention is trifast_amd.triangle_attention
+    import trifast.torch as rt
+
+    for name in ("triangle_attention", "_triangle_attention", "triangle_attention_bwd", "backwards", "setup_context"):
+        assert hasattr(rt, name)
+    assert hasattr(torch.ops.trifast, "triangle_attention")
+    assert hasattr(torch.ops.trifast, "triangle_attention_backward")
+    from trifast.utils import clone_and_clear_grad, disable_tf32, enable_tf32, gen_tensors  # noqa: F401
+
+
+def test_fake_kernels_give_reference_shapes():
+    q, k, v, b, m = meta_inputs()
+    o, lse = torch.ops.trifast.triangle_attention(q, k, v, b, m)
+    assert o.shape == q.shape and o.dtype == q.dtype
+    assert lse.shape == (1, 2, 8, 8) and lse.dtype == torch.float32
+    outs = torch.ops.trifast.triangle_attention_backward(o, q, k, v, b, o, lse, m)
+    assert [t.shape for t in outs] == [q.shape, q.shape, q.shape, b.shape, m.shape]
+    assert outs[4].dtype == torch.bool
+
+
+def test_cpu_tensors_are_rejected_not_computed():
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(1, 1, 4, 4, 16, generator=g)
+    b = torch.randn(1, 1, 4, 4, generator=g)
+    m = torch.zeros(1, 4, 4, dtype=torch.bool)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        trifast_amd.triangle_attention(q, q, q, b, m)
+
+
+@pytest.mark.parametrize(
+    "mutate, err",
+    [
+        (lambda a: a.__setitem__(0, a[0][..., :3, :, :]), ValueError),      # not square
+        (lambda a: a.__setitem__(3, a[3][..., :3]), ValueError),            # bias shape
+        (lambda a: a.__setitem__(4, a[4].to(torch.uint8)), TypeError),      # mask dtype
+        (lambda a: a.__setitem__(1, a[1].to(torch.float16)), TypeError),    # mixed dtypes
+        (lambda a: a.__setitem__(0, a[0][0]), ValueError),                  # rank
+    ],
+)
+def test_input_validation(mutate, err):
+    q = torch.zeros(1, 2, 4, 4, 16, dtype=torch.bfloat16)
+    args = [q, q.clone(), q.clone(), torch.zeros(1, 2, 4, 4, dtype=torch.bfloat16), torch.zeros(1, 4, 4, dtype=torch.bool)]
+    mutate(args)
+    with pytest.raises(err):
+        tt._check_inputs(*args)
+
+
+def test_vector_ready_keeps_transposed_views_and_copies_the_rest():
+    x = torch.zeros(1, 2, 8, 8, 16, dtype=torch.bfloat16)
+    assert tt._vector_ready(x) is x
+    xt = x.transpose(2, 3)
+    assert tt._vector_ready(xt) is xt                       # i<->j view: read in place
+    assert tt._vector_ready(x[..., ::2]).is_contiguous()    # d stride 2: copied
+    ones = torch.ones((), dtype=torch.bfloat16).expand(1, 2, 8, 8, 16)
+    assert tt._vector_ready(ones).is_contiguous()           # stride-0 upstream gradient
+    assert tt._strides(torch.zeros(1, 2, 8, 8, 16))[0] == 0  # size-1 dims report stride 0
+
+
+def test_key_and_closest_n():
+    assert tuner.closest_n(1) == 1 and tuner.closest_n(17) == 32 and tuner.closest_n(1024) == 1024 and tuner.closest_n(1025) == 2048
+    assert tuner.make_key(191, 4, 32, torch.bfloat16) == "4_32_256_torch.bfloat16"
+
+
+def test_tile_cache_roundtrip_and_corruption(tmp_path, monkeypatch, capsys):
+    monkeypatch.setenv("TRIFAST_CONFIG_DIR", str(tmp_path))
+    monkeypatch.setattr(tuner, "_device_tag", lambda device=None: "Test-GPU_9-5")
+    tuner.reset()
+    c = tuner.TileCache(_lib.KERNEL_FWD)
+    assert c.cache_file == tmp_path / "_fwd_Test-GPU_9-5.json"
+    c.cache["4_32_1024_torch.bfloat16"] = 1
+    c.write()
+    raw = json.loads(c.cache_file.read_text())
+    assert raw["4_32_1024_torch.bfloat16"]["tile"] == 1
+    assert raw["4_32_1024_torch.bfloat16"]["kwargs"] == {k: v for k, v in _lib.tile_info(0, 1).items() if k != "num_waves"}
+    assert tuner.TileCache(_lib.KERNEL_FWD).cache == {"4_32_1024_torch.bfloat16": 1}
+    # an entry from another tile table is dropped, a corrupt file is reported and ignored
+    raw["4_32_1024_torch.bfloat16"]["kwargs"]["BLOCK_J"] = 12345
+    c.cache_file.write_text(json.dumps(raw))
+    assert tuner.TileCache(_lib.KERNEL_FWD).cache == {}
+    c.cache_file.write_text("{not json")
+    assert tuner.TileCache(_lib.KERNEL_FWD).cache == {}
+    assert "Could not load autotune cache" in capsys.readouterr().out
+    tuner.reset()
+
+
+def test_pick_without_autotune_uses_library_heuristic(monkeypatch):
+    monkeypatch.setenv("TRIFAST_AUTOTUNE", "0")
+    monkeypatch.delenv("TRIFAST_FORCE_TUNE", raising=False)
+    called = []
+    t = tuner.pick(_lib.KERNEL_FWD, 1024, 4, 32, torch.bfloat16, called.append)
+    assert t == _lib.load().trifast_default_tile(0, 1024, 4, 32, _lib.BF16) and called == []
+
+
+def test_pick_times_every_supported_tile_on_a_miss(tmp_path, monkeypatch):
+    monkeypatch.setenv("TRIFAST_CONFIG_DIR", str(tmp_path))
+    monkeypatch.setenv("TRIFAST_AUTOTUNE", "1")
+    monkeypatch.delenv("TRIFAST_FORCE_TUNE", raising=False)
+    monkeypatch.setattr(tuner, "_device_tag", lambda device=None: "Test-GPU_9-5")
+    fake_ms = {0: 3.0, 1: 1.0, 2: 5.0, 3: 2.0}
+    monkeypatch.setattr(tuner, "_time_launch", lambda launch, tile, **kw: fake_ms[tile])
+    tuner.reset()
+    assert tuner.pick(_lib.KERNEL_FWD, 300, 4, 32, torch.bfloat16, lambda t: None) == 1
+    assert json.loads((tmp_path / "_fwd_Test-GPU_9-5.json").read_text())["4_32_512_torch.bfloat16"]["tile"] == 1
+    # a hit does not time again
+    monkeypatch.setattr(tuner, "_time_launch", lambda *a, **k: pytest.fail("re-tuned on a cache hit"))
+    assert tuner.pick(_lib.KERNEL_FWD, 400, 4, 32, torch.bfloat16, lambda t: None) == 1
+    # TRIFAST_FORCE_TUNE re-tunes even on a hit
+    monkeypatch.setenv("TRIFAST_FORCE_TUNE", "yes")
+    monkeypatch.setattr(tuner, "_time_launch", lambda launch, tile, **kw: float(tile != 3))
+    assert tuner.pick(_lib.KERNEL_FWD, 400, 4, 32, torch.bfloat16, lambda t: None) == 3
+    tuner.reset()
+
+
+def test_tune_cli_flags_and_sweep():
+    p = tune.build_parser()
+    a = p.parse_args([])
+    assert (a.min_n, a.max_n, a.h, a.d, a.dtype) == (16, 1024, [4], [32], [torch.bfloat16])
+    a = p.parse_args(["--min-n", "64", "--max-n", "300", "--dtype", "float16,float32", "--h", "1,4", "--d", "16,64"])
+    assert a.h == [1, 4] and a.d == [16, 64] and set(a.dtype) == {torch.float16, torch.float32}
+    assert tune.sweep_ns(a.min_n, a.max_n) == [64, 128, 256]
+    assert len(tune.valid_dtypes("all")) == 3
+    with pytest.raises(SystemExit):
+        p.parse_args(["--dtype", "int8"])
