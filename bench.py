@@ -123,7 +123,7 @@ def kernel_breakdown(q, k, v, bias, mask, do, reps):
     b, h, n, _, d = q.shape
     code = tt._DTYPE_CODE[q.dtype]
     qv, kv, vv, dov = (tt._vector_ready(t) for t in (q, k, v, do))
-    bv = tt._bias_ready(bias)
+    bv = bias
     mu8 = mask.view(torch.uint8)
     o, lse = tt._triangle_attention(q, k, v, bias, mask)
     dq, dk, dv = (torch.empty_like(o) for _ in range(3))

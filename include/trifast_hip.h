@@ -16,13 +16,14 @@
  *   - Launches are asynchronous on `stream` (a hipStream_t passed as void*).
  *   - Layouts (reference src/trifast/torch.py:220-226):
  *       q, k, v, do : [b, h, n, n, d]  element strides {sb, sh, si, sj, sd}, sd == 1
- *       bias        : [b, h, n, n]     element strides {sb, sh, sj, sk}, sk == 1
+ *       bias        : [b, h, n, n]     element strides {sb, sh, sj, sk}, any
  *       mask        : [b, n, n] bytes  strides {sb, si, sk}, any; nonzero = key masked OUT
  *       o, dq, dk, dv : contiguous [b, h, n, n, d];  db : contiguous [b, h, n, n]
  *       lse         : contiguous float32 [b, h, n, n], natural log, indexed [i, j]
  *     Vector loads need 16-byte alignment: base pointers of q, k, v, do, o must be
  *     16-byte aligned and their si/sj/sh/sb strides multiples of 16/sizeof(elem).
- *     bias may have any row stride (an unaligned row takes an element-wise path).
+ *     bias and mask are re-tiled by pre-pass kernels into the workspace, so they
+ *     carry no alignment or contiguity requirement.
  */
 #ifndef TRIFAST_HIP_H
 #define TRIFAST_HIP_H

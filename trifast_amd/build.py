@@ -25,6 +25,8 @@ HIPCC_FLAGS = [
     "-std=c++17",
     "-fPIC",
     "-fno-gpu-rdc",
+    # keep MFMA accumulators in VGPRs: no accvgpr copies around the softmax math
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     # packed fp32 VALU forms are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]

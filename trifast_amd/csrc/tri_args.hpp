@@ -4,10 +4,8 @@
 
 namespace tri {
 
-// strides are in elements; the last (d) stride of q/k/v/do is 1, the last (k)
-// stride of bias is 1.
+// strides are in elements; the last (d) stride of q/k/v/do is 1
 struct Str5 { int64_t b, h, i, j; };   // [b, h, i, j, d], d contiguous
-struct Str4 { int64_t b, h, j; };      // bias [b, h, j, k], k contiguous
 
 struct MaskPrepArgs {
   const uint8_t* mask;       // [b, n, n] bytes, nonzero = masked out
@@ -17,32 +15,44 @@ struct MaskPrepArgs {
   int n, nwords;
 };
 
+// The bias is re-tiled once per call into the exact register layout the kernels
+// consume, zero-padded to whole 32 x 32 tiles, so that every wave-level load is
+// one contiguous 1 KiB read with no bounds or alignment cases:
+//   pack[((((bh*NP + jt)*NP + kt)*2 + r)*64 + lane)*8 + e]
+//   packq (lane owns a query): bias[32 jt + lane%32][32 kt + 16 r + 8 (lane/32) + e]
+//   packk (lane owns a key):   bias[32 jt + 16 r + 8 (lane/32) + e][32 kt + lane%32]
+struct BiasPrepArgs {
+  const void* bias;          // [b, h, n, n], any strides
+  int64_t sb, sh, sj, sk;
+  void* packq;               // may be null
+  void* packk;               // may be null
+  int H, N, NP;
+};
+
 struct FwdArgs {
-  const void *q, *k, *v, *bias;
+  const void *q, *k, *v;
+  const void* packq;
   const uint32_t* keep;
   const uint8_t* rowflag;
   void* o;
   float* lse;
   Str5 sq, sk, sv;
-  Str4 sbias;
-  int H, N, nwords;
-  int bias_vec_ok;           // bias rows 16-byte aligned: vector path allowed
+  int H, N, NP, nwords;
   float c;                   // log2(e) / sqrt(d): raw score -> log2 domain
   float sqrt_d;              // bias multiplier into the raw-score domain
   float neg_inf;             // finfo(dtype).min, reported in lse of fully masked rows
 };
 
 struct BwdArgs {
-  const void *q, *k, *v, *bias, *o, *dout;
+  const void *q, *k, *v, *o, *dout;
+  const void *packq, *packk;
   const float* lse;
   const uint32_t* keep;
   const uint8_t* rowflag;
   float* delta;              // [b*h, n, n] fp32 workspace, indexed [i, j]
   void *dq, *dk, *dv, *db;
   Str5 sq, sk, sv, sdo;
-  Str4 sbias;
-  int H, N, nwords;
-  int bias_vec_ok;
+  int H, N, NP, nwords;
   float c;                   // log2(e) / sqrt(d)
   float sqrt_d;
   float scale;               // 1 / sqrt(d)

@@ -12,7 +12,7 @@
 #pragma once
 #include "tri_args.hpp"
 #include "tri_common.hpp"
-#include "tri_fwd.hpp"
+#include "tri_tile.hpp"
 
 namespace tri {
 
@@ -49,7 +49,7 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
   const T* kbase = reinterpret_cast<const T*>(a.k) + b * a.sk.b + h * a.sk.h;
   const T* vbase = reinterpret_cast<const T*>(a.v) + b * a.sv.b + h * a.sv.h;
   const T* dobase = reinterpret_cast<const T*>(a.dout) + b * a.sdo.b + h * a.sdo.h;
-  const T* bias_bh = reinterpret_cast<const T*>(a.bias) + b * a.sbias.b + h * a.sbias.h;
+  const T* pack_bh = reinterpret_cast<const T*>(a.packq) + (int64_t)bh * a.NP * a.NP * 1024;
   const float* lse_bh = a.lse + (int64_t)bh * N * N;
   const float* delta_bh = a.delta + (int64_t)bh * N * N;
   const uint32_t* keep_b = a.keep + (int64_t)b * N * a.nwords;
@@ -59,18 +59,10 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
   // bias tile in the raw-score domain, used as the accumulator init of every row
   f32x16 biasr[WJ][WK];
 #pragma unroll
-  for (int tj = 0; tj < WJ; ++tj) {
-    const int j = j_wave + 32 * tj + jl;
-    const T* brow = bias_bh + (int64_t)j * a.sbias.j;
+  for (int tj = 0; tj < WJ; ++tj)
 #pragma unroll
-    for (int tk = 0; tk < WK; ++tk) {
-      float bv[16];
-      load_bias8<T>(brow, k_wave + 32 * tk + 8 * g, N, j < N, a.bias_vec_ok, bv);
-      load_bias8<T>(brow, k_wave + 32 * tk + 16 + 8 * g, N, j < N, a.bias_vec_ok, bv + 8);
-#pragma unroll
-      for (int v = 0; v < 16; ++v) biasr[tj][tk][v] = bv[v] * a.sqrt_d;
-    }
-  }
+    for (int tk = 0; tk < WK; ++tk)
+      biasr[tj][tk] = bias_tile<T>(pack_bh, a.NP, (j_wave >> 5) + tj, (k_wave >> 5) + tk, lane, a.sqrt_d, 0.f);
 
   f32x16 dbacc[WJ][WK];
 #pragma unroll

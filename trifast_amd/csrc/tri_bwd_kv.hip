@@ -20,12 +20,10 @@ struct BwdKVFamily {
   template <typename T, int D, int NW, int KT, int BJ>
   static hipError_t run(const BwdArgs& a, int bh, hipStream_t st, bool dry) {
     constexpr int PAD = 16 / sizeof(T);
-    constexpr int DROWS = ((D + 31) / 32) * 32;
-    constexpr int lds = (sizeof(T) == 2 ? (2 * BJ * (D + PAD) + 2 * DROWS * (BJ + PAD)) * 2
-                                        : 2 * BJ * (D + PAD) * 4 + 32) + 8 * BJ;
+    constexpr int lds = 2 * BJ * (D + PAD) * (int)sizeof(T) + 8 * BJ;
     if constexpr (lds <= kMaxStaticLds) {
       if (dry) return hipSuccess;
-      dim3 grid((a.N + NW * KT * 32 - 1) / (NW * KT * 32), a.N, bh);
+      dim3 grid((a.N + NW * KT * 32 - 1) / (NW * KT * 32), (a.N + 7) / 8 * 8, bh);
       hipLaunchKernelGGL((tri_bwd_kv_kernel<T, D, NW, KT, BJ>), grid, dim3(NW * 64), 0, st, a);
       return hipGetLastError();
     } else {

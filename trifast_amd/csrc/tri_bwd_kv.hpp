@@ -2,18 +2,19 @@
 //
 // Work unit: (batch*head, row i, block of NW*KT*32 keys).  Each wave keeps KT
 // tiles of 32 keys (K and V rows as B operands) in registers and streams the
-// queries of the row through LDS in tiles of BJ.  Scores are computed
-// UN-transposed here, S = Q K^T, so that a lane owns one key (column) and 16
-// queries of every 32-query tile: P and dS are then already in B-operand layout
-// for the two products that contract over queries,
-//   dv^T += dO^T P,   dk^T += Q^T dS,   dk = dk^T / sqrt(d).
-// The key mask is a per-lane constant folded into the score accumulator init.
+// queries of the row through LDS in tiles of BJ (natural layout).  Scores are
+// computed UN-transposed here, S = Q K^T, so that a lane owns one key (column)
+// and 16 queries of every 32-query tile: P and dS are then already in B-operand
+// layout for the two products that contract over queries,
+//   dv^T += dO^T P,   dk^T += Q^T dS,   dk = dk^T / sqrt(d),
+// whose A operands dO^T, Q^T come from the natural tiles through transposing LDS
+// reads.  The key mask is a per-lane constant folded into the bias conversion.
 //
 // Replaces _bwd_kv of reference src/trifast/triton.py:143-263.
 #pragma once
 #include "tri_args.hpp"
 #include "tri_common.hpp"
-#include "tri_fwd.hpp"
+#include "tri_tile.hpp"
 
 namespace tri {
 
@@ -24,30 +25,27 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
   constexpr int KP = E::KP;
   constexpr int DS = D / (2 * KP);
   constexpr int DM = (D + 31) / 32;
-  constexpr int DROWS = DM * 32;
   constexpr int PS = 32 / (2 * KP);
   constexpr int JU = BJ / 32;
   constexpr int PAD = 16 / sizeof(T);
+  constexpr int LD = D + PAD;
   constexpr int NT = NW * 64;
 
-  __shared__ __attribute__((aligned(16))) T Qs[BJ][D + PAD];
-  __shared__ __attribute__((aligned(16))) T dOs[BJ][D + PAD];
-  // fp32 operands are single elements, so the natural-layout tiles serve the
-  // transposed reads as well and no transposed copy is kept
-  constexpr bool kTr = KP > 1;
-  constexpr int TROWS = kTr ? DROWS : 1, TLD = kTr ? BJ + PAD : 4;
-  __shared__ __attribute__((aligned(16))) T Qt[TROWS][TLD];
-  __shared__ __attribute__((aligned(16))) T dOt[TROWS][TLD];
+  __shared__ __attribute__((aligned(16))) T Qs[BJ][LD];
+  __shared__ __attribute__((aligned(16))) T dOs[BJ][LD];
   __shared__ __attribute__((aligned(16))) float lse2s[BJ];
   __shared__ __attribute__((aligned(16))) float deltas[BJ];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int kl = lane & 31, g = lane >> 5;
-  const int bh = blockIdx.z, i = blockIdx.y;
-  const int b = bh / a.H, h = bh % a.H;
   const int N = a.N;
-  const int k_wave = blockIdx.x * (NW * KT * 32) + wave * (KT * 32);
+  int bx, i;
+  xcd_remap(gridDim.x, bx, i);
+  if (i >= N) return;
+  const int bh = blockIdx.z;
+  const int b = bh / a.H, h = bh % a.H;
+  const int k_wave = bx * (NW * KT * 32) + wave * (KT * 32);
   const bool wave_active = k_wave < N;
 
   const bool flagged = a.rowflag[(int64_t)b * N + i] != 0;
@@ -57,16 +55,9 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
   const T* krow = reinterpret_cast<const T*>(a.k) + b * a.sk.b + h * a.sk.h + i * a.sk.i;
   const T* vrow = reinterpret_cast<const T*>(a.v) + b * a.sv.b + h * a.sv.h + i * a.sv.i;
   const T* dorow = reinterpret_cast<const T*>(a.dout) + b * a.sdo.b + h * a.sdo.h + i * a.sdo.i;
-  const T* bias_bh = reinterpret_cast<const T*>(a.bias) + b * a.sbias.b + h * a.sbias.h;
+  const T* pack_bh = reinterpret_cast<const T*>(a.packk) + (int64_t)bh * a.NP * a.NP * 1024;
   const float* lse_row = a.lse + ((int64_t)bh * N + i) * N;
   const float* delta_row = a.delta + ((int64_t)bh * N + i) * N;
-
-  if constexpr (kTr && DROWS > D) {
-    for (int c = tid; c < (DROWS - D) * (BJ + PAD); c += NT) {
-      Qt[D + c / (BJ + PAD)][c % (BJ + PAD)] = (T)0.f;
-      dOt[D + c / (BJ + PAD)][c % (BJ + PAD)] = (T)0.f;
-    }
-  }
 
   // K and V tiles as B operands: lane owns key k_wave + 32 t + kl
   frag kf[KT][DS], vf[KT][DS];
@@ -105,12 +96,8 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
   const float lse2_flagged = fast_log2((float)N);
   for (int jt0 = 0; jt0 < N; jt0 += BJ) {
     __syncthreads();
-    lds_load_natural<T, D, BJ, D + PAD, NT>(Qs, qrow + (int64_t)jt0 * a.sq.j, a.sq.j, N - jt0, tid);
-    lds_load_natural<T, D, BJ, D + PAD, NT>(dOs, dorow + (int64_t)jt0 * a.sdo.j, a.sdo.j, N - jt0, tid);
-    if constexpr (kTr) {
-      lds_load_transposed<T, D, BJ, TLD, NT>(Qt, qrow + (int64_t)jt0 * a.sq.j, a.sq.j, N - jt0, tid);
-      lds_load_transposed<T, D, BJ, TLD, NT>(dOt, dorow + (int64_t)jt0 * a.sdo.j, a.sdo.j, N - jt0, tid);
-    }
+    lds_load_natural<T, D, BJ, LD, NT>(Qs, qrow + (int64_t)jt0 * a.sq.j, a.sq.j, N - jt0, tid);
+    lds_load_natural<T, D, BJ, LD, NT>(dOs, dorow + (int64_t)jt0 * a.sdo.j, a.sdo.j, N - jt0, tid);
     for (int x = tid; x < BJ; x += NT) {
       const int j = jt0 + x;
       lse2s[x] = (j < N) ? (flagged ? lse2_flagged : lse_row[j] * kLog2e) : 0.f;
@@ -135,14 +122,8 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
       for (int mt = 0; mt < DM; ++mt)
 #pragma unroll
         for (int s2 = 0; s2 < PS; ++s2) {
-          if constexpr (kTr) {
-            qtf[mt][s2] = *reinterpret_cast<const frag*>(&Qt[32 * mt + kl][32 * u + cidx(KP * s2, g)]);
-            dotf[mt][s2] = *reinterpret_cast<const frag*>(&dOt[32 * mt + kl][32 * u + cidx(KP * s2, g)]);
-          } else {
-            const bool din = 32 * mt + kl < D;
-            qtf[mt][s2] = din ? *reinterpret_cast<const frag*>(&Qs[32 * u + cidx(s2, g)][32 * mt + kl]) : E::zero();
-            dotf[mt][s2] = din ? *reinterpret_cast<const frag*>(&dOs[32 * u + cidx(s2, g)][32 * mt + kl]) : E::zero();
-          }
+          qtf[mt][s2] = tr_operand<T, LD>(Qs, 32 * u, s2, 32 * mt, D, lane);
+          dotf[mt][s2] = tr_operand<T, LD>(dOs, 32 * u, s2, 32 * mt, D, lane);
         }
       // per-query statistics of the 16 queries this lane sees: two runs of 8
       float l2[16], dl[16];
@@ -162,15 +143,9 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
 #pragma unroll
       for (int t = 0; t < KT; ++t) {
         if (!tile_live[t]) continue;
-        const int key = k_wave + 32 * t + kl;
         f32x16 s;
         if (!flagged) {
-#pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int j = jt0 + 32 * u + cidx(v, g);
-            const float bval = (j < N && key < N) ? (float)bias_bh[(int64_t)j * a.sbias.j + key] : 0.f;
-            s[v] = __builtin_fmaf(bval, a.sqrt_d, lanebias[t]);
-          }
+          s = bias_tile<T>(pack_bh, a.NP, (jt0 >> 5) + u, (k_wave >> 5) + t, lane, a.sqrt_d, lanebias[t]);
         } else {
 #pragma unroll
           for (int v = 0; v < 16; ++v) s[v] = lanebias[t];
@@ -208,23 +183,8 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
   for (int t = 0; t < KT; ++t) {
     const int key = k_wave + 32 * t + kl;
     if (key >= N) continue;
-#pragma unroll
-    for (int mt = 0; mt < DM; ++mt) {
-#pragma unroll
-      for (int a4 = 0; a4 < 4; ++a4) {
-        const int d0 = 32 * mt + 8 * a4 + 4 * g;
-        if (d0 < D) {
-          typename E::vec4 kv, vv;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            kv[e] = (T)(dkacc[t][mt][4 * a4 + e] * a.scale);
-            vv[e] = (T)(dvacc[t][mt][4 * a4 + e]);
-          }
-          *reinterpret_cast<typename E::vec4*>(dkrow + (int64_t)key * D + d0) = kv;
-          *reinterpret_cast<typename E::vec4*>(dvrow + (int64_t)key * D + d0) = vv;
-        }
-      }
-    }
+    store_rows<T, D, DM>(dkrow + (int64_t)key * D, dkacc[t], a.scale, g);
+    store_rows<T, D, DM>(dvrow + (int64_t)key * D, dvacc[t], 1.0f, g);
   }
 }
 

@@ -20,12 +20,10 @@ struct BwdQFamily {
   template <typename T, int D, int NW, int QT, int BK>
   static hipError_t run(const BwdArgs& a, int bh, hipStream_t st, bool dry) {
     constexpr int PAD = 16 / sizeof(T);
-    constexpr int DROWS = ((D + 31) / 32) * 32;
-    constexpr int lds = sizeof(T) == 2 ? (2 * BK * (D + PAD) + DROWS * (BK + PAD)) * 2
-                                       : 2 * BK * (D + PAD) * 4 + 16;
+    constexpr int lds = 2 * BK * (D + PAD) * (int)sizeof(T);
     if constexpr (lds <= kMaxStaticLds) {
       if (dry) return hipSuccess;
-      dim3 grid((a.N + NW * QT * 32 - 1) / (NW * QT * 32), a.N, bh);
+      dim3 grid((a.N + NW * QT * 32 - 1) / (NW * QT * 32), (a.N + 7) / 8 * 8, bh);
       hipLaunchKernelGGL((tri_bwd_q_kernel<T, D, NW, QT, BK>), grid, dim3(NW * 64), 0, st, a);
       return hipGetLastError();
     } else {

@@ -51,6 +51,54 @@ hipError_t mask_prep_launch(const MaskPrepArgs& a, int b, hipStream_t st) {
   return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// Bias pre-pass: re-tile bias[b, h, j, k] (any strides) into the register layouts
+// of the kernels (see BiasPrepArgs), zero-padded to whole tiles.  One thread
+// writes the 8 elements of one (tile, r, lane) slot of each requested layout.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void bias_prep_kernel(const BiasPrepArgs a) {
+  const int bh = blockIdx.y;
+  const int b = bh / a.H, h = bh % a.H;
+  const int64_t slot = (int64_t)blockIdx.x * 256 + threadIdx.x;  // ((jt*NP + kt)*2 + r)*64 + lane
+  if (slot >= (int64_t)a.NP * a.NP * 128) return;
+  const int lane = slot & 63, r = (slot >> 6) & 1;
+  const int tile = (int)(slot >> 7);
+  const int jt = tile / a.NP, kt = tile % a.NP;
+  const int l32 = lane & 31, g = lane >> 5;
+  const T* src = reinterpret_cast<const T*>(a.bias) + b * a.sb + h * a.sh;
+  const int64_t out = ((int64_t)bh * a.NP * a.NP * 128 + slot) * 8;
+  if (a.packq) {
+    T* dst = reinterpret_cast<T*>(a.packq) + out;
+    const int j = 32 * jt + l32;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int key = 32 * kt + 16 * r + 8 * g + e;
+      dst[e] = (j < a.N && key < a.N) ? src[j * a.sj + key * a.sk] : (T)0.f;
+    }
+  }
+  if (a.packk) {
+    T* dst = reinterpret_cast<T*>(a.packk) + out;
+    const int key = 32 * kt + l32;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = 32 * jt + 16 * r + 8 * g + e;
+      dst[e] = (j < a.N && key < a.N) ? src[j * a.sj + key * a.sk] : (T)0.f;
+    }
+  }
+}
+
+hipError_t bias_prep_launch(const BiasPrepArgs& a, int bh, int dtype, hipStream_t st) {
+  const int64_t slots = (int64_t)a.NP * a.NP * 128;
+  dim3 grid((unsigned)((slots + 255) / 256), bh);
+  switch (dtype) {
+    case kF32: hipLaunchKernelGGL(bias_prep_kernel<float>, grid, dim3(256), 0, st, a); break;
+    case kBF16: hipLaunchKernelGGL(bias_prep_kernel<__bf16>, grid, dim3(256), 0, st, a); break;
+    default: hipLaunchKernelGGL(bias_prep_kernel<_Float16>, grid, dim3(256), 0, st, a); break;
+  }
+  return hipGetLastError();
+}
+
 }  // namespace tri
 
 namespace {
@@ -81,11 +129,14 @@ float dtype_min(int dtype) {
   }
 }
 
+// workspace layout: keep words | row flags | packq | (backward only) packk | delta
 struct Workspace {
   uint32_t* keep;
   uint8_t* rowflag;
+  void* packq;
+  void* packk;
   float* delta;
-  int nwords;
+  int nwords, np;
 };
 
 int64_t ws_mask_bytes(int64_t b, int64_t n) {
@@ -93,7 +144,12 @@ int64_t ws_mask_bytes(int64_t b, int64_t n) {
   return align256(b * n * nwords * 4) + align256(b * n);
 }
 
-Workspace carve(void* ws, int64_t b, int64_t n) {
+int64_t ws_pack_bytes(int64_t b, int64_t h, int64_t n, int dtype) {
+  const int64_t np = (n + 31) / 32;
+  return align256(b * h * np * np * 1024 * elem_size(dtype));
+}
+
+Workspace carve(void* ws, int64_t b, int64_t h, int64_t n, int dtype) {
   Workspace w;
   const int64_t nwords = (n + 31) / 32;
   char* p = static_cast<char*>(ws);
@@ -101,8 +157,13 @@ Workspace carve(void* ws, int64_t b, int64_t n) {
   p += align256(b * n * nwords * 4);
   w.rowflag = reinterpret_cast<uint8_t*>(p);
   p += align256(b * n);
+  w.packq = p;
+  p += ws_pack_bytes(b, h, n, dtype);
+  w.packk = p;
+  p += ws_pack_bytes(b, h, n, dtype);
   w.delta = reinterpret_cast<float*>(p);
   w.nwords = (int)nwords;
+  w.np = (int)nwords;
   return w;
 }
 
@@ -127,8 +188,17 @@ int check_qlike(const char* name, const void* p, const int64_t* s, int dtype) {
 
 tri::Str5 str5(const int64_t* s) { return tri::Str5{s[0], s[1], s[2], s[3]}; }
 
-int bias_vec_ok(const void* bias, const int64_t* s) {
-  return ((reinterpret_cast<uintptr_t>(bias) & 15) == 0 && s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0) ? 1 : 0;
+int run_bias_prep(const void* bias, const int64_t* bs, const Workspace& w, bool want_k, int64_t b, int64_t h,
+                  int64_t n, int dtype, hipStream_t st) {
+  tri::BiasPrepArgs p;
+  p.bias = bias;
+  p.sb = bs[0]; p.sh = bs[1]; p.sj = bs[2]; p.sk = bs[3];
+  p.packq = w.packq;
+  p.packk = want_k ? w.packk : nullptr;
+  p.H = (int)h; p.N = (int)n; p.NP = w.np;
+  hipError_t e = tri::bias_prep_launch(p, (int)(b * h), dtype, st);
+  if (e != hipSuccess) return hip_fail(e, "bias pre-pass launch");
+  return 0;
 }
 
 int run_mask_prep(const uint8_t* mask, const int64_t* ms, const Workspace& w, int64_t b, int64_t n, hipStream_t st) {
@@ -212,15 +282,15 @@ int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype)
 }
 
 int64_t trifast_fwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype) {
-  (void)h; (void)d; (void)dtype;
-  if (b < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
-  return ws_mask_bytes(b, n);
+  (void)d;
+  if (b < 1 || h < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
+  return ws_mask_bytes(b, n) + ws_pack_bytes(b, h, n, dtype);
 }
 
 int64_t trifast_bwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype) {
-  (void)d; (void)dtype;
+  (void)d;
   if (b < 1 || h < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
-  return ws_mask_bytes(b, n) + align256(b * h * n * n * 4);
+  return ws_mask_bytes(b, n) + 2 * ws_pack_bytes(b, h, n, dtype) + align256(b * h * n * n * 4);
 }
 
 int trifast_fwd(void* o, float* lse, const void* q, const void* k, const void* v, const void* bias,
@@ -236,7 +306,6 @@ int trifast_fwd(void* o, float* lse, const void* q, const void* k, const void* v
   if ((rc = check_qlike("k", k, k_strides, dtype))) return rc;
   if ((rc = check_qlike("v", v, v_strides, dtype))) return rc;
   if ((reinterpret_cast<uintptr_t>(o) & 15) != 0) return fail(TRIFAST_EALIGN, "o: base pointer is not 16-byte aligned");
-  if (bias_strides[3] != 1) return fail(TRIFAST_EALIGN, "bias: last stride must be 1 (got %lld)", (long long)bias_strides[3]);
   if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
       workspace_bytes < trifast_fwd_workspace_bytes(b, h, n, d, dtype))
     return fail(TRIFAST_EWORKSPACE, "workspace missing, misaligned or smaller than trifast_fwd_workspace_bytes");
@@ -245,17 +314,16 @@ int trifast_fwd(void* o, float* lse, const void* q, const void* k, const void* v
   if (!tri::fwd_supports(tile, n, (int)d, dtype)) return fail(TRIFAST_EUNSUPPORTED, "forward tile %d does not support n=%lld d=%lld dtype=%d", tile, (long long)n, (long long)d, dtype);
 
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const Workspace w = carve(workspace, b, n);
+  const Workspace w = carve(workspace, b, h, n, dtype);
   if ((rc = run_mask_prep(mask, mask_strides, w, b, n, st))) return rc;
+  if ((rc = run_bias_prep(bias, bias_strides, w, false, b, h, n, dtype, st))) return rc;
 
   tri::FwdArgs a;
-  a.q = q; a.k = k; a.v = v; a.bias = bias;
+  a.q = q; a.k = k; a.v = v; a.packq = w.packq;
   a.keep = w.keep; a.rowflag = w.rowflag;
   a.o = o; a.lse = lse;
   a.sq = str5(q_strides); a.sk = str5(k_strides); a.sv = str5(v_strides);
-  a.sbias = tri::Str4{bias_strides[0], bias_strides[1], bias_strides[2]};
-  a.H = (int)h; a.N = (int)n; a.nwords = w.nwords;
-  a.bias_vec_ok = bias_vec_ok(bias, bias_strides);
+  a.H = (int)h; a.N = (int)n; a.NP = w.np; a.nwords = w.nwords;
   a.c = (float)(1.4426950408889634 / std::sqrt((double)d));
   a.sqrt_d = (float)std::sqrt((double)d);
   a.neg_inf = dtype_min(dtype);
@@ -278,7 +346,6 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   if ((rc = check_qlike("q", q, q_strides, dtype))) return rc;
   if ((rc = check_qlike("k", k, k_strides, dtype))) return rc;
   if ((rc = check_qlike("v", v, v_strides, dtype))) return rc;
-  if (bias_strides[3] != 1) return fail(TRIFAST_EALIGN, "bias: last stride must be 1 (got %lld)", (long long)bias_strides[3]);
   if ((reinterpret_cast<uintptr_t>(o) & 15) != 0) return fail(TRIFAST_EALIGN, "o: base pointer is not 16-byte aligned");
   if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
       workspace_bytes < trifast_bwd_workspace_bytes(b, h, n, d, dtype))
@@ -302,20 +369,20 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   if (do_b && !tri::bwd_b_supports(tb, n, (int)d, dtype)) return fail(TRIFAST_EUNSUPPORTED, "bwd_b tile %d unsupported for this shape", tb);
 
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const Workspace w = carve(workspace, b, n);
-  // The pre-pass is cheap (n^2 bytes) and makes every single-kernel call
-  // self-contained, so it runs whenever the first kernel of a call needs it.
+  const Workspace w = carve(workspace, b, h, n, dtype);
+  // The pre-passes are cheap (n^2 elements) and make every single-kernel call
+  // self-contained, so they run on every call.
   if ((rc = run_mask_prep(mask, mask_strides, w, b, n, st))) return rc;
+  if ((rc = run_bias_prep(bias, bias_strides, w, true, b, h, n, dtype, st))) return rc;
 
   tri::BwdArgs a;
-  a.q = q; a.k = k; a.v = v; a.bias = bias; a.o = o; a.dout = dout;
+  a.q = q; a.k = k; a.v = v; a.o = o; a.dout = dout;
+  a.packq = w.packq; a.packk = w.packk;
   a.lse = lse;
   a.keep = w.keep; a.rowflag = w.rowflag; a.delta = w.delta;
   a.dq = dq; a.dk = dk; a.dv = dv; a.db = db;
   a.sq = str5(q_strides); a.sk = str5(k_strides); a.sv = str5(v_strides); a.sdo = str5(do_strides);
-  a.sbias = tri::Str4{bias_strides[0], bias_strides[1], bias_strides[2]};
-  a.H = (int)h; a.N = (int)n; a.nwords = w.nwords;
-  a.bias_vec_ok = bias_vec_ok(bias, bias_strides);
+  a.H = (int)h; a.N = (int)n; a.NP = w.np; a.nwords = w.nwords;
   a.c = (float)(1.4426950408889634 / std::sqrt((double)d));
   a.sqrt_d = (float)std::sqrt((double)d);
   a.scale = (float)(1.0 / std::sqrt((double)d));

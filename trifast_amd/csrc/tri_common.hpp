@@ -102,14 +102,77 @@ struct Elem<float> {
   static TRI_DEV frag pack(const float* x) { return x[0]; }
 };
 
+typedef short s16x4v __attribute__((__vector_size__(4 * sizeof(short))));
+#define TRI_LDS __attribute__((address_space(3)))
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane L receives element e
+// (0..3) from the 64 bits supplied by lane 4e + L/4, at position L%4.  With lane
+// L' pointing at tile[row0 + L'/4][col0 + 4*(L'%4)], lane L ends up with
+// tile[row0 + e][col0 + L]: a column of four rows, i.e. the tile read transposed.
+TRI_DEV bf16x4 lds_tr4(const __bf16* p) {
+  const s16x4v r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TRI_LDS s16x4v*)(p));
+  return __builtin_bit_cast(bf16x4, r);
+}
+TRI_DEV f16x4 lds_tr4(const _Float16* p) {
+  const s16x4v r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TRI_LDS s16x4v*)(p));
+  return __builtin_bit_cast(f16x4, r);
+}
+
+// Operand with the contraction index in-lane, read from a natural row-major LDS
+// tile[rows = contraction index][cols]: the lane gets tile[row0 .. row0+7][col0 + lane%32]
+// (row0 must already include the lane group's +8*g).  Two transposed reads.
+template <typename T, int LD>
+TRI_DEV typename Elem<T>::frag lds_tr_frag(const T (*tile)[LD], int row0, int col0, int lane) {
+  static_assert(sizeof(T) == 2, "transposed LDS reads exist for 16-bit types only");
+  const int L = lane & 15, chalf = (lane >> 4) & 1;
+  const T* p = &tile[row0 + (L >> 2)][col0 + 16 * chalf + 4 * (L & 3)];
+  const auto lo = lds_tr4(p);
+  const auto hi = lds_tr4(p + 4 * LD);
+  typename Elem<T>::frag f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) { f[e] = lo[e]; f[4 + e] = hi[e]; }
+  return f;
+}
+
+// sum of the KP values of a packed operand, added to acc (consistent with what
+// the MFMA consumes: the rounded values are what is summed)
+TRI_DEV float frag_sum(bf16x8 f, float acc) {
+  const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+#pragma unroll
+  for (int e = 0; e < 8; e += 2) {
+    const bf16x2 pr = {f[e], f[e + 1]};
+    acc = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, acc, false);
+  }
+  return acc;
+}
+TRI_DEV float frag_sum(f16x8 f, float acc) {
+  const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+  for (int e = 0; e < 8; e += 2) {
+    const f16x2 pr = {f[e], f[e + 1]};
+    acc = __builtin_amdgcn_fdot2(pr, ones, acc, false);
+  }
+  return acc;
+}
+TRI_DEV float frag_sum(float f, float acc) { return acc + f; }
+
 template <typename T>
 TRI_DEV float to_f32(T x) { return (float)x; }
 
 TRI_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 TRI_DEV float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-// exchange with the lane that holds the other half of the same column
-TRI_DEV float xhalf(float x) { return __shfl_xor(x, 32, 64); }
+// Lane l and lane l^32 hold the two halves of one column.  v_permlane32_swap
+// hands every lane its own value and its partner's (in an order that depends on
+// the half), which is all a max or a sum of the two needs.
+TRI_DEV void half_pair(float x, float& a, float& b) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  a = __builtin_bit_cast(float, (unsigned)r[0]);
+  b = __builtin_bit_cast(float, (unsigned)r[1]);
+}
+TRI_DEV float half_max(float x) { float a, b; half_pair(x, a, b); return fmaxf(a, b); }
+TRI_DEV float half_sum(float x) { float a, b; half_pair(x, a, b); return a + b; }
 
 TRI_DEV f32x16 zero16() {
   f32x16 z;

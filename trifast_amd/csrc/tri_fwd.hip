@@ -20,11 +20,10 @@ struct FwdFamily {
   template <typename T, int D, int NW, int QT, int BK>
   static hipError_t run(const FwdArgs& a, int bh, hipStream_t st, bool dry) {
     constexpr int PAD = 16 / sizeof(T);
-    constexpr int DROWS = ((D + 31) / 32) * 32;
-    constexpr bool fits = (BK * (D + PAD) + DROWS * (BK + PAD)) * sizeof(T) <= kMaxStaticLds;
+    constexpr bool fits = 2 * BK * (D + PAD) * sizeof(T) <= kMaxStaticLds;
     if constexpr (fits) {
       if (dry) return hipSuccess;
-      dim3 grid((a.N + NW * QT * 32 - 1) / (NW * QT * 32), a.N, bh);
+      dim3 grid((a.N + NW * QT * 32 - 1) / (NW * QT * 32), (a.N + 7) / 8 * 8, bh);
       hipLaunchKernelGGL((tri_fwd_kernel<T, D, NW, QT, BK>), grid, dim3(NW * 64), 0, st, a);
       return hipGetLastError();
     } else {

@@ -32,6 +32,7 @@ bool bwd_b_supports(int tile, int64_t n, int d, int dtype);
 hipError_t bwd_b_launch(const BwdArgs& a, int bh, int d, int dtype, int tile, hipStream_t st);
 
 hipError_t mask_prep_launch(const MaskPrepArgs& a, int b, hipStream_t st);
+hipError_t bias_prep_launch(const BiasPrepArgs& a, int bh, int dtype, hipStream_t st);
 
 inline bool head_dim_ok(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }
 

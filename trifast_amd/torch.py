@@ -67,10 +67,6 @@ def _vector_ready(t: torch.Tensor) -> torch.Tensor:
     return t.contiguous()
 
 
-def _bias_ready(b: torch.Tensor) -> torch.Tensor:
-    return b if (b.stride(-1) == 1 or b.shape[-1] == 1) else b.contiguous()
-
-
 def _workspace(nbytes: int, device) -> torch.Tensor:
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
 
@@ -90,7 +86,8 @@ def _triangle_attention(
     lib = _lib.load()
     bs, h, n, d = _check_inputs(q, k, v, b, mask)
     code = _dtype_code(q)
-    q, k, v, b = _vector_ready(q), _vector_ready(k), _vector_ready(v), _bias_ready(b)
+    # bias and mask are re-tiled by the library's pre-passes, so any strides go
+    q, k, v = _vector_ready(q), _vector_ready(k), _vector_ready(v)
     mask_u8 = mask.view(torch.uint8)
 
     o = torch.empty((bs, h, n, n, d), dtype=q.dtype, device=q.device)
@@ -142,7 +139,8 @@ def triangle_attention_bwd(
     # the upstream gradient is often an expanded (stride-0) tensor, e.g. from
     # o.sum().backward(): _vector_ready materialises exactly those
     do = _vector_ready(do)
-    q, k, v, b = _vector_ready(q), _vector_ready(k), _vector_ready(v), _bias_ready(b)
+    # bias and mask are re-tiled by the library's pre-passes, so any strides go
+    q, k, v = _vector_ready(q), _vector_ready(k), _vector_ready(v)
     o = o.contiguous()
     l = l.contiguous()
     mask_u8 = mask.view(torch.uint8)
