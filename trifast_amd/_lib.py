@@ -10,7 +10,10 @@ import ctypes
 from ctypes import POINTER, c_char_p, c_int, c_int64, c_void_p
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "libtrifast_hip.so"
+import os
+
+# TRIFAST_LIB points at another build of the same library (kernel experiments)
+LIB_PATH = Path(os.environ.get("TRIFAST_LIB") or Path(__file__).resolve().parent / "libtrifast_hip.so")
 
 ABI_VERSION = 1
 

@@ -43,8 +43,8 @@ def sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
 
 
-def _compile(src: Path, obj: Path, verbose: bool) -> None:
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
+def _compile(src: Path, obj: Path, verbose: bool, extra: tuple[str, ...] = ()) -> None:
+    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src.name}:\n{res.stdout}\n{res.stderr}")
@@ -56,28 +56,38 @@ def _compile(src: Path, obj: Path, verbose: bool) -> None:
             print(msg, file=sys.stderr)
 
 
-def build(verbose: bool = False, jobs: int | None = None) -> Path:
-    """Compile every translation unit and link the shared library.  Always rebuilds."""
-    build_dir = PKG_DIR / "build"
-    build_dir.mkdir(exist_ok=True)
+def build(verbose: bool = False, jobs: int | None = None, out: Path | None = None, extra: tuple[str, ...] = ()) -> Path:
+    """Compile every translation unit and link the shared library.  Always rebuilds.
+
+    ``out`` / ``extra`` build a variant (other output path, extra hipcc flags such as
+    ``-DNAME``) without touching the in-tree library; used for kernel experiments."""
+    out = Path(out) if out else LIB_PATH
+    build_dir = PKG_DIR / "build" / (out.stem if out != LIB_PATH else "main")
+    build_dir.mkdir(parents=True, exist_ok=True)
     srcs = sources()
     if not srcs:
         raise RuntimeError(f"no .hip sources under {CSRC}")
     objs = [build_dir / (s.stem + ".o") for s in srcs]
     jobs = jobs or min(len(srcs), int(os.environ.get("MAX_JOBS", "8")))
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        futs = [pool.submit(_compile, s, o, verbose) for s, o in zip(srcs, objs)]
+        futs = [pool.submit(_compile, s, o, verbose, tuple(extra)) for s, o in zip(srcs, objs)]
         for f in futs:
             f.result()
-    tmp = PKG_DIR / (LIB_NAME + ".tmp")
+    tmp = out.with_suffix(".so.tmp")
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    os.replace(tmp, out)
+    return out
 
 
 if __name__ == "__main__":
-    path = build(verbose=True)
+    import argparse
+
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--out", default=None, help="write the library here instead of in-tree")
+    ap.add_argument("extra", nargs="*", help="extra hipcc flags, e.g. -DNAME (after --)")
+    ns = ap.parse_args()
+    path = build(verbose=True, out=ns.out, extra=tuple(ns.extra))
     print(f"built {path}")

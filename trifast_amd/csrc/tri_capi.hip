@@ -266,9 +266,9 @@ int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype)
   int pick = 0;
   switch (kernel) {
     case TRIFAST_KERNEL_FWD:
-      if (n <= 64) pick = 2;
-      else if (n <= 256 || d >= 128 || dtype == TRIFAST_F32) pick = 0;
-      else pick = 1;
+      // more pair rows per workgroup = fewer bias reads; fall back when it does not fit
+      pick = n <= 64 ? 0 : 2;
+      while (pick > 0 && !trifast_supports(kernel, pick, n, h, d, dtype)) --pick;
       break;
     default: pick = 0; break;
   }

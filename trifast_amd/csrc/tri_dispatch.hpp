@@ -45,5 +45,22 @@ hipError_t dispatch(const Args& a, int bh, int d, int dtype, int tile, hipStream
 }
 
 constexpr int kMaxStaticLds = 64 * 1024;
+constexpr int kMaxLds = 160 * 1024;  // LDS per workgroup on gfx950
+
+// Launch with `lds` bytes of dynamic LDS; above the default 64 KiB limit the
+// kernel's attribute has to be raised first (once per instantiation).
+template <typename Kernel, typename Args>
+hipError_t launch_dyn(Kernel kernel, dim3 grid, dim3 block, int lds, hipStream_t st, const Args& a) {
+  if (lds > kMaxStaticLds) {
+    static thread_local const void* raised = nullptr;
+    if (raised != reinterpret_cast<const void*>(kernel)) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      if (e != hipSuccess) return e;
+      raised = reinterpret_cast<const void*>(kernel);
+    }
+  }
+  hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
+  return hipGetLastError();
+}
 
 }  // namespace tri

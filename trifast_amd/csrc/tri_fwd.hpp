@@ -1,14 +1,22 @@
-// Forward kernel: flash-style triangle attention for one pair row per workgroup.
+// Forward kernel: flash-style triangle attention.
 //
-// Work unit: (batch*head, row i, block of NW*QT*32 queries j).  K[i] and V[i] are
-// streamed through LDS in tiles of BK keys (natural row-major layout); each wave
-// keeps QT tiles of 32 queries in registers.  Scores are computed TRANSPOSED,
-// S^T = K Q^T, so that a lane owns one query (column) and 16 keys of every 32-key
-// tile: the softmax running max / sum are per-lane scalars, and the
-// probabilities are already in B-operand layout for O^T += V^T P^T, whose A
-// operand V^T comes from the natural V tile through transposing LDS reads.
+// Work unit: (batch*head, R consecutive pair rows i, block of NW*32 queries j).
+// Wave w owns one tile of 32 queries for all R rows.  The three operands of the
+// iteration space (i, j, k) live in three places:
+//   * bias[j, k] does not depend on the row: one packed bias tile (registers) is
+//     reused by the R rows, which divides its L2 traffic by R;
+//   * K[i], V[i] do not depend on the query: they are streamed through LDS in
+//     tiles of BK keys (natural row-major layout, double-buffered) and shared by
+//     the NW waves;
+//   * Q[i, j] and the output accumulator stay in registers for the whole sweep.
+// Scores are computed TRANSPOSED, S^T = K Q^T, so that a lane owns one query
+// (column) and 16 keys of every 32-key tile: the softmax running reference / sum
+// are per-lane scalars, and the probabilities are already in B-operand layout
+// for O^T += V^T P^T, whose A operand V^T comes from the natural V tile through
+// transposing LDS reads.
 //
-// Raw-score domain: acc = bias * sqrt(d) + q.k  (bias is the accumulator init);
+// Raw-score domain: acc = sqrt(d) * bias + q.k (the converted bias tile is the
+// accumulator init of the score MFMA and is shared by the R rows);
 // p = exp2(acc * c - ref * c) with c = log2(e) / sqrt(d).  `ref` is the running
 // reference of the online softmax: it is raised to the running maximum only when
 // some query of the wave exceeds it by more than kLazy (in log2 units), so the
@@ -24,7 +32,7 @@ namespace tri {
 
 constexpr float kLazy = 8.0f;
 
-template <typename T, int D, int NW, int QT, int BK>
+template <typename T, int D, int NW, int R, int BK>
 __global__ __launch_bounds__(NW * 64) void tri_fwd_kernel(const FwdArgs a) {
   using E = Elem<T>;
   using frag = typename E::frag;
@@ -37,148 +45,268 @@ __global__ __launch_bounds__(NW * 64) void tri_fwd_kernel(const FwdArgs a) {
   constexpr int LD = D + PAD;
   constexpr int NT = NW * 64;
 
-  __shared__ __attribute__((aligned(16))) T Ks[BK][LD];
-  __shared__ __attribute__((aligned(16))) T Vs[BK][LD];
+  // [buffer][K rows of row 0..R-1, then V rows of row 0..R-1]; dynamic so that
+  // the larger instantiations may use more than the 64 KiB static limit
+  extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
+  T(*KVs)[2 * R * BK][LD] = reinterpret_cast<T(*)[2 * R * BK][LD]>(tri_smem);
+  // keep words of the R rows, copied to LDS once: reading them there keeps the
+  // global-load counter of the main loop free for the prefetched tiles
+  uint32_t* keep_s = reinterpret_cast<uint32_t*>(tri_smem + 2 * sizeof(T) * (2 * R * BK) * LD);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int jl = lane & 31, g = lane >> 5;
   const int N = a.N;
-  int bx, i;
-  xcd_remap(gridDim.x, bx, i);
-  if (i >= N) return;
+  int bx, by;
+  xcd_remap(gridDim.x, bx, by);
+  const int i0 = by * R;
+  if (i0 >= N) return;
   const int bh = blockIdx.z;
   const int b = bh / a.H, h = bh % a.H;
-  const int j_wave = bx * (NW * QT * 32) + wave * (QT * 32);
+  const int j_wave = bx * (NW * 32) + wave * 32;
+  const int j = j_wave + jl;
   const bool wave_active = j_wave < N;
+  const int jt = j_wave >> 5;
 
-  const bool flagged = a.rowflag[(int64_t)b * N + i] != 0;
-  const uint32_t* keep_row = a.keep + ((int64_t)b * N + i) * a.nwords;
-
-  const T* qrow = reinterpret_cast<const T*>(a.q) + b * a.sq.b + h * a.sq.h + i * a.sq.i;
-  const T* krow = reinterpret_cast<const T*>(a.k) + b * a.sk.b + h * a.sk.h + i * a.sk.i;
-  const T* vrow = reinterpret_cast<const T*>(a.v) + b * a.sv.b + h * a.sv.h + i * a.sv.i;
+  const T* qbh = reinterpret_cast<const T*>(a.q) + b * a.sq.b + h * a.sq.h;
+  const T* kbh = reinterpret_cast<const T*>(a.k) + b * a.sk.b + h * a.sk.h;
+  const T* vbh = reinterpret_cast<const T*>(a.v) + b * a.sv.b + h * a.sv.h;
   const T* pack_bh = reinterpret_cast<const T*>(a.packq) + (int64_t)bh * a.NP * a.NP * 1024;
 
-  // Q tiles as B operands: lane owns query j, slots 2*KP*s + KP*g .. +KP-1 of d.
-  // A fully masked row drops the q.k and bias terms (all logits equal).
-  frag qf[QT][DS];
+  // per-row state.  A fully masked row drops the q.k and bias terms (all logits
+  // equal): its Q operand is zero and it skips the bias.
+  bool flagged[R];
+  frag qf[R][DS];
+  f32x16 oacc[R][DM];
+  float mref[R], mc[R], lrun[R];
 #pragma unroll
-  for (int t = 0; t < QT; ++t) {
-    const int j = j_wave + 32 * t + jl;
+  for (int r = 0; r < R; ++r) {
+    const int i = min(i0 + r, N - 1);  // rows past the end repeat the last one and are not stored
+    flagged[r] = a.rowflag[(int64_t)b * N + i] != 0;
+    for (int w = tid; w < a.nwords; w += NT) keep_s[r * a.nwords + w] = a.keep[((int64_t)b * N + i) * a.nwords + w];
 #pragma unroll
     for (int s = 0; s < DS; ++s) {
-      if (j < N && !flagged)
-        qf[t][s] = *reinterpret_cast<const frag*>(qrow + (int64_t)j * a.sq.j + 2 * KP * s + KP * g);
+      if (j < N && !flagged[r])
+        qf[r][s] = *reinterpret_cast<const frag*>(qbh + i * a.sq.i + (int64_t)j * a.sq.j + 2 * KP * s + KP * g);
       else
-        qf[t][s] = E::zero();
+        qf[r][s] = E::zero();
     }
-  }
-
-  f32x16 oacc[QT][DM];
-  float mref[QT], mc[QT], lrun[QT];
+    mref[r] = kNeg;
+    mc[r] = kNeg;
+    lrun[r] = 0.f;
 #pragma unroll
-  for (int t = 0; t < QT; ++t) {
-    mref[t] = kNeg;
-    mc[t] = kNeg;
-    lrun[t] = 0.f;
-#pragma unroll
-    for (int mt = 0; mt < DM; ++mt) oacc[t][mt] = zero16();
+    for (int mt = 0; mt < DM; ++mt) oacc[r][mt] = zero16();
   }
 
   const float c = a.c;
-  const float lazy_raw = kLazy / c;
-  for (int kt0 = 0; kt0 < N; kt0 += BK) {
-    uint32_t keepw[KU];
+
+  // keep words of the BK keys starting at kt0 for every row; false when no row
+  // attends to any of them (such stages are skipped: their probabilities are zero)
+  auto stage_keep = [&](int kt0, uint32_t (*keepw)[KU]) -> bool {
     uint32_t any = 0;
 #pragma unroll
-    for (int u = 0; u < KU; ++u) {
-      const int w = kt0 / 32 + u;
-      keepw[u] = (w < a.nwords) ? keep_row[w] : 0u;
-      any |= keepw[u];
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int u = 0; u < KU; ++u) {
+        const int w = kt0 / 32 + u;
+        keepw[r][u] = (w < a.nwords) ? keep_s[r * a.nwords + w] : 0u;
+        any |= keepw[r][u];
+      }
+    return any != 0;
+  };
+  auto next_live = [&](int kt0, uint32_t (*keepw)[KU]) -> int {
+    while (kt0 < N && !stage_keep(kt0, keepw)) kt0 += BK;
+    return kt0;
+  };
+
+  // global -> register -> LDS staging of the K and V tiles of all R rows
+  constexpr int CPR = D / E::VEC;
+  constexpr int CHUNKS = 2 * R * BK * CPR;
+  constexpr int CNT = (CHUNKS + NT - 1) / NT;
+  typename E::vec stage[CNT];
+
+  // Loads are issued unconditionally (indices clamped into range instead of
+  // branching) so that the number of loads in flight is the same on every path
+  // and the waits on them can be exact.  A clamped key row duplicates the last
+  // valid one; its keep bit is clear, so it contributes exactly zero.
+  const int jt_ld = min(jt, a.NP - 1);
+  auto issue_loads = [&](int kt0, BiasRegs<T>* bias) {
+#pragma unroll
+    for (int x = 0; x < CNT; ++x) {
+      const int ch = (CHUNKS % NT == 0) ? x * NT + tid : min(x * NT + tid, CHUNKS - 1);
+      const int arr = ch / (BK * CPR);  // 0..R-1: K of row arr; R..2R-1: V of row arr-R
+      const int rem = ch % (BK * CPR);
+      const int row = min(kt0 + rem / CPR, N - 1), col = (rem % CPR) * E::VEC;
+      const int i = min(i0 + arr % R, N - 1);
+      const T* src = (arr >= R) ? vbh + i * a.sv.i + (int64_t)row * a.sv.j
+                                : kbh + i * a.sk.i + (int64_t)row * a.sk.j;
+      stage[x] = *reinterpret_cast<const typename E::vec*>(src + col);
     }
-    if (any == 0) continue;  // every key of this tile is masked or out of range
+#pragma unroll
+    for (int u = 0; u < KU; ++u) bias[u].load(pack_bh, a.NP, jt_ld, min((kt0 >> 5) + u, a.NP - 1), lane);
+  };
+  auto store_stage = [&](int buf) {
+#pragma unroll
+    for (int x = 0; x < CNT; ++x) {
+      const int ch = x * NT + tid;
+      const int arr = ch / (BK * CPR);
+      const int rem = ch % (BK * CPR);
+      const int row = rem / CPR, col = (rem % CPR) * E::VEC;
+      if (CHUNKS % NT == 0 || ch < CHUNKS) *reinterpret_cast<typename E::vec*>(&KVs[buf][arr * BK + row][col]) = stage[x];
+    }
+  };
 
-    __syncthreads();
-    lds_load_natural<T, D, BK, LD, NT>(Ks, krow + (int64_t)kt0 * a.sk.j, a.sk.j, N - kt0, tid);
-    lds_load_natural<T, D, BK, LD, NT>(Vs, vrow + (int64_t)kt0 * a.sv.j, a.sv.j, N - kt0, tid);
-    __syncthreads();
-    if (!wave_active) continue;
-
+  // one stage of compute from LDS buffer `buf`
+  auto compute_stage = [&](int buf, const uint32_t (*kw)[KU], const BiasRegs<T>* bias) {
+    if (wave_active) {
+      // The KU*R tiles of the stage run as a software pipeline inside the wave: the
+      // MFMA chain that produces the scores of tile t+1 is issued before the
+      // softmax arithmetic of tile t, so the matrix pipe works on t+1 while the
+      // vector ALU works on t (dependent MFMAs queue in the matrix pipe without
+      // holding up the wave's other instructions).  K operands are read from LDS
+      // two tiles ahead, V^T operands one softmax ahead of their use.
+      constexpr int TS = KU * R;
+      auto k_operand = [&](int t, frag* kf) {
+        const int u = t / R, r = t % R;
+        const T(*Kt)[LD] = &KVs[buf][r * BK];
 #pragma unroll
-    for (int u = 0; u < KU; ++u) {
-      if (keepw[u] == 0) continue;
-      // K tile rows as A operand; tile row m stands for key perm32(m)
-      frag kf[DS];
+        for (int sd = 0; sd < DS; ++sd)
+          kf[sd] = *reinterpret_cast<const frag*>(&Kt[32 * u + perm32(jl)][2 * KP * sd + KP * g]);
+      };
+      // The bias tile does not depend on the pair row: it is converted to fp32 in
+      // the raw-score domain once per stage and key tile, and then serves as the
+      // accumulator init (C operand) of the first score MFMA of each of the R rows.
+      f32x16 biasv[KU];
 #pragma unroll
-      for (int s = 0; s < DS; ++s)
-        kf[s] = *reinterpret_cast<const frag*>(&Ks[32 * u + perm32(jl)][2 * KP * s + KP * g]);
-      // V^T rows as A operand of the second product
-      frag vf[DM][PS];
-#pragma unroll
-      for (int mt = 0; mt < DM; ++mt)
-#pragma unroll
-        for (int s2 = 0; s2 < PS; ++s2) vf[mt][s2] = tr_operand<T, LD>(Vs, 32 * u, s2, 32 * mt, D, lane);
-
-      const uint32_t myw = keepw[u] >> (8 * g);
-      const bool mixed = keepw[u] != 0xffffffffu;
-
-#pragma unroll
-      for (int t = 0; t < QT; ++t) {
-        f32x16 s;
-        if (!flagged)
-          s = bias_tile<T>(pack_bh, a.NP, (j_wave >> 5) + t, (kt0 >> 5) + u, lane, a.sqrt_d, 0.f);
-        else
-          s = zero16();
-#pragma unroll
-        for (int sd = 0; sd < DS; ++sd) s = E::mfma(kf[sd], qf[t][sd], s);
+      for (int u = 0; u < KU; ++u) biasv[u] = bias_tile<T>(bias[u], a.sqrt_d, 0.f);
+      auto scores = [&](int t, const frag* kf) -> f32x16 {
+        const int u = t / R, r = t % R;
+        f32x16 sc;
+        const bool mixed = kw[r][u] != 0xffffffffu;
         if (mixed) {
+          sc = mask_tile(kw[r][u], g);
+          if (!flagged[r]) {
 #pragma unroll
-          for (int v = 0; v < 16; ++v)
-            s[v] = ((myw >> (16 * (v / 8) + (v % 8))) & 1u) ? s[v] : kNeg;
+            for (int v = 0; v < 16; ++v) sc[v] += biasv[u][v];
+          }
+          sc = E::mfma(kf[0], qf[r][0], sc);
+        } else if (flagged[r]) {
+          sc = E::mfma(kf[0], qf[r][0], zero16());
+        } else {
+          sc = E::mfma(kf[0], qf[r][0], biasv[u]);
         }
-        float mx = fmaxf(s[0], s[1]);
 #pragma unroll
-        for (int v = 2; v < 16; v += 2) mx = fmaxf(mx, fmaxf(s[v], s[v + 1]));
-        mx = half_max(mx);
-        if (__any(mx > mref[t] + lazy_raw)) {
-          const float mnew = fmaxf(mref[t], mx);
-          const float alpha = fast_exp2((mref[t] - mnew) * c);
-          lrun[t] *= alpha;
+        for (int sd = 1; sd < DS; ++sd) sc = E::mfma(kf[sd], qf[r][sd], sc);
+        return sc;
+      };
+
+      frag kf1[DS], kf2[DS];
+      k_operand(0, kf1);
+      if constexpr (TS > 1) k_operand(1, kf2);
+      f32x16 sc = scores(0, kf1);
+#pragma unroll
+      for (int t = 0; t < TS; ++t) {
+        const int u = t / R, r = t % R;
+        f32x16 sn;
+        if (t + 1 < TS) {
+#pragma unroll
+          for (int sd = 0; sd < DS; ++sd) kf1[sd] = kf2[sd];
+          if (t + 2 < TS) k_operand(t + 2, kf2);
+          sn = scores(t + 1, kf1);
+        }
+        if (kw[r][u] != 0) {  // a row that attends to no key of this tile adds nothing
+          // V^T rows as A operand of the second product
+          const T(*Vt)[LD] = &KVs[buf][(R + r) * BK];
+          frag vf[DM][PS];
 #pragma unroll
           for (int mt = 0; mt < DM; ++mt)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) oacc[t][mt][v] *= alpha;
-          mref[t] = mnew;
-          mc[t] = mnew * c;
+            for (int s2 = 0; s2 < PS; ++s2) vf[mt][s2] = tr_operand<T, LD>(Vt, 32 * u, s2, 32 * mt, D, lane);
+          // exponent arguments against the current reference; results of an fma are
+          // canonical floats, so the max below needs no extra canonicalisation
+          float arg[16];
+#pragma unroll
+          for (int v = 0; v < 16; ++v) arg[v] = __builtin_fmaf(sc[v], c, -mc[r]);
+          float amax = fmaxf(arg[0], arg[1]);
+#pragma unroll
+          for (int v = 2; v < 16; v += 2) amax = fmaxf(amax, fmaxf(arg[v], arg[v + 1]));
+          amax = half_max(amax);
+          if (__any(amax > kLazy)) {
+            // some query outgrew the reference: raise it to the running maximum
+            float mx = fmaxf(sc[0], sc[1]);
+#pragma unroll
+            for (int v = 2; v < 16; ++v) mx = fmaxf(mx, sc[v]);
+            mx = half_max(mx);
+            const float mnew = fmaxf(mref[r], mx);
+            const float alpha = fast_exp2((mref[r] - mnew) * c);
+            lrun[r] *= alpha;
+#pragma unroll
+            for (int mt = 0; mt < DM; ++mt)
+#pragma unroll
+              for (int v = 0; v < 16; ++v) oacc[r][mt][v] *= alpha;
+            mref[r] = mnew;
+            mc[r] = mnew * c;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) arg[v] = __builtin_fmaf(sc[v], c, -mc[r]);
+          }
+          float p[16];
+#pragma unroll
+          for (int v = 0; v < 16; ++v) p[v] = fast_exp2(arg[v]);
+#pragma unroll
+          for (int s2 = 0; s2 < PS; ++s2) {
+            const frag pf = E::pack(&p[KP * s2]);
+            lrun[r] = frag_sum(pf, lrun[r]);
+#pragma unroll
+            for (int mt = 0; mt < DM; ++mt) oacc[r][mt] = E::mfma(vf[mt][s2], pf, oacc[r][mt]);
+          }
         }
-        float p[16];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) p[v] = fast_exp2(__builtin_fmaf(s[v], c, -mc[t]));
-#pragma unroll
-        for (int s2 = 0; s2 < PS; ++s2) {
-          const frag pf = E::pack(&p[KP * s2]);
-          lrun[t] = frag_sum(pf, lrun[t]);
-#pragma unroll
-          for (int mt = 0; mt < DM; ++mt) oacc[t][mt] = E::mfma(vf[mt][s2], pf, oacc[t][mt]);
-        }
+        if (t + 1 < TS) sc = sn;
       }
     }
+
+  };
+
+  // The stage loop is unrolled by two so that the two sets of bias registers and
+  // keep words swap roles without being copied.
+  BiasRegs<T> bias0[KU], bias1[KU];
+  uint32_t keep0[R][KU], keep1[R][KU];
+  __syncthreads();  // keep words visible
+  int kt0 = next_live(0, keep0);
+  issue_loads(min(kt0, N - 1), bias0);
+  store_stage(0);
+  // everything loaded so far (Q operands, first stage) has landed before the loop,
+  // so waits inside it only ever concern the loads issued inside it
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  while (kt0 < N) {
+    // past the last live stage the prefetch re-reads a valid stage that nobody uses
+    int kt1 = next_live(kt0 + BK, keep1);
+    issue_loads(min(kt1, N - 1), bias1);
+    compute_stage(0, keep0, bias0);
+    store_stage(1);
+    __syncthreads();
+    if (kt1 >= N) break;
+    kt0 = kt1;
+    kt1 = next_live(kt0 + BK, keep0);
+    issue_loads(min(kt1, N - 1), bias0);
+    compute_stage(1, keep1, bias1);
+    store_stage(0);
+    __syncthreads();
+    kt0 = kt1;
   }
 
   if (!wave_active) return;
-  T* orow = reinterpret_cast<T*>(a.o) + (((int64_t)bh * N + i) * N) * D;
-  float* lrow = a.lse + ((int64_t)bh * N + i) * N;
 #pragma unroll
-  for (int t = 0; t < QT; ++t) {
-    const int j = j_wave + 32 * t + jl;
-    const float ltot = half_sum(lrun[t]);
-    if (j >= N) continue;
-    store_rows<T, D, DM>(orow + (int64_t)j * D, oacc[t], 1.0f / ltot, g);
+  for (int r = 0; r < R; ++r) {
+    const int i = i0 + r;
+    const float ltot = half_sum(lrun[r]);
+    if (i >= N || j >= N) continue;
+    T* orow = reinterpret_cast<T*>(a.o) + (((int64_t)bh * N + i) * N) * D;
+    store_rows<T, D, DM>(orow + (int64_t)j * D, oacc[r], 1.0f / ltot, g);
     if (g == 0) {
-      float lse = kLn2 * (mc[t] + fast_log2(ltot));
-      if (flagged) lse = a.neg_inf + lse;
-      lrow[j] = lse;
+      float lse = kLn2 * (mc[r] + fast_log2(ltot));
+      if (flagged[r]) lse = a.neg_inf + lse;
+      a.lse[((int64_t)bh * N + i) * N + j] = lse;
     }
   }
 }

@@ -40,6 +40,63 @@ TRI_DEV void lds_load_natural(T (*dst)[LD], const T* src, int64_t stride, int nr
   }
 }
 
+// Two-phase version of the same copy, for software pipelining: the global loads
+// of the next tile are issued into registers before the current tile is computed
+// and written to LDS afterwards.
+template <typename T, int D, int ROWS, int NT>
+struct TileRegs {
+  using vec = typename Elem<T>::vec;
+  static constexpr int VEC = Elem<T>::VEC;
+  static constexpr int CPR = D / VEC;
+  static constexpr int CNT = (ROWS * CPR + NT - 1) / NT;
+  vec v[CNT];
+  TRI_DEV void load(const T* src, int64_t stride, int nrows, int tid) {
+#pragma unroll
+    for (int x = 0; x < CNT; ++x) {
+      const int c = x * NT + tid;
+      const int row = c / CPR, col = (c % CPR) * VEC;
+      if (c < ROWS * CPR && row < nrows) {
+        v[x] = *reinterpret_cast<const vec*>(src + (int64_t)row * stride + col);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[x][e] = (T)0.f;
+      }
+    }
+  }
+  template <int LD>
+  TRI_DEV void store(T (*dst)[LD], int tid) const {
+#pragma unroll
+    for (int x = 0; x < CNT; ++x) {
+      const int c = x * NT + tid;
+      const int row = c / CPR, col = (c % CPR) * VEC;
+      if (c < ROWS * CPR) *reinterpret_cast<vec*>(&dst[row][col]) = v[x];
+    }
+  }
+};
+
+// The packed bias operand of tile (jt, kt) for one lane: 2 x 8 elements.
+template <typename T>
+struct BiasRegs {
+  typename Elem<T>::vec v[2 * (sizeof(T) == 2 ? 1 : 2)];
+  TRI_DEV void load(const T* pack_bh, int NP, int jt, int kt, int lane_q) {
+    const T* p = pack_bh + ((((int64_t)jt * NP + kt) * 2) * 64 + lane_q) * 8;
+    if constexpr (sizeof(T) == 2) {
+      v[0] = *reinterpret_cast<const typename Elem<T>::vec*>(p);
+      v[1] = *reinterpret_cast<const typename Elem<T>::vec*>(p + 512);
+    } else {
+      v[0] = *reinterpret_cast<const f32x4*>(p);
+      v[1] = *reinterpret_cast<const f32x4*>(p + 4);
+      v[2] = *reinterpret_cast<const f32x4*>(p + 512);
+      v[3] = *reinterpret_cast<const f32x4*>(p + 516);
+    }
+  }
+  // element x (0..15) as float
+  TRI_DEV float at(int x) const {
+    if constexpr (sizeof(T) == 2) return (float)v[x / 8][x % 8];
+    else return v[x / 4][x % 4];
+  }
+};
+
 // The 16 bias values of one lane for tile (jt, kt), in the raw-score domain
 // (times sqrt(d)) plus a per-lane additive term, from a packed bias array.
 template <typename T>
@@ -63,6 +120,120 @@ TRI_DEV f32x16 bias_tile(const T* pack_bh, int NP, int jt, int kt, int lane, flo
     }
   }
   return s;
+}
+
+// The bias enters the raw scores through the matrix pipe rather than the vector
+// ALU: S^T[key, j] += sum_k' (sqrt(d) * I)[key, k'] * bias^T[k', j].  The packed
+// bias tile is the B operand as stored (no conversion); the A operand is the
+// scaled identity, whose row m stands for key perm32(m).  sqrt(d) is split into
+// hi + lo parts of the operand type so the product is exact to ~2^-17 (for d a
+// power of 4 the lo part is zero and is skipped).  fp32 needs no split.
+template <typename T>
+struct BiasIdentity {
+  using frag = typename Elem<T>::frag;
+  static constexpr int KP = Elem<T>::KP;
+  static constexpr int PS = 32 / (2 * KP);
+  frag hi[PS], lo[PS];
+  bool has_lo;
+  TRI_DEV void init(float sqrt_d, int lane) {
+    const int m = perm32(lane & 31), g = lane >> 5;
+    const T h = (T)sqrt_d;
+    const T l = (T)(sqrt_d - (float)h);
+    has_lo = (float)l != 0.f;
+#pragma unroll
+    for (int s = 0; s < PS; ++s) {
+      if constexpr (KP == 1) {
+        hi[s] = (cidx(s, g) == m) ? sqrt_d : 0.f;
+        lo[s] = 0.f;
+      } else {
+#pragma unroll
+        for (int e = 0; e < KP; ++e) {
+          const bool on = cidx(KP * s + e, g) == m;
+          hi[s][e] = on ? h : (T)0.f;
+          lo[s][e] = on ? l : (T)0.f;
+        }
+      }
+    }
+  }
+};
+
+// Adds sqrt(d) * bias tile (jt, kt) to the raw-score accumulator.  `lane_q` is
+// the lane whose packed slot this lane reads: its own in the transposed-score
+// kernels (the bias is the B operand), the row-permuted one in the dk/dv kernel
+// (the bias is the A operand and the identity the B operand).
+template <typename T, bool BIAS_IS_B>
+TRI_DEV f32x16 add_bias_mfma(f32x16 acc, const BiasIdentity<T>& id, const T* pack_bh, int NP, int jt, int kt, int lane_q) {
+  using E = Elem<T>;
+  using frag = typename E::frag;
+  constexpr int KP = E::KP;
+  constexpr int PS = 32 / (2 * KP);
+  const T* p = pack_bh + ((((int64_t)jt * NP + kt) * 2) * 64 + lane_q) * 8;
+  frag bf[PS];
+  if constexpr (KP == 1) {
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const f32x4 x0 = *reinterpret_cast<const f32x4*>(p + r * 512);
+      const f32x4 x1 = *reinterpret_cast<const f32x4*>(p + r * 512 + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { bf[8 * r + e] = x0[e]; bf[8 * r + 4 + e] = x1[e]; }
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < 2; ++r) bf[r] = *reinterpret_cast<const frag*>(p + r * 512);
+  }
+#pragma unroll
+  for (int s = 0; s < PS; ++s) {
+    if constexpr (BIAS_IS_B) acc = E::mfma(id.hi[s], bf[s], acc);
+    else acc = E::mfma(bf[s], id.hi[s], acc);
+  }
+  if constexpr (KP > 1) {
+    if (id.has_lo) {
+#pragma unroll
+      for (int s = 0; s < PS; ++s) {
+        if constexpr (BIAS_IS_B) acc = E::mfma(id.lo[s], bf[s], acc);
+        else acc = E::mfma(bf[s], id.lo[s], acc);
+      }
+    }
+  }
+  return acc;
+}
+
+// Same, from bias operands already in registers.
+template <typename T, bool BIAS_IS_B>
+TRI_DEV f32x16 add_bias_mfma(f32x16 acc, const BiasIdentity<T>& id, const BiasRegs<T>& b) {
+  using E = Elem<T>;
+  static_assert(E::KP > 1, "the fp32 path adds the bias on the vector ALU");
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    if constexpr (BIAS_IS_B) acc = E::mfma(id.hi[s], b.v[s], acc);
+    else acc = E::mfma(b.v[s], id.hi[s], acc);
+  }
+  if (id.has_lo) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      if constexpr (BIAS_IS_B) acc = E::mfma(id.lo[s], b.v[s], acc);
+      else acc = E::mfma(b.v[s], id.lo[s], acc);
+    }
+  }
+  return acc;
+}
+
+template <typename T>
+TRI_DEV f32x16 bias_tile(const BiasRegs<T>& b, float sqrt_d, float add) {
+  f32x16 s;
+#pragma unroll
+  for (int x = 0; x < 16; ++x) s[x] = __builtin_fmaf(b.at(x), sqrt_d, add);
+  return s;
+}
+
+// Additive key mask of one 32-key tile in the transposed-score layout: value v
+// of lane group g is 0 when key cidx(v, g) is attended to and kNeg otherwise.
+TRI_DEV f32x16 mask_tile(uint32_t keepw, int g) {
+  const uint32_t myw = keepw >> (8 * g);
+  f32x16 m;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) m[v] = ((myw >> (16 * (v / 8) + (v % 8))) & 1u) ? 0.f : kNeg;
+  return m;
 }
 
 // Operand whose contraction index is in-lane, from a natural LDS tile
