@@ -50,9 +50,12 @@ struct BwdArgs {
   const uint32_t* keep;
   const uint8_t* rowflag;
   float* delta;              // [b*h, n, n] fp32 workspace, indexed [i, j]
+  float* dbpart;             // [nchunks, b*h, n, n] fp32 partial db (nchunks > 1 only)
   void *dq, *dk, *dv, *db;
   Str5 sq, sk, sv, sdo;
   int H, N, NP, nwords;
+  int BH;                    // b * h
+  int nchunks, rows_per_chunk;  // db kernel: split of the pair rows over workgroups
   float c;                   // log2(e) / sqrt(d)
   float sqrt_d;
   float scale;               // 1 / sqrt(d)

@@ -1,12 +1,17 @@
 // Backward kernel 3 of 3: db[j, k] = sum over rows i of dS[i, j, k].
 //
-// Work unit: (batch*head, block of queries j, block of keys k); the kernel walks
-// all n pair rows i and keeps the db tile in fp32 registers the whole time, so
-// the reduction over i has one fixed order and needs no atomics.  Per row a wave
-// recomputes, for its WJ x WK tiles of 32x32,
+// Work unit: (batch*head, block of 2*WJ*32 queries j, block of 2*WK*32 keys k,
+// chunk of pair rows i).  The 2 x 2 waves of a workgroup each own WJ x WK tiles of
+// 32 x 32 and keep their db tiles in fp32 registers while the workgroup walks its
+// rows, so the reduction over i has one fixed order and needs no atomics.  The
+// bias tiles (register-resident, fp32, raw-score domain) are the accumulator init
+// of the score MFMA of every row.  Per row the workgroup stages the Q, dO rows of
+// its queries and the K, V rows of its keys in LDS (direct global->LDS loads,
+// double-buffered, swizzled), and each wave recomputes for its tiles
 //   S^T = K Q^T (+bias), P^T = exp2(S^T c - lse), dP^T = V dO^T, dS^T = P^T (dP^T - delta)
-// with every operand in its natural row-major layout (rows of Q, dO, K, V are
-// read straight from global memory as MFMA operands), and adds dS^T into db.
+// with every operand in its natural row-major layout, adding dS^T into db.
+// When the rows are split into several chunks (to fill the GPU at small n), each
+// chunk writes an fp32 partial and a second kernel adds the partials in order.
 //
 // Replaces _bwd_b of reference src/trifast/triton.py:394-501.
 #pragma once
@@ -17,33 +22,38 @@
 namespace tri {
 
 template <typename T, int D, int WJ, int WK>
-struct BRowFrags {
-  using frag = typename Elem<T>::frag;
-  static constexpr int DS = D / (2 * Elem<T>::KP);
-  frag q[WJ][DS], dout[WJ][DS], k[WK][DS], v[WK][DS];
-  float lse2[WJ], delta[WJ];
-  uint32_t keepw[WK];
-  bool flagged;
-};
-
-template <typename T, int D, int WJ, int WK, bool PREFETCH>
 __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
   using E = Elem<T>;
   using frag = typename E::frag;
+  using Tile = LdsTile<T, D>;
   constexpr int KP = E::KP;
   constexpr int DS = D / (2 * KP);
-  using Row = BRowFrags<T, D, WJ, WK>;
+  constexpr int NW = 4;
+  constexpr int BJ = 2 * WJ * 32, BKB = 2 * WK * 32;  // queries / keys per workgroup
+  constexpr int ROWB = Tile::ROWB;
+  // one stage: Q rows | dO rows | K rows | V rows | lse[BJ] | delta[BJ]
+  constexpr int OFF_Q = 0, OFF_DO = BJ * ROWB, OFF_K = 2 * BJ * ROWB, OFF_V = OFF_K + BKB * ROWB;
+  constexpr int OFF_LSE = OFF_V + BKB * ROWB, OFF_DELTA = OFF_LSE + BJ * 4;
+  constexpr int STAGE = OFF_DELTA + BJ * 4;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
+  // after the two stages: keep words [rows][WKW] and row flags [rows] of this chunk
+  constexpr int WKW = BKB / 32;
+  uint32_t* keep_s = reinterpret_cast<uint32_t*>(tri_smem + 2 * STAGE);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int jl = lane & 31, g = lane >> 5;
-  const int bh = blockIdx.z;
-  const int b = bh / a.H, h = bh % a.H;
   const int N = a.N;
-  // 2 x 2 waves per workgroup; they share nothing but the launch
-  const int j_wave = (blockIdx.x * 2 + (wave & 1)) * (WJ * 32);
-  const int k_wave = (blockIdx.y * 2 + (wave >> 1)) * (WK * 32);
-  if (j_wave >= N || k_wave >= N) return;
+  const int bh = blockIdx.z % a.BH, chunk = blockIdx.z / a.BH;
+  const int b = bh / a.H, h = bh % a.H;
+  const int j_blk = blockIdx.x * BJ, k_blk = blockIdx.y * BKB;
+  const int wj = wave & 1, wk = wave >> 1;
+  const int j_wave = j_blk + wj * (WJ * 32), k_wave = k_blk + wk * (WK * 32);
+  const int i_begin = chunk * a.rows_per_chunk;
+  const int i_end = min(N, i_begin + a.rows_per_chunk);
+  const int nrows = i_end - i_begin;
+  uint32_t* flag_s = keep_s + a.rows_per_chunk * WKW;
 
   const T* qbase = reinterpret_cast<const T*>(a.q) + b * a.sq.b + h * a.sq.h;
   const T* kbase = reinterpret_cast<const T*>(a.k) + b * a.sk.b + h * a.sk.h;
@@ -52,17 +62,21 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
   const T* pack_bh = reinterpret_cast<const T*>(a.packq) + (int64_t)bh * a.NP * a.NP * 1024;
   const float* lse_bh = a.lse + (int64_t)bh * N * N;
   const float* delta_bh = a.delta + (int64_t)bh * N * N;
-  const uint32_t* keep_b = a.keep + (int64_t)b * N * a.nwords;
-  const uint8_t* flag_b = a.rowflag + (int64_t)b * N;
-  const float lse2_flagged = fast_log2((float)N);
 
-  // bias tile in the raw-score domain, used as the accumulator init of every row
+  // keep words and row flags of the chunk's rows, once
+  for (int x = tid; x < nrows * WKW; x += 256) {
+    const int i = i_begin + x / WKW, w = k_blk / 32 + x % WKW;
+    keep_s[x] = (w < a.nwords) ? a.keep[((int64_t)b * N + i) * a.nwords + w] : 0u;
+  }
+  for (int x = tid; x < nrows; x += 256) flag_s[x] = a.rowflag[(int64_t)b * N + i_begin + x];
+
+  // bias tiles in the raw-score domain: accumulator init of every row's score MFMA
   f32x16 biasr[WJ][WK];
 #pragma unroll
   for (int tj = 0; tj < WJ; ++tj)
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk)
-      biasr[tj][tk] = bias_tile<T>(pack_bh, a.NP, (j_wave >> 5) + tj, (k_wave >> 5) + tk, lane, a.sqrt_d, 0.f);
+      biasr[tj][tk] = bias_tile<T>(pack_bh, a.NP, min((j_wave >> 5) + tj, a.NP - 1), min((k_wave >> 5) + tk, a.NP - 1), lane, a.sqrt_d, 0.f);
 
   f32x16 dbacc[WJ][WK];
 #pragma unroll
@@ -70,93 +84,104 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk) dbacc[tj][tk] = zero16();
 
-  auto load_row = [&](Row& r, int i) {
-    r.flagged = flag_b[i] != 0;
-#pragma unroll
-    for (int tk = 0; tk < WK; ++tk) {
-      const int w = k_wave / 32 + tk;
-      r.keepw[tk] = (w < a.nwords) ? keep_b[(int64_t)i * a.nwords + w] : 0u;
-      const int key = k_wave + 32 * tk + perm32(jl);  // tile row m stands for key perm32(m)
-#pragma unroll
-      for (int s = 0; s < DS; ++s) {
-        const int dofs = 2 * KP * s + KP * g;
-        if (key < N) {
-          r.k[tk][s] = *reinterpret_cast<const frag*>(kbase + i * a.sk.i + (int64_t)key * a.sk.j + dofs);
-          r.v[tk][s] = *reinterpret_cast<const frag*>(vbase + i * a.sv.i + (int64_t)key * a.sv.j + dofs);
-        } else {
-          r.k[tk][s] = E::zero();
-          r.v[tk][s] = E::zero();
-        }
-      }
-    }
-#pragma unroll
-    for (int tj = 0; tj < WJ; ++tj) {
-      const int j = j_wave + 32 * tj + jl;
-#pragma unroll
-      for (int s = 0; s < DS; ++s) {
-        const int dofs = 2 * KP * s + KP * g;
-        if (j < N) {
-          r.q[tj][s] = *reinterpret_cast<const frag*>(qbase + i * a.sq.i + (int64_t)j * a.sq.j + dofs);
-          r.dout[tj][s] = *reinterpret_cast<const frag*>(dobase + i * a.sdo.i + (int64_t)j * a.sdo.j + dofs);
-        } else {
-          r.q[tj][s] = E::zero();
-          r.dout[tj][s] = E::zero();
-        }
-      }
-      if (j < N) {
-        r.lse2[tj] = r.flagged ? lse2_flagged : lse_bh[(int64_t)i * N + j] * kLog2e;
-        r.delta[tj] = delta_bh[(int64_t)i * N + j];
-      } else {
-        r.lse2[tj] = 0.f;
-        r.delta[tj] = 0.f;
-      }
-    }
+  // issue the loads of row i into stage buffer `buf` (indices clamped, never branched)
+  auto issue_row = [&](int i, int buf) {
+    unsigned char* st = tri_smem + buf * STAGE;
+    i = min(i, N - 1);
+    Tile::template fill<BJ, NW>(st + OFF_Q, [&](int r) { return qbase + i * a.sq.i + (int64_t)min(j_blk + r, N - 1) * a.sq.j; }, wave, lane);
+    Tile::template fill<BJ, NW>(st + OFF_DO, [&](int r) { return dobase + i * a.sdo.i + (int64_t)min(j_blk + r, N - 1) * a.sdo.j; }, wave, lane);
+    Tile::template fill<BKB, NW>(st + OFF_K, [&](int r) { return kbase + i * a.sk.i + (int64_t)min(k_blk + r, N - 1) * a.sk.j; }, wave, lane);
+    Tile::template fill<BKB, NW>(st + OFF_V, [&](int r) { return vbase + i * a.sv.i + (int64_t)min(k_blk + r, N - 1) * a.sv.j; }, wave, lane);
+    fill_floats<BJ, NW>(reinterpret_cast<float*>(st + OFF_LSE), [&](int x) { return lse_bh + (int64_t)i * N + min(j_blk + x, N - 1); }, wave, lane);
+    fill_floats<BJ, NW>(reinterpret_cast<float*>(st + OFF_DELTA), [&](int x) { return delta_bh + (int64_t)i * N + min(j_blk + x, N - 1); }, wave, lane);
   };
 
   const float c = a.c;
-  auto compute_row = [&](const Row& r) {
+  const float lse2_flagged = fast_log2((float)N);
+  const bool wave_live = j_wave < N && k_wave < N;
+
+  auto compute_row = [&](int ir, int buf) {
+    const unsigned char* st = tri_smem + buf * STAGE;
+    const bool flagged = flag_s[ir] != 0;
+    // operands of this wave's tiles; tile row m of the key tiles stands for key perm32(m)
+    frag qf[WJ][DS], dof[WJ][DS], kf[WK][DS], vf[WK][DS];
+    float lse2[WJ], delta[WJ];
+#pragma unroll
+    for (int tj = 0; tj < WJ; ++tj) {
+      const int r = wj * (WJ * 32) + 32 * tj + jl;
+#pragma unroll
+      for (int s = 0; s < DS; ++s) {
+        // a fully masked row ignores q.k as well as the bias
+        qf[tj][s] = flagged ? E::zero() : Tile::operand(st + OFF_Q, r, s, g);
+        dof[tj][s] = Tile::operand(st + OFF_DO, r, s, g);
+      }
+      lse2[tj] = flagged ? lse2_flagged : reinterpret_cast<const float*>(st + OFF_LSE)[r] * kLog2e;
+      delta[tj] = reinterpret_cast<const float*>(st + OFF_DELTA)[r];
+    }
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk) {
-      if (r.keepw[tk] == 0) continue;
-      const uint32_t myw = r.keepw[tk] >> (8 * g);
-      const bool mixed = r.keepw[tk] != 0xffffffffu;
+      const int r = wk * (WK * 32) + 32 * tk + perm32(jl);
+#pragma unroll
+      for (int s = 0; s < DS; ++s) {
+        kf[tk][s] = Tile::operand(st + OFF_K, r, s, g);
+        vf[tk][s] = Tile::operand(st + OFF_V, r, s, g);
+      }
+    }
+#pragma unroll
+    for (int tk = 0; tk < WK; ++tk) {
+      const uint32_t keepw = keep_s[ir * WKW + wk * WK + tk];
+      if (keepw == 0) continue;  // no attended key in this tile: dS = 0
+      const bool mixed = keepw != 0xffffffffu;
 #pragma unroll
       for (int tj = 0; tj < WJ; ++tj) {
-        f32x16 s = r.flagged ? zero16() : biasr[tj][tk];
-        f32x16 dp = zero16();
+        f32x16 s;
+        if (mixed) {
+          s = mask_tile(keepw, g);
+          if (!flagged) {
 #pragma unroll
-        for (int sd = 0; sd < DS; ++sd) {
-          // a fully masked row ignores q.k as well as the bias
-          s = E::mfma(r.k[tk][sd], r.flagged ? E::zero() : r.q[tj][sd], s);
-          dp = E::mfma(r.v[tk][sd], r.dout[tj][sd], dp);
+            for (int v = 0; v < 16; ++v) s[v] += biasr[tj][tk][v];
+          }
+          s = E::mfma(kf[tk][0], qf[tj][0], s);
+        } else if (flagged) {
+          s = E::mfma(kf[tk][0], qf[tj][0], zero16());
+        } else {
+          s = E::mfma(kf[tk][0], qf[tj][0], biasr[tj][tk]);
+        }
+        f32x16 dp = E::mfma(vf[tk][0], dof[tj][0], zero16());
+#pragma unroll
+        for (int sd = 1; sd < DS; ++sd) {
+          s = E::mfma(kf[tk][sd], qf[tj][sd], s);
+          dp = E::mfma(vf[tk][sd], dof[tj][sd], dp);
         }
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          float p = fast_exp2(__builtin_fmaf(s[v], c, -r.lse2[tj]));
-          if (mixed) p = ((myw >> (16 * (v / 8) + (v % 8))) & 1u) ? p : 0.f;
-          dbacc[tj][tk][v] += p * (dp[v] - r.delta[tj]);
+          const float p = fast_exp2(__builtin_fmaf(s[v], c, -lse2[tj]));
+          dbacc[tj][tk][v] = __builtin_fmaf(p, dp[v] - delta[tj], dbacc[tj][tk][v]);
         }
       }
     }
   };
 
-  if constexpr (PREFETCH) {
-    Row cur, nxt;
-    load_row(cur, 0);
-    for (int i = 0; i < N; ++i) {
-      if (i + 1 < N) load_row(nxt, i + 1);
-      compute_row(cur);
-      cur = nxt;
-    }
-  } else {
-    Row cur;
-    for (int i = 0; i < N; ++i) {
-      load_row(cur, i);
-      compute_row(cur);
-    }
+  issue_row(i_begin, 0);
+  wait_dma();
+  __syncthreads();
+  for (int ir = 0; ir < nrows; ir += 2) {
+    issue_row(i_begin + ir + 1, 1);
+    if (wave_live) compute_row(ir, 0);
+    wait_dma();
+    __syncthreads();
+    if (ir + 1 >= nrows) break;
+    issue_row(i_begin + ir + 2, 0);
+    if (wave_live) compute_row(ir + 1, 1);
+    wait_dma();
+    __syncthreads();
   }
+  if (!wave_live) return;
 
+  // a single chunk writes db itself; several chunks write fp32 partials
+  const bool direct = a.nchunks == 1;
   T* db_bh = reinterpret_cast<T*>(a.db) + (int64_t)bh * N * N;
+  float* part = a.dbpart + ((int64_t)chunk * a.BH + bh) * N * N;
   const bool vec_store = (N % 8) == 0;
 #pragma unroll
   for (int tj = 0; tj < WJ; ++tj) {
@@ -167,6 +192,23 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
 #pragma unroll
       for (int r = 0; r < 2; ++r) {
         const int key0 = k_wave + 32 * tk + 16 * r + 8 * g;
+        if (!direct) {
+          float* dst = part + (int64_t)j * N + key0;
+          if (vec_store && key0 + 8 <= N) {
+#pragma unroll
+            for (int e4 = 0; e4 < 2; ++e4) {
+              f32x4 ov;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) ov[e] = dbacc[tj][tk][8 * r + 4 * e4 + e];
+              *reinterpret_cast<f32x4*>(dst + 4 * e4) = ov;
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (key0 + e < N) dst[e] = dbacc[tj][tk][8 * r + e];
+          }
+          continue;
+        }
         T* dst = db_bh + (int64_t)j * N + key0;
         if (vec_store && key0 + 8 <= N) {
           if constexpr (sizeof(T) == 2) {
@@ -191,6 +233,16 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
       }
     }
   }
+}
+
+// db = sum over chunks of the fp32 partials, in chunk order
+template <typename T>
+__global__ __launch_bounds__(256) void tri_bwd_b_reduce_kernel(const float* part, T* db, int64_t count, int nchunks) {
+  const int64_t x = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (x >= count) return;
+  float acc = part[x];
+  for (int ch = 1; ch < nchunks; ++ch) acc += part[(int64_t)ch * count + x];
+  db[x] = (T)acc;
 }
 
 }  // namespace tri

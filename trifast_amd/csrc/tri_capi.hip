@@ -129,13 +129,14 @@ float dtype_min(int dtype) {
   }
 }
 
-// workspace layout: keep words | row flags | packq | (backward only) packk | delta
+// workspace layout: keep words | row flags | packq | (backward only) packk | delta | db partials
 struct Workspace {
   uint32_t* keep;
   uint8_t* rowflag;
   void* packq;
   void* packk;
   float* delta;
+  float* dbpart;
   int nwords, np;
 };
 
@@ -162,6 +163,8 @@ Workspace carve(void* ws, int64_t b, int64_t h, int64_t n, int dtype) {
   w.packk = p;
   p += ws_pack_bytes(b, h, n, dtype);
   w.delta = reinterpret_cast<float*>(p);
+  p += align256(b * h * n * n * 4);
+  w.dbpart = reinterpret_cast<float*>(p);
   w.nwords = (int)nwords;
   w.np = (int)nwords;
   return w;
@@ -290,7 +293,9 @@ int64_t trifast_fwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, 
 int64_t trifast_bwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype) {
   (void)d;
   if (b < 1 || h < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
-  return ws_mask_bytes(b, n) + 2 * ws_pack_bytes(b, h, n, dtype) + align256(b * h * n * n * 4);
+  const int64_t chunks = tri::bwd_b_chunks(n, b * h);
+  return ws_mask_bytes(b, n) + 2 * ws_pack_bytes(b, h, n, dtype) + align256(b * h * n * n * 4) +
+         (chunks > 1 ? align256(chunks * b * h * n * n * 4) : 0);
 }
 
 int trifast_fwd(void* o, float* lse, const void* q, const void* k, const void* v, const void* bias,
@@ -379,7 +384,10 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   a.q = q; a.k = k; a.v = v; a.o = o; a.dout = dout;
   a.packq = w.packq; a.packk = w.packk;
   a.lse = lse;
-  a.keep = w.keep; a.rowflag = w.rowflag; a.delta = w.delta;
+  a.keep = w.keep; a.rowflag = w.rowflag; a.delta = w.delta; a.dbpart = w.dbpart;
+  a.BH = (int)(b * h);
+  a.nchunks = tri::bwd_b_chunks(n, b * h);
+  a.rows_per_chunk = (int)((n + a.nchunks - 1) / a.nchunks);
   a.dq = dq; a.dk = dk; a.dv = dv; a.db = db;
   a.sq = str5(q_strides); a.sk = str5(k_strides); a.sv = str5(v_strides); a.sdo = str5(do_strides);
   a.H = (int)h; a.N = (int)n; a.NP = w.np; a.nwords = w.nwords;

@@ -40,6 +40,92 @@ TRI_DEV void lds_load_natural(T (*dst)[LD], const T* src, int64_t stride, int nr
   }
 }
 
+// ---------------------------------------------------------------------------
+// Swizzled LDS tiles filled by direct global->LDS loads.
+//
+// A tile holds ROWS rows of D elements, unpadded; the 16-byte chunks of a row are
+// stored XOR-swizzled by swz(row) so that the operand reads of a wave (16 rows at
+// one logical chunk, or 4 rows x 32 bytes for the transposing read) spread over
+// all banks.  global_load_lds writes lane l's 16 bytes at (wave-uniform LDS base)
+// + 16*l, so the swizzle costs nothing: it only decides which global address a
+// lane reads.  The loads use no registers and are tracked by vmcnt; the caller
+// waits with wait_dma() before the barrier that publishes the tile.
+// ---------------------------------------------------------------------------
+#define TRI_G1 __attribute__((address_space(1)))
+#define TRI_L3 __attribute__((address_space(3)))
+
+TRI_DEV void wait_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+template <typename T, int D>
+struct LdsTile {
+  static constexpr int ROWB = D * (int)sizeof(T);  // bytes per row
+  static constexpr int CPR = ROWB / 16;            // 16-byte chunks per row (power of two)
+  static constexpr int RPB = (256 / ROWB) > 0 ? 256 / ROWB : 1;  // rows per 256 bytes
+  static constexpr int VEC = 16 / (int)sizeof(T);
+  TRI_DEV static int swz(int r) { return (r / RPB) % CPR; }
+  // byte offset, from the tile base, of byte `o` of row r (o must not straddle a chunk)
+  TRI_DEV static int off(int r, int o) { return (r * CPR + ((o >> 4) ^ swz(r))) * 16 + (o & 15); }
+  template <typename V>
+  TRI_DEV static V read(const unsigned char* base, int r, int elem) {
+    return *reinterpret_cast<const V*>(base + off(r, elem * (int)sizeof(T)));
+  }
+  // Fill ROWS rows; row_ptr(r) gives the global address of row r (callers clamp r
+  // into range instead of branching).  NW waves share the work.
+  template <int ROWS, int NW, typename RowPtr>
+  TRI_DEV static void fill(unsigned char* base, RowPtr row_ptr, int wave, int lane) {
+    constexpr int GROUPS = ROWS * CPR / 64;
+    static_assert(ROWS * CPR % 64 == 0, "tile must be a whole number of 1 KiB wave loads");
+#pragma unroll
+    for (int x = 0; x < (GROUPS + NW - 1) / NW; ++x) {
+      const int gi = x * NW + wave;
+      if (GROUPS % NW == 0 || gi < GROUPS) {
+        const int p = gi * 64 + lane;
+        const int r = p / CPR, c = (p % CPR) ^ swz(r);
+        const T* src = row_ptr(r) + c * VEC;
+        __builtin_amdgcn_global_load_lds((const TRI_G1 void*)src, (TRI_L3 void*)(base + gi * 1024), 16, 0, 0);
+      }
+    }
+  }
+  // A/B operand with the head-dim index in-lane: row `r`, MFMA step s over d
+  TRI_DEV static typename Elem<T>::frag operand(const unsigned char* base, int r, int s, int g) {
+    constexpr int KP = Elem<T>::KP;
+    return read<typename Elem<T>::frag>(base, r, 2 * KP * s + KP * g);
+  }
+  // operand with the row (contraction) index in-lane: rows base_row + cidx(KP*step .. , g),
+  // column col0 + lane%32; columns >= ncols read as zero
+  TRI_DEV static typename Elem<T>::frag tr_operand(const unsigned char* base, int base_row, int step, int col0, int ncols, int lane) {
+    constexpr int KP = Elem<T>::KP;
+    const int g = lane >> 5;
+    if (col0 + (lane & 31) >= ncols) return Elem<T>::zero();
+    if constexpr (KP == 1) {
+      return read<float>(base, base_row + cidx(step, g), col0 + (lane & 31));
+    } else {
+      const int L = lane & 15, chalf = (lane >> 4) & 1;
+      const int row0 = base_row + cidx(KP * step, g);
+      const int col = col0 + 16 * chalf + 4 * (L & 3);
+      const auto lo = lds_tr4(reinterpret_cast<const T*>(base + off(row0 + (L >> 2), col * 2)));
+      const auto hi = lds_tr4(reinterpret_cast<const T*>(base + off(row0 + 4 + (L >> 2), col * 2)));
+      typename Elem<T>::frag f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { f[e] = lo[e]; f[4 + e] = hi[e]; }
+      return f;
+    }
+  }
+};
+
+// 4-byte-per-lane variant for rows of floats (lse, delta): 64 floats per wave load
+template <int COUNT, int NW, typename Ptr>
+TRI_DEV void fill_floats(float* base, Ptr elem_ptr, int wave, int lane) {
+  constexpr int GROUPS = COUNT / 64;
+  static_assert(COUNT % 64 == 0, "whole wave loads only");
+#pragma unroll
+  for (int x = 0; x < (GROUPS + NW - 1) / NW; ++x) {
+    const int gi = x * NW + wave;
+    if (GROUPS % NW == 0 || gi < GROUPS)
+      __builtin_amdgcn_global_load_lds((const TRI_G1 void*)elem_ptr(gi * 64 + lane), (TRI_L3 void*)(base + gi * 64), 4, 0, 0);
+  }
+}
+
 // Two-phase version of the same copy, for software pipelining: the global loads
 // of the next tile are issued into registers before the current tile is computed
 // and written to LDS afterwards.
