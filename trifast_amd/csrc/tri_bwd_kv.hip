@@ -7,25 +7,25 @@ namespace {
 
 struct BwdKVFamily {
   static constexpr int kNumTiles = 4;
-  // {NW, KT, BJ}: block of NW*KT*32 keys, queries streamed BJ at a time
+  // {NW, R, BJ}: block of NW*32 keys x R pair rows, queries streamed BJ at a time
   static constexpr int P(int tile, int which) {
     constexpr int t[kNumTiles][3] = {
-        {4, 1, 32},  // 0: 128 keys x 32 queries
-        {4, 1, 64},  // 1: 128 keys x 64 queries
-        {4, 2, 64},  // 2: 256 keys x 64 queries
-        {2, 1, 32},  // 3:  64 keys x 32 queries
+        {4, 1, 64},  // 0: 128 keys x 1 row,  64 queries per stage (fits every dtype / head dim)
+        {4, 2, 32},  // 1: 128 keys x 2 rows, 32 queries per stage
+        {4, 2, 64},  // 2: 128 keys x 2 rows, 64 queries per stage
+        {2, 2, 32},  // 3:  64 keys x 2 rows, 32 queries per stage
     };
     return t[tile][which];
   }
-  template <typename T, int D, int NW, int KT, int BJ>
+  template <typename T, int D, int NW, int R, int BJ>
   static hipError_t run(const BwdArgs& a, int bh, hipStream_t st, bool dry) {
-    constexpr int PAD = 16 / sizeof(T);
-    constexpr int lds = 2 * BJ * (D + PAD) * (int)sizeof(T) + 8 * BJ;
-    if constexpr (lds <= kMaxStaticLds) {
+    constexpr int stage = 2 * R * BJ * D * (int)sizeof(T) + 2 * R * BJ * 4 + NW * (BJ / 32) * 1024 * (int)sizeof(T);
+    // K, V operands and the dk, dv accumulators of the R rows stay in registers
+    constexpr int acc_regs = R * (2 * ((D + 31) / 32) * 16 + 2 * (D / 2) * (int)sizeof(T) / 4);
+    if constexpr (2 * stage <= kMaxLds && acc_regs <= 200) {
       if (dry) return hipSuccess;
-      dim3 grid((a.N + NW * KT * 32 - 1) / (NW * KT * 32), (a.N + 7) / 8 * 8, bh);
-      hipLaunchKernelGGL((tri_bwd_kv_kernel<T, D, NW, KT, BJ>), grid, dim3(NW * 64), 0, st, a);
-      return hipGetLastError();
+      dim3 grid((a.N + NW * 32 - 1) / (NW * 32), ((a.N + R - 1) / R + 7) / 8 * 8, bh);
+      return launch_dyn(tri_bwd_kv_kernel<T, D, NW, R, BJ>, grid, dim3(NW * 64), 2 * stage, st, a);
     } else {
       return hipErrorInvalidConfiguration;
     }
@@ -38,7 +38,7 @@ int bwd_kv_num_tiles() { return BwdKVFamily::kNumTiles; }
 
 TileInfo bwd_kv_tile_info(int tile) {
   // block_j = queries per LDS stage, block_k = keys per workgroup
-  return TileInfo{BwdKVFamily::P(tile, 2), BwdKVFamily::P(tile, 0) * BwdKVFamily::P(tile, 1) * 32, BwdKVFamily::P(tile, 0)};
+  return TileInfo{BwdKVFamily::P(tile, 2), BwdKVFamily::P(tile, 0) * 32, BwdKVFamily::P(tile, 0)};
 }
 
 bool bwd_kv_supports(int tile, int64_t n, int d, int dtype) {

@@ -41,17 +41,18 @@ __global__ __launch_bounds__(NW * 64) void tri_fwd_kernel(const FwdArgs a) {
   constexpr int DM = (D + 31) / 32;  // 32-row tiles of O^T
   constexpr int PS = 32 / (2 * KP);  // MFMA steps over a 32-key tile
   constexpr int KU = BK / 32;
-  constexpr int PAD = 16 / sizeof(T);
-  constexpr int LD = D + PAD;
   constexpr int NT = NW * 64;
 
-  // [buffer][K rows of row 0..R-1, then V rows of row 0..R-1]; dynamic so that
-  // the larger instantiations may use more than the 64 KiB static limit
+  // One stage: K rows of the R pair rows | V rows | packed bias tiles of the NW waves.
+  // Two stages (double buffer), then the keep words of the R rows.  The tiles are
+  // filled by direct global->LDS loads and read through the swizzle of LdsTile.
+  using Tile = LdsTile<T, D>;
+  constexpr int ROWB = Tile::ROWB;
+  constexpr int OFF_K = 0, OFF_V = R * BK * ROWB, OFF_B = 2 * R * BK * ROWB;
+  constexpr int BIAS_B = 2 * 64 * 8 * (int)sizeof(T);  // one packed 32 x 32 bias tile
+  constexpr int STAGE = OFF_B + NW * KU * BIAS_B;
   extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
-  T(*KVs)[2 * R * BK][LD] = reinterpret_cast<T(*)[2 * R * BK][LD]>(tri_smem);
-  // keep words of the R rows, copied to LDS once: reading them there keeps the
-  // global-load counter of the main loop free for the prefetched tiles
-  uint32_t* keep_s = reinterpret_cast<uint32_t*>(tri_smem + 2 * sizeof(T) * (2 * R * BK) * LD);
+  uint32_t* keep_s = reinterpret_cast<uint32_t*>(tri_smem + 2 * STAGE);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -119,45 +120,55 @@ __global__ __launch_bounds__(NW * 64) void tri_fwd_kernel(const FwdArgs a) {
     return kt0;
   };
 
-  // global -> register -> LDS staging of the K and V tiles of all R rows
-  constexpr int CPR = D / E::VEC;
-  constexpr int CHUNKS = 2 * R * BK * CPR;
-  constexpr int CNT = (CHUNKS + NT - 1) / NT;
-  typename E::vec stage[CNT];
-
-  // Loads are issued unconditionally (indices clamped into range instead of
-  // branching) so that the number of loads in flight is the same on every path
-  // and the waits on them can be exact.  A clamped key row duplicates the last
-  // valid one; its keep bit is clear, so it contributes exactly zero.
+  // Stage loads: direct global->LDS, issued unconditionally (indices clamped into
+  // range instead of branching).  A clamped key row duplicates the last valid one;
+  // its keep bit is clear, so it contributes exactly zero.
   const int jt_ld = min(jt, a.NP - 1);
-  auto issue_loads = [&](int kt0, BiasRegs<T>* bias) {
+  auto issue_loads = [&](int kt0, int buf) {
+    unsigned char* st = tri_smem + buf * STAGE;
+    Tile::template fill<R * BK, NW>(st + OFF_K, [&](int x) {
+      return kbh + min(i0 + x / BK, N - 1) * a.sk.i + (int64_t)min(kt0 + x % BK, N - 1) * a.sk.j; }, wave, lane);
+    Tile::template fill<R * BK, NW>(st + OFF_V, [&](int x) {
+      return vbh + min(i0 + x / BK, N - 1) * a.sv.i + (int64_t)min(kt0 + x % BK, N - 1) * a.sv.j; }, wave, lane);
+    // each wave fetches the packed bias tiles of its own query tile: 2 x 1 KiB per key tile
 #pragma unroll
-    for (int x = 0; x < CNT; ++x) {
-      const int ch = (CHUNKS % NT == 0) ? x * NT + tid : min(x * NT + tid, CHUNKS - 1);
-      const int arr = ch / (BK * CPR);  // 0..R-1: K of row arr; R..2R-1: V of row arr-R
-      const int rem = ch % (BK * CPR);
-      const int row = min(kt0 + rem / CPR, N - 1), col = (rem % CPR) * E::VEC;
-      const int i = min(i0 + arr % R, N - 1);
-      const T* src = (arr >= R) ? vbh + i * a.sv.i + (int64_t)row * a.sv.j
-                                : kbh + i * a.sk.i + (int64_t)row * a.sk.j;
-      stage[x] = *reinterpret_cast<const typename E::vec*>(src + col);
+    for (int u = 0; u < KU; ++u) {
+      const T* p = pack_bh + (((int64_t)jt_ld * a.NP + min((kt0 >> 5) + u, a.NP - 1)) * 2 * 64 + lane) * 8;
+#pragma unroll
+      for (int r2 = 0; r2 < 2; ++r2) {
+        unsigned char* dst = st + OFF_B + (wave * KU + u) * BIAS_B + r2 * (BIAS_B / 2);
+        if constexpr (sizeof(T) == 2) {
+          __builtin_amdgcn_global_load_lds((const TRI_G1 void*)(p + r2 * 512), (TRI_L3 void*)dst, 16, 0, 0);
+        } else {
+          __builtin_amdgcn_global_load_lds((const TRI_G1 void*)(p + r2 * 512), (TRI_L3 void*)dst, 16, 0, 0);
+          __builtin_amdgcn_global_load_lds((const TRI_G1 void*)(p + r2 * 512 + 4), (TRI_L3 void*)(dst + 1024), 16, 0, 0);
+        }
+      }
     }
-#pragma unroll
-    for (int u = 0; u < KU; ++u) bias[u].load(pack_bh, a.NP, jt_ld, min((kt0 >> 5) + u, a.NP - 1), lane);
   };
-  auto store_stage = [&](int buf) {
+  // the 16 bias values of this lane for key tile u of the stage, raw-score domain
+  auto bias_from_lds = [&](int buf, int u) -> f32x16 {
+    const unsigned char* src = tri_smem + buf * STAGE + OFF_B + (wave * KU + u) * BIAS_B;
+    f32x16 bv;
 #pragma unroll
-    for (int x = 0; x < CNT; ++x) {
-      const int ch = x * NT + tid;
-      const int arr = ch / (BK * CPR);
-      const int rem = ch % (BK * CPR);
-      const int row = rem / CPR, col = (rem % CPR) * E::VEC;
-      if (CHUNKS % NT == 0 || ch < CHUNKS) *reinterpret_cast<typename E::vec*>(&KVs[buf][arr * BK + row][col]) = stage[x];
+    for (int r2 = 0; r2 < 2; ++r2) {
+      if constexpr (sizeof(T) == 2) {
+        const typename E::vec x = *reinterpret_cast<const typename E::vec*>(src + r2 * (BIAS_B / 2) + lane * 16);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bv[8 * r2 + e] = (float)x[e] * a.sqrt_d;
+      } else {
+        const f32x4 x0 = *reinterpret_cast<const f32x4*>(src + r2 * (BIAS_B / 2) + lane * 16);
+        const f32x4 x1 = *reinterpret_cast<const f32x4*>(src + r2 * (BIAS_B / 2) + 1024 + lane * 16);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { bv[8 * r2 + e] = x0[e] * a.sqrt_d; bv[8 * r2 + 4 + e] = x1[e] * a.sqrt_d; }
+      }
     }
+    return bv;
   };
 
   // one stage of compute from LDS buffer `buf`
-  auto compute_stage = [&](int buf, const uint32_t (*kw)[KU], const BiasRegs<T>* bias) {
+  auto compute_stage = [&](int buf, const uint32_t (*kw)[KU]) {
+    const unsigned char* st = tri_smem + buf * STAGE;
     if (wave_active) {
       // The KU*R tiles of the stage run as a software pipeline inside the wave: the
       // MFMA chain that produces the scores of tile t+1 is issued before the
@@ -168,17 +179,15 @@ __global__ __launch_bounds__(NW * 64) void tri_fwd_kernel(const FwdArgs a) {
       constexpr int TS = KU * R;
       auto k_operand = [&](int t, frag* kf) {
         const int u = t / R, r = t % R;
-        const T(*Kt)[LD] = &KVs[buf][r * BK];
 #pragma unroll
-        for (int sd = 0; sd < DS; ++sd)
-          kf[sd] = *reinterpret_cast<const frag*>(&Kt[32 * u + perm32(jl)][2 * KP * sd + KP * g]);
+        for (int sd = 0; sd < DS; ++sd) kf[sd] = Tile::operand(st + OFF_K, r * BK + 32 * u + perm32(jl), sd, g);
       };
       // The bias tile does not depend on the pair row: it is converted to fp32 in
       // the raw-score domain once per stage and key tile, and then serves as the
       // accumulator init (C operand) of the first score MFMA of each of the R rows.
       f32x16 biasv[KU];
 #pragma unroll
-      for (int u = 0; u < KU; ++u) biasv[u] = bias_tile<T>(bias[u], a.sqrt_d, 0.f);
+      for (int u = 0; u < KU; ++u) biasv[u] = bias_from_lds(buf, u);
       auto scores = [&](int t, const frag* kf) -> f32x16 {
         const int u = t / R, r = t % R;
         f32x16 sc;
@@ -216,12 +225,11 @@ __global__ __launch_bounds__(NW * 64) void tri_fwd_kernel(const FwdArgs a) {
         }
         if (kw[r][u] != 0) {  // a row that attends to no key of this tile adds nothing
           // V^T rows as A operand of the second product
-          const T(*Vt)[LD] = &KVs[buf][(R + r) * BK];
           frag vf[DM][PS];
 #pragma unroll
           for (int mt = 0; mt < DM; ++mt)
 #pragma unroll
-            for (int s2 = 0; s2 < PS; ++s2) vf[mt][s2] = tr_operand<T, LD>(Vt, 32 * u, s2, 32 * mt, D, lane);
+            for (int s2 = 0; s2 < PS; ++s2) vf[mt][s2] = Tile::tr_operand(st + OFF_V, r * BK + 32 * u, s2, 32 * mt, D, lane);
           // exponent arguments against the current reference; results of an fma are
           // canonical floats, so the max below needs no extra canonicalisation
           float arg[16];
@@ -266,31 +274,27 @@ __global__ __launch_bounds__(NW * 64) void tri_fwd_kernel(const FwdArgs a) {
 
   };
 
-  // The stage loop is unrolled by two so that the two sets of bias registers and
-  // keep words swap roles without being copied.
-  BiasRegs<T> bias0[KU], bias1[KU];
+  // The stage loop is unrolled by two so that the two sets of keep words swap
+  // roles without being copied.
   uint32_t keep0[R][KU], keep1[R][KU];
   __syncthreads();  // keep words visible
   int kt0 = next_live(0, keep0);
-  issue_loads(min(kt0, N - 1), bias0);
-  store_stage(0);
-  // everything loaded so far (Q operands, first stage) has landed before the loop,
-  // so waits inside it only ever concern the loads issued inside it
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  issue_loads(min(kt0, N - 1), 0);
+  wait_dma();
   __syncthreads();
   while (kt0 < N) {
     // past the last live stage the prefetch re-reads a valid stage that nobody uses
     int kt1 = next_live(kt0 + BK, keep1);
-    issue_loads(min(kt1, N - 1), bias1);
-    compute_stage(0, keep0, bias0);
-    store_stage(1);
+    issue_loads(min(kt1, N - 1), 1);
+    compute_stage(0, keep0);
+    wait_dma();
     __syncthreads();
     if (kt1 >= N) break;
     kt0 = kt1;
     kt1 = next_live(kt0 + BK, keep0);
-    issue_loads(min(kt1, N - 1), bias0);
-    compute_stage(1, keep1, bias1);
-    store_stage(0);
+    issue_loads(min(kt1, N - 1), 0);
+    compute_stage(1, keep1);
+    wait_dma();
     __syncthreads();
     kt0 = kt1;
   }
