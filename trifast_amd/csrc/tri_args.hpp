@@ -11,7 +11,7 @@ struct MaskPrepArgs {
   const uint8_t* mask;       // [b, n, n] bytes, nonzero = masked out
   int64_t sb, si, sk;
   uint32_t* keep;            // [b, n, nwords]: bit set = key is attended to
-  uint8_t* rowflag;          // [b, n]: 1 = every valid key of the row is masked
+  uint32_t* rowflag;         // [b, n]: 1 = every valid key of the row is masked
   int n, nwords;
 };
 
@@ -33,7 +33,7 @@ struct FwdArgs {
   const void *q, *k, *v;
   const void* packq;
   const uint32_t* keep;
-  const uint8_t* rowflag;
+  const uint32_t* rowflag;
   void* o;
   float* lse;
   Str5 sq, sk, sv;
@@ -48,7 +48,7 @@ struct BwdArgs {
   const void *packq, *packk;
   const float* lse;
   const uint32_t* keep;
-  const uint8_t* rowflag;
+  const uint32_t* rowflag;
   float* delta;              // [b*h, n, n] fp32 workspace, indexed [i, j]
   float* dbpart;             // [nchunks, b*h, n, n] fp32 partial db (nchunks > 1 only)
   void *dq, *dk, *dv, *db;

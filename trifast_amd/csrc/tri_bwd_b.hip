@@ -18,19 +18,21 @@ struct BwdBFamily {
   }
   template <typename T, int D, int WJ, int WK>
   static constexpr int stage_bytes() {
-    return (2 * 2 * WJ * 32 + 2 * 2 * WK * 32) * D * (int)sizeof(T) + 2 * (2 * WJ * 32) * 4;
+    return (2 * 2 * WJ * 32 + 2 * 2 * WK * 32) * D * (int)sizeof(T) + 2 * (2 * WJ * 32) * 4 + 256;
   }
   template <typename T, int D, int WJ, int WK, int>
   static hipError_t run(const BwdArgs& a, int bh, hipStream_t st, bool dry) {
     // registers of one row's operands, the db accumulators and the bias tiles
     constexpr int frag_regs = (2 * WJ + 2 * WK) * (D / 2) * (int)sizeof(T) / 4;
-    constexpr bool fits = 2 * WJ * WK * 16 + frag_regs <= 320 && 2 * stage_bytes<T, D, WJ, WK>() + 1024 <= kMaxLds;
+    constexpr int stage = stage_bytes<T, D, WJ, WK>();
+    constexpr int nbuf = 2 * stage <= kMaxLds ? 2 : 1;
+    // the smallest tile always runs (at the price of register spills for large head dims)
+    constexpr bool fits = stage <= kMaxLds && (2 * WJ * WK * 16 + frag_regs <= 320 || WJ * WK == 1);
     if constexpr (fits) {
       if (dry) return hipSuccess;
-      const int lds = 2 * stage_bytes<T, D, WJ, WK>() + a.rows_per_chunk * (2 * WK + 1) * 4;
-      if (lds > kMaxLds) return hipErrorInvalidConfiguration;
+      const int lds = nbuf * stage;
       dim3 grid((a.N + 2 * WJ * 32 - 1) / (2 * WJ * 32), (a.N + 2 * WK * 32 - 1) / (2 * WK * 32), bh * a.nchunks);
-      hipError_t e = launch_dyn(tri_bwd_b_kernel<T, D, WJ, WK>, grid, dim3(256), lds, st, a);
+      hipError_t e = launch_dyn(tri_bwd_b_kernel<T, D, WJ, WK, nbuf>, grid, dim3(256), lds, st, a);
       if (e != hipSuccess || a.nchunks == 1) return e;
       const int64_t count = (int64_t)bh * a.N * a.N;
       hipLaunchKernelGGL(tri_bwd_b_reduce_kernel<T>, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st,

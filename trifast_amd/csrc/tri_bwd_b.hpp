@@ -21,7 +21,7 @@
 
 namespace tri {
 
-template <typename T, int D, int WJ, int WK>
+template <typename T, int D, int WJ, int WK, int NBUF>
 __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
   using E = Elem<T>;
   using frag = typename E::frag;
@@ -31,15 +31,15 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
   constexpr int NW = 4;
   constexpr int BJ = 2 * WJ * 32, BKB = 2 * WK * 32;  // queries / keys per workgroup
   constexpr int ROWB = Tile::ROWB;
-  // one stage: Q rows | dO rows | K rows | V rows | lse[BJ] | delta[BJ]
+  // one stage: Q rows | dO rows | K rows | V rows | lse[BJ] | delta[BJ] | row meta
+  // (64 words: the WKW keep words of the key block, then the row's flag)
   constexpr int OFF_Q = 0, OFF_DO = BJ * ROWB, OFF_K = 2 * BJ * ROWB, OFF_V = OFF_K + BKB * ROWB;
   constexpr int OFF_LSE = OFF_V + BKB * ROWB, OFF_DELTA = OFF_LSE + BJ * 4;
-  constexpr int STAGE = OFF_DELTA + BJ * 4;
+  constexpr int OFF_META = OFF_DELTA + BJ * 4;
+  constexpr int STAGE = OFF_META + 256;
+  constexpr int WKW = BKB / 32;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
-  // after the two stages: keep words [rows][WKW] and row flags [rows] of this chunk
-  constexpr int WKW = BKB / 32;
-  uint32_t* keep_s = reinterpret_cast<uint32_t*>(tri_smem + 2 * STAGE);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -53,7 +53,6 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
   const int i_begin = chunk * a.rows_per_chunk;
   const int i_end = min(N, i_begin + a.rows_per_chunk);
   const int nrows = i_end - i_begin;
-  uint32_t* flag_s = keep_s + a.rows_per_chunk * WKW;
 
   const T* qbase = reinterpret_cast<const T*>(a.q) + b * a.sq.b + h * a.sq.h;
   const T* kbase = reinterpret_cast<const T*>(a.k) + b * a.sk.b + h * a.sk.h;
@@ -62,13 +61,6 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
   const T* pack_bh = reinterpret_cast<const T*>(a.packq) + (int64_t)bh * a.NP * a.NP * 1024;
   const float* lse_bh = a.lse + (int64_t)bh * N * N;
   const float* delta_bh = a.delta + (int64_t)bh * N * N;
-
-  // keep words and row flags of the chunk's rows, once
-  for (int x = tid; x < nrows * WKW; x += 256) {
-    const int i = i_begin + x / WKW, w = k_blk / 32 + x % WKW;
-    keep_s[x] = (w < a.nwords) ? a.keep[((int64_t)b * N + i) * a.nwords + w] : 0u;
-  }
-  for (int x = tid; x < nrows; x += 256) flag_s[x] = a.rowflag[(int64_t)b * N + i_begin + x];
 
   // bias tiles in the raw-score domain: accumulator init of every row's score MFMA
   f32x16 biasr[WJ][WK];
@@ -94,15 +86,22 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
     Tile::template fill<BKB, NW>(st + OFF_V, [&](int r) { return vbase + i * a.sv.i + (int64_t)min(k_blk + r, N - 1) * a.sv.j; }, wave, lane);
     fill_floats<BJ, NW>(reinterpret_cast<float*>(st + OFF_LSE), [&](int x) { return lse_bh + (int64_t)i * N + min(j_blk + x, N - 1); }, wave, lane);
     fill_floats<BJ, NW>(reinterpret_cast<float*>(st + OFF_DELTA), [&](int x) { return delta_bh + (int64_t)i * N + min(j_blk + x, N - 1); }, wave, lane);
+    if (wave == NW - 1) {
+      // lanes 0..WKW-1: keep words of this key block; lane WKW: the row flag
+      const uint32_t* src = (lane == WKW) ? a.rowflag + (int64_t)b * N + i
+                                          : a.keep + ((int64_t)b * N + i) * a.nwords + min(k_blk / 32 + min(lane, WKW - 1), a.nwords - 1);
+      __builtin_amdgcn_global_load_lds((const TRI_G1 void*)src, (TRI_L3 void*)(st + OFF_META), 4, 0, 0);
+    }
   };
 
   const float c = a.c;
   const float lse2_flagged = fast_log2((float)N);
   const bool wave_live = j_wave < N && k_wave < N;
 
-  auto compute_row = [&](int ir, int buf) {
+  auto compute_row = [&](int buf) {
     const unsigned char* st = tri_smem + buf * STAGE;
-    const bool flagged = flag_s[ir] != 0;
+    const uint32_t* meta = reinterpret_cast<const uint32_t*>(st + OFF_META);
+    const bool flagged = meta[WKW] != 0;
     // operands of this wave's tiles; tile row m of the key tiles stands for key perm32(m)
     frag qf[WJ][DS], dof[WJ][DS], kf[WK][DS], vf[WK][DS];
     float lse2[WJ], delta[WJ];
@@ -129,7 +128,8 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
     }
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk) {
-      const uint32_t keepw = keep_s[ir * WKW + wk * WK + tk];
+      // a key tile past the last word of the row has no attended key
+      const uint32_t keepw = (k_wave / 32 + tk < a.nwords) ? meta[wk * WK + tk] : 0u;
       if (keepw == 0) continue;  // no attended key in this tile: dS = 0
       const bool mixed = keepw != 0xffffffffu;
 #pragma unroll
@@ -162,19 +162,30 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
     }
   };
 
-  issue_row(i_begin, 0);
-  wait_dma();
-  __syncthreads();
-  for (int ir = 0; ir < nrows; ir += 2) {
-    issue_row(i_begin + ir + 1, 1);
-    if (wave_live) compute_row(ir, 0);
+  if constexpr (NBUF == 2) {
+    issue_row(i_begin, 0);
     wait_dma();
     __syncthreads();
-    if (ir + 1 >= nrows) break;
-    issue_row(i_begin + ir + 2, 0);
-    if (wave_live) compute_row(ir + 1, 1);
-    wait_dma();
-    __syncthreads();
+    for (int ir = 0; ir < nrows; ir += 2) {
+      issue_row(i_begin + ir + 1, 1);
+      if (wave_live) compute_row(0);
+      wait_dma();
+      __syncthreads();
+      if (ir + 1 >= nrows) break;
+      issue_row(i_begin + ir + 2, 0);
+      if (wave_live) compute_row(1);
+      wait_dma();
+      __syncthreads();
+    }
+  } else {
+    // one stage only (the double buffer does not fit in LDS): load, then compute
+    for (int ir = 0; ir < nrows; ++ir) {
+      issue_row(i_begin + ir, 0);
+      wait_dma();
+      __syncthreads();
+      if (wave_live) compute_row(0);
+      __syncthreads();
+    }
   }
   if (!wave_live) return;
 

@@ -22,10 +22,12 @@ struct BwdKVFamily {
     constexpr int stage = 2 * R * BJ * D * (int)sizeof(T) + 2 * R * BJ * 4 + NW * (BJ / 32) * 1024 * (int)sizeof(T);
     // K, V operands and the dk, dv accumulators of the R rows stay in registers
     constexpr int acc_regs = R * (2 * ((D + 31) / 32) * 16 + 2 * (D / 2) * (int)sizeof(T) / 4);
-    if constexpr (2 * stage <= kMaxLds && acc_regs <= 200) {
+    // the one-row tile always runs (at the price of register spills for large head dims)
+    constexpr int nbuf = 2 * stage <= kMaxLds ? 2 : 1;
+    if constexpr (stage <= kMaxLds && (acc_regs <= 200 || R == 1)) {
       if (dry) return hipSuccess;
       dim3 grid((a.N + NW * 32 - 1) / (NW * 32), ((a.N + R - 1) / R + 7) / 8 * 8, bh);
-      return launch_dyn(tri_bwd_kv_kernel<T, D, NW, R, BJ>, grid, dim3(NW * 64), 2 * stage, st, a);
+      return launch_dyn(tri_bwd_kv_kernel<T, D, NW, R, BJ, nbuf>, grid, dim3(NW * 64), nbuf * stage, st, a);
     } else {
       return hipErrorInvalidConfiguration;
     }

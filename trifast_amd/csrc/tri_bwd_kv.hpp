@@ -21,7 +21,7 @@
 
 namespace tri {
 
-template <typename T, int D, int NW, int R, int BJ>
+template <typename T, int D, int NW, int R, int BJ, int NBUF>
 __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
   using E = Elem<T>;
   using frag = typename E::frag;
@@ -212,19 +212,30 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
     }
   };
 
-  issue_loads(0, 0);
-  wait_dma();
-  __syncthreads();
-  for (int jt0 = 0; jt0 < N; jt0 += 2 * BJ) {
-    issue_loads(min(jt0 + BJ, N - 1), 1);
-    if (wave_active) compute_stage(jt0, 0);
+  if constexpr (NBUF == 2) {
+    issue_loads(0, 0);
     wait_dma();
     __syncthreads();
-    if (jt0 + BJ >= N) break;
-    issue_loads(min(jt0 + 2 * BJ, N - 1), 0);
-    if (wave_active) compute_stage(jt0 + BJ, 1);
-    wait_dma();
-    __syncthreads();
+    for (int jt0 = 0; jt0 < N; jt0 += 2 * BJ) {
+      issue_loads(min(jt0 + BJ, N - 1), 1);
+      if (wave_active) compute_stage(jt0, 0);
+      wait_dma();
+      __syncthreads();
+      if (jt0 + BJ >= N) break;
+      issue_loads(min(jt0 + 2 * BJ, N - 1), 0);
+      if (wave_active) compute_stage(jt0 + BJ, 1);
+      wait_dma();
+      __syncthreads();
+    }
+  } else {
+    // one stage only (the double buffer does not fit in LDS): load, then compute
+    for (int jt0 = 0; jt0 < N; jt0 += BJ) {
+      issue_loads(jt0, 0);
+      wait_dma();
+      __syncthreads();
+      if (wave_active) compute_stage(jt0, 0);
+      __syncthreads();
+    }
   }
 
   if (!wave_active || key >= N) return;

@@ -132,7 +132,7 @@ float dtype_min(int dtype) {
 // workspace layout: keep words | row flags | packq | (backward only) packk | delta | db partials
 struct Workspace {
   uint32_t* keep;
-  uint8_t* rowflag;
+  uint32_t* rowflag;
   void* packq;
   void* packk;
   float* delta;
@@ -142,7 +142,7 @@ struct Workspace {
 
 int64_t ws_mask_bytes(int64_t b, int64_t n) {
   const int64_t nwords = (n + 31) / 32;
-  return align256(b * n * nwords * 4) + align256(b * n);
+  return align256(b * n * nwords * 4) + align256(b * n * 4);
 }
 
 int64_t ws_pack_bytes(int64_t b, int64_t h, int64_t n, int dtype) {
@@ -156,8 +156,8 @@ Workspace carve(void* ws, int64_t b, int64_t h, int64_t n, int dtype) {
   char* p = static_cast<char*>(ws);
   w.keep = reinterpret_cast<uint32_t*>(p);
   p += align256(b * n * nwords * 4);
-  w.rowflag = reinterpret_cast<uint8_t*>(p);
-  p += align256(b * n);
+  w.rowflag = reinterpret_cast<uint32_t*>(p);
+  p += align256(b * n * 4);
   w.packq = p;
   p += ws_pack_bytes(b, h, n, dtype);
   w.packk = p;
@@ -266,15 +266,17 @@ int trifast_supports(int kernel, int tile, int64_t n, int64_t h, int64_t d, int 
 
 int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype) {
   (void)h;
+  // Picks measured on MI355X at d = 32; anything that does not fit the shape
+  // falls back to tile 0, which every dtype and head dim supports.
   int pick = 0;
   switch (kernel) {
-    case TRIFAST_KERNEL_FWD:
-      // more pair rows per workgroup = fewer bias reads; fall back when it does not fit
-      pick = n <= 64 ? 0 : 2;
-      while (pick > 0 && !trifast_supports(kernel, pick, n, h, d, dtype)) --pick;
-      break;
-    default: pick = 0; break;
+    case TRIFAST_KERNEL_FWD: pick = n <= 64 ? 0 : 3; break;     // 4 pair rows share a bias tile
+    case TRIFAST_KERNEL_BWD_Q: pick = n <= 64 ? 0 : 2; break;   // 2 pair rows, 32 keys per stage
+    case TRIFAST_KERNEL_BWD_KV: pick = n <= 64 ? 0 : 2; break;  // 2 pair rows, 64 queries per stage
+    case TRIFAST_KERNEL_BWD_B: pick = 2; break;                 // 64 x 64 block, most workgroups per CU
+    default: return fail(TRIFAST_EINVAL, "unknown kernel id %d", kernel);
   }
+  if (!trifast_supports(kernel, pick, n, h, d, dtype)) pick = 0;
   if (!trifast_supports(kernel, pick, n, h, d, dtype)) {
     const int nt = trifast_num_tiles(kernel);
     for (int t = 0; t < nt; ++t)

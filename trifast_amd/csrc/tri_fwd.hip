@@ -23,7 +23,7 @@ struct FwdFamily {
     constexpr int lds = 2 * (2 * R * BK * D + NW * (BK / 32) * 1024) * (int)sizeof(T);
     // R rows of accumulators and Q operands per wave must stay in registers
     constexpr int acc_regs = R * (((D + 31) / 32) * 16 + D / 2 * (int)sizeof(T) / 4);
-    if constexpr (lds <= kMaxLds && acc_regs <= 160) {
+    if constexpr (lds <= kMaxLds && (acc_regs <= 160 || R == 1)) {
       if (dry) return hipSuccess;
       dim3 grid((a.N + NW * 32 - 1) / (NW * 32), ((a.N + R - 1) / R + 7) / 8 * 8, bh);
       const int lds_total = lds + R * a.nwords * 4;  // + keep words of the R rows
