@@ -201,6 +201,9 @@ def main():
     ap.add_argument("--workload", default="M", choices=[w for w in WORKLOADS if w != "C1"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain 256 MiB device copy, the known-size kernel that "
+                         "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -225,6 +228,14 @@ def main():
     def fwd_only():
         with torch.no_grad():
             trifast_amd.triangle_attention(q, k, v, bias, mask)
+
+    if args.calibrate_copy:
+        src = torch.zeros(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):  # also warms the tile cache
         step()

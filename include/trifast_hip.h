@@ -96,9 +96,10 @@ int trifast_fwd(void* o, float* lse,
  * Backward: dq, dk, dv, db from do and the saved q, k, v, bias, mask, o, lse.
  * Replaces the _bwd_q, _bwd_kv and _bwd_b launches of reference
  * src/trifast/torch.py:111-174 (one call, fixed launch order, deterministic).
- * do may have any strides with sd == 1 or sd == 0 patterns excluded: the caller
- * materialises a do whose last stride is not 1.  o and lse are the forward's
- * contiguous outputs.  tiles[3] = {bwd_q, bwd_kv, bwd_b} tile ids (<0: default).
+ * do may have any strides over b, h, i, j (stride 0 included, as a broadcast
+ * gradient has), but its rows must be 16-byte aligned with last stride 1: the
+ * caller materialises a do that is not.  o and lse are the forward's contiguous
+ * outputs.  tiles[3] = {bwd_q, bwd_kv, bwd_b} tile ids (<0: default).
  */
 int trifast_bwd(void* dq, void* dk, void* dv, void* db,
                 const void* dout, const void* q, const void* k, const void* v,
