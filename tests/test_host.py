@@ -120,7 +120,7 @@ def test_pick_times_every_supported_tile_on_a_miss(tmp_path, monkeypatch):
     monkeypatch.delenv("TRIFAST_FORCE_TUNE", raising=False)
     monkeypatch.setattr(tuner, "_device_tag", lambda device=None: "Test-GPU_9-5")
     fake_ms = {0: 3.0, 1: 1.0, 2: 5.0, 3: 2.0}
-    monkeypatch.setattr(tuner, "_time_launch", lambda launch, tile, **kw: fake_ms[tile])
+    monkeypatch.setattr(tuner, "_time_launch", lambda launch, tile, **kw: fake_ms.get(tile, 9.0))
     tuner.reset()
     assert tuner.pick(_lib.KERNEL_FWD, 300, 4, 32, torch.bfloat16, lambda t: None) == 1
     assert json.loads((tmp_path / "_fwd_Test-GPU_9-5.json").read_text())["4_32_512_torch.bfloat16"]["tile"] == 1

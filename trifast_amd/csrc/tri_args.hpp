@@ -49,7 +49,8 @@ struct BwdArgs {
   const float* lse;
   const uint32_t* keep;
   const uint32_t* rowflag;
-  float* delta;              // [b*h, n, n] fp32 workspace, indexed [i, j]
+  float* delta;              // [b*h, n, n] fp32 workspace, indexed [i, j]: MINUS rowsum(o * do)
+  float* lse2;               // [b*h, n, n] fp32 workspace: lse * log2(e); log2(n) for fully masked rows
   float* dbpart;             // [nchunks, b*h, n, n] fp32 partial db (nchunks > 1 only)
   void *dq, *dk, *dv, *db;
   Str5 sq, sk, sv, sdo;

@@ -156,7 +156,7 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const float p = fast_exp2(__builtin_fmaf(s[v], c, -lse2[tj]));
-          dbacc[tj][tk][v] = __builtin_fmaf(p, dp[v] - delta[tj], dbacc[tj][tk][v]);
+          dbacc[tj][tk][v] = __builtin_fmaf(p, dp[v] + delta[tj], dbacc[tj][tk][v]);  // the workspace holds -delta
         }
       }
     }

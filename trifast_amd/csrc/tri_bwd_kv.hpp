@@ -184,7 +184,7 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
               const int v = 8 * r2 + 4 * e4 + e;
               const float l2 = flagged[r] ? lse2_flagged : x[e] * kLog2e;
               p[v] = fast_exp2(__builtin_fmaf(sc[v], c, -l2));
-              ds[v] = p[v] * (dp[v] - y[e]);
+              ds[v] = p[v] * (dp[v] + y[e]);  // the workspace holds -delta
             }
           }
         // masked keys (this lane's column) and queries past the end contribute nothing

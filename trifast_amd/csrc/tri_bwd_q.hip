@@ -25,7 +25,7 @@ struct BwdQFamily {
     if constexpr (lds <= kMaxLds && (acc_regs <= 160 || R == 1)) {
       if (dry) return hipSuccess;
       dim3 grid((a.N + NW * 32 - 1) / (NW * 32), ((a.N + R - 1) / R + 7) / 8 * 8, bh);
-      const int lds_total = lds + R * a.nwords * 4;  // + keep words of the R rows
+      const int lds_total = lds + KeyTileMasks::lds_bytes(a.nwords);  // + key-tile bitmaps
       if (lds_total > kMaxLds) return hipErrorInvalidConfiguration;
       return launch_dyn(tri_bwd_q_kernel<T, D, NW, R, BK>, grid, dim3(NW * 64), lds_total, st, a);
     } else {

@@ -8,13 +8,20 @@
 // tile (fp32, raw-score domain) is shared by the R rows as the accumulator init of
 // the score MFMA.  With transposed scores (a lane owns one query) P is recomputed
 // from the saved log-sum-exp,
-//   P^T = exp2(S^T c - lse*log2e),  dP^T = V dO^T,  dS^T = P^T * (dP^T - delta),
+//   P^T = exp2(S^T c - lse*log2e),  dP^T - delta = V dO^T - delta,  dS^T = P^T * (dP^T - delta),
 //   dq^T += K^T dS^T,               dq = dq^T / sqrt(d),
-// with K^T read from the natural K tile through transposing LDS reads.
-// delta is written (fp32) for the dk/dv and db kernels, so this one runs first.
+// with K^T read from the natural K tile through transposing LDS reads.  -delta is
+// the accumulator init of the dP MFMA (16 registers per row that never change),
+// so the subtraction costs nothing.  Masked keys get a large negative score
+// through one extra MFMA (see mask_operand), which makes their P and dS zero.
+//
+// This kernel runs first: it writes -delta and lse*log2e (log2 n for fully
+// masked rows) in fp32 for the dk/dv and db kernels.
 //
 // Replaces _bwd_q of reference src/trifast/triton.py:274-383.
 #pragma once
+#include <type_traits>
+
 #include "tri_args.hpp"
 #include "tri_common.hpp"
 #include "tri_tile.hpp"
@@ -22,7 +29,7 @@
 namespace tri {
 
 template <typename T, int D, int NW, int R, int BK>
-__global__ __launch_bounds__(NW * 64) void tri_bwd_q_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(const BwdArgs a) {
   using E = Elem<T>;
   using frag = typename E::frag;
   using Tile = LdsTile<T, D>;
@@ -32,15 +39,16 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_q_kernel(const BwdArgs a) {
   constexpr int PS = 32 / (2 * KP);
   constexpr int KU = BK / 32;
   constexpr int ROWB = Tile::ROWB;
-  // one stage: K rows of the R pair rows | V rows | packed bias tiles of the NW waves
+  // one stage: K rows of the R pair rows | V rows | packed bias tiles of the NW waves;
+  // two stages, then the key-tile bitmaps
   constexpr int OFF_K = 0, OFF_V = R * BK * ROWB, OFF_B = 2 * R * BK * ROWB;
   constexpr int BIAS_B = 2 * 64 * 8 * (int)sizeof(T);
   constexpr int STAGE = OFF_B + NW * KU * BIAS_B;
   extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
-  uint32_t* keep_s = reinterpret_cast<uint32_t*>(tri_smem + 2 * STAGE);
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int jl = lane & 31, g = lane >> 5;
   const int N = a.N;
   int bx, by;
@@ -53,7 +61,6 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_q_kernel(const BwdArgs a) {
   const int j = j_wave + jl;
   const bool wave_active = j_wave < N;
   const int jt_ld = min(j_wave >> 5, a.NP - 1);
-  constexpr int NT = NW * 64;
 
   const T* qbh = reinterpret_cast<const T*>(a.q) + b * a.sq.b + h * a.sq.h;
   const T* kbh = reinterpret_cast<const T*>(a.k) + b * a.sk.b + h * a.sk.h;
@@ -63,14 +70,18 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_q_kernel(const BwdArgs a) {
 
   // per-row state; a fully masked row drops the q.k and bias terms (all logits equal)
   bool flagged[R];
+  bool any_flagged = false;
+  const uint32_t* keep_row[R];
   frag qf[R][DS], dof[R][DS];
-  float lse2[R], delta[R];
+  float lse2[R];
+  f32x16 ndelta[R];  // -delta in all 16 slots: accumulator init of the dP MFMA
   f32x16 dqacc[R][DM];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int i = min(i0 + r, N - 1);  // rows past the end repeat the last one and are not stored
     flagged[r] = a.rowflag[(int64_t)b * N + i] != 0;
-    for (int w = tid; w < a.nwords; w += NT) keep_s[r * a.nwords + w] = a.keep[((int64_t)b * N + i) * a.nwords + w];
+    any_flagged |= flagged[r];
+    keep_row[r] = a.keep + ((int64_t)b * N + i) * a.nwords;
     const int jc = min(j, N - 1);
     const T* orow = reinterpret_cast<const T*>(a.o) + (((int64_t)bh * N + i) * N + jc) * D;
     float dsum = 0.f;
@@ -88,43 +99,47 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_q_kernel(const BwdArgs a) {
       }
     }
     dsum = half_sum(dsum);
-    delta[r] = dsum;
     lse2[r] = (j >= N) ? 0.f : (flagged[r] ? fast_log2((float)N) : a.lse[((int64_t)bh * N + i) * N + jc] * kLog2e);
-    if (j < N && i0 + r < N && g == 0) a.delta[((int64_t)bh * N + i) * N + j] = dsum;
+    if (j < N && i0 + r < N && g == 0) {
+      a.delta[((int64_t)bh * N + i) * N + j] = -dsum;
+      a.lse2[((int64_t)bh * N + i) * N + j] = lse2[r];
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) ndelta[r][v] = -dsum;
 #pragma unroll
     for (int mt = 0; mt < DM; ++mt) dqacc[r][mt] = zero16();
   }
-
   const float c = a.c;
 
-  auto stage_keep = [&](int kt0, uint32_t (*keepw)[KU]) -> bool {
-    uint32_t any = 0;
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int u = 0; u < KU; ++u) {
-        const int w = kt0 / 32 + u;
-        keepw[r][u] = (w < a.nwords) ? keep_s[r * a.nwords + w] : 0u;
-        any |= keepw[r][u];
-      }
-    return any != 0;
-  };
-  auto next_live = [&](int kt0, uint32_t (*keepw)[KU]) -> int {
-    while (kt0 < N && !stage_keep(kt0, keepw)) kt0 += BK;
-    return kt0;
-  };
+  KeyTileMasks masks;
+  masks.build<R, NW>(reinterpret_cast<uint64_t*>(tri_smem + 2 * STAGE), [&](int r) { return keep_row[r]; }, a.nwords, any_flagged, wave, lane);
 
-  // Stage loads: direct global->LDS, issued unconditionally with clamped indices.
-  // A clamped key row duplicates the last valid one; its keep bit is clear.
+  // lane-constant LDS offsets: K and V rows as natural operands (tile row m stands
+  // for key perm32(m)), K rows again through transposing reads for dq
+  OperandOffsets<T, D> ofs;
+  ofs.init(perm32(jl), lane);
+
+  TileStream<T, D, R * BK, NW> kstream, vstream;
+  kstream.init([&](int x) { return kbh + min(i0 + x / BK, N - 1) * a.sk.i + (int64_t)(x % BK) * a.sk.j; }, wave, lane);
+  vstream.init([&](int x) { return vbh + min(i0 + x / BK, N - 1) * a.sv.i + (int64_t)(x % BK) * a.sv.j; }, wave, lane);
+
+  // Stage loads: direct global->LDS; a ragged last stage clamps key indices (the
+  // duplicated rows have clear keep bits)
+  const T* bias_lane = pack_bh + ((int64_t)jt_ld * a.NP * 2 * 64 + lane) * 8;
   auto issue_loads = [&](int kt0, int buf) {
     unsigned char* st = tri_smem + buf * STAGE;
-    Tile::template fill<R * BK, NW>(st + OFF_K, [&](int x) {
-      return kbh + min(i0 + x / BK, N - 1) * a.sk.i + (int64_t)min(kt0 + x % BK, N - 1) * a.sk.j; }, wave, lane);
-    Tile::template fill<R * BK, NW>(st + OFF_V, [&](int x) {
-      return vbh + min(i0 + x / BK, N - 1) * a.sv.i + (int64_t)min(kt0 + x % BK, N - 1) * a.sv.j; }, wave, lane);
+    if (kt0 + BK <= N) {
+      kstream.issue(st + OFF_K, (int64_t)kt0 * a.sk.j, wave);
+      vstream.issue(st + OFF_V, (int64_t)kt0 * a.sv.j, wave);
+    } else {
+      Tile::template fill<R * BK, NW>(st + OFF_K, [&](int x) {
+        return kbh + min(i0 + x / BK, N - 1) * a.sk.i + (int64_t)min(kt0 + x % BK, N - 1) * a.sk.j; }, wave, lane);
+      Tile::template fill<R * BK, NW>(st + OFF_V, [&](int x) {
+        return vbh + min(i0 + x / BK, N - 1) * a.sv.i + (int64_t)min(kt0 + x % BK, N - 1) * a.sv.j; }, wave, lane);
+    }
 #pragma unroll
     for (int u = 0; u < KU; ++u) {
-      const T* p = pack_bh + (((int64_t)jt_ld * a.NP + min((kt0 >> 5) + u, a.NP - 1)) * 2 * 64 + lane) * 8;
+      const T* p = bias_lane + (int64_t)min((kt0 >> 5) + u, a.NP - 1) * 1024;
 #pragma unroll
       for (int r2 = 0; r2 < 2; ++r2) {
         unsigned char* dst = st + OFF_B + (wave * KU + u) * BIAS_B + r2 * (BIAS_B / 2);
@@ -153,27 +168,48 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_q_kernel(const BwdArgs a) {
     return bv;
   };
 
-  auto compute_stage = [&](int buf, const uint32_t (*kw)[KU]) {
+  // One stage of compute from LDS buffer `buf`, keys kt0 .. kt0+BK-1.  The KU*R
+  // tiles run as a software pipeline inside the wave: the two MFMA chains (scores,
+  // dP) of tile t+1 are issued before the exponentials of tile t.
+  auto compute_stage = [&](auto plain_tag, int kt0, int buf) __attribute__((always_inline)) {
+    constexpr bool PLAIN = decltype(plain_tag)::value;
     const unsigned char* st = tri_smem + buf * STAGE;
-    // The KU*R tiles of the stage run as a software pipeline inside the wave: the
-    // two MFMA chains (scores, dP) of tile t+1 are issued before the exponentials
-    // of tile t.
+    if (!wave_active) return;
     constexpr int TS = KU * R;
+    uint32_t kw[R][KU];
+    if constexpr (!PLAIN) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int u = 0; u < KU; ++u) {
+          const int w = (kt0 >> 5) + u;
+          kw[r][u] = (w < a.nwords) ? keep_row[r][w] : 0u;
+        }
+    }
     f32x16 biasv[KU];
 #pragma unroll
     for (int u = 0; u < KU; ++u) biasv[u] = bias_from_lds(st, u);
 
     auto chains = [&](int t, f32x16& sc, f32x16& dp) {
       const int u = t / R, r = t % R;
-      // key rows as A operands; tile row m stands for key perm32(m)
-      const int row = r * BK + 32 * u + perm32(jl);
-      if (flagged[r]) sc = zero16();
-      else sc = E::mfma(Tile::operand(st + OFF_K, row, 0, g), qf[r][0], biasv[u]);
-      dp = E::mfma(Tile::operand(st + OFF_V, row, 0, g), dof[r][0], zero16());
+      const unsigned char* kt = st + OFF_K + (r * BK + 32 * u) * ROWB;
+      const unsigned char* vt = st + OFF_V + (r * BK + 32 * u) * ROWB;
+      if constexpr (PLAIN) {
+        sc = E::mfma(ofs.natural(kt, 0), qf[r][0], biasv[u]);
+      } else {
+        // a fully masked row has no bias (and a zero Q), but keys past the end of a
+        // ragged last tile stay masked for it too
+        f32x16 init;
+        if (flagged[r]) init = zero16();
+        else init = biasv[u];
+        if (kw[r][u] != 0xffffffffu) init = E::mfma(mask_operand<T>(kw[r][u], perm32(jl)), E::splat(1.0f), init);
+        sc = E::mfma(ofs.natural(kt, 0), qf[r][0], init);
+      }
+      dp = E::mfma(ofs.natural(vt, 0), dof[r][0], ndelta[r]);
 #pragma unroll
       for (int sd = 1; sd < DS; ++sd) {
-        if (!flagged[r]) sc = E::mfma(Tile::operand(st + OFF_K, row, sd, g), qf[r][sd], sc);
-        dp = E::mfma(Tile::operand(st + OFF_V, row, sd, g), dof[r][sd], dp);
+        sc = E::mfma(ofs.natural(kt, sd), qf[r][sd], sc);
+        dp = E::mfma(ofs.natural(vt, sd), dof[r][sd], dp);
       }
     };
 
@@ -184,51 +220,54 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_q_kernel(const BwdArgs a) {
       const int u = t / R, r = t % R;
       f32x16 sn, dn;
       if (t + 1 < TS) chains(t + 1, sn, dn);
-      if (kw[r][u] != 0) {  // a row that attends to no key of this tile has dS = 0
+      bool tile_on = true;  // a row that attends to no key of this tile has dS = 0
+      if constexpr (!PLAIN) tile_on = kw[r][u] != 0;
+      if (tile_on) {
         float ds[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const float p = fast_exp2(__builtin_fmaf(sc[v], c, -lse2[r]));
-          ds[v] = p * (dp[v] - delta[r]);
-        }
-        if (kw[r][u] != 0xffffffffu) {
-          const uint32_t myw = kw[r][u] >> (8 * g);
-#pragma unroll
-          for (int v = 0; v < 16; ++v) ds[v] = ((myw >> (16 * (v / 8) + (v % 8))) & 1u) ? ds[v] : 0.f;
+          ds[v] = p * dp[v];
         }
 #pragma unroll
         for (int s2 = 0; s2 < PS; ++s2) {
           const frag dsf = E::pack(&ds[KP * s2]);
 #pragma unroll
           for (int mt = 0; mt < DM; ++mt)
-            dqacc[r][mt] = E::mfma(Tile::tr_operand(st + OFF_K, r * BK + 32 * u, s2, 32 * mt, D, lane), dsf, dqacc[r][mt]);
+            dqacc[r][mt] = E::mfma(ofs.transposed(st + OFF_K + (r * BK + 32 * u) * ROWB, s2, mt), dsf, dqacc[r][mt]);
         }
       }
       if (t + 1 < TS) { sc = sn; dp = dn; }
     }
   };
 
-  uint32_t keep0[R][KU], keep1[R][KU];
-  __syncthreads();  // keep words visible
-  int kt0 = next_live(0, keep0);
-  issue_loads(min(kt0, N - 1), 0);
-  wait_dma();
-  __syncthreads();
-  while (kt0 < N) {
-    int kt1 = next_live(kt0 + BK, keep1);
-    issue_loads(min(kt1, N - 1), 1);
-    if (wave_active) compute_stage(0, keep0);
+  // Stage loop over the live stages, unrolled by two for the two LDS buffers; a
+  // workgroup whose rows attend to every key runs the loop specialised for it.
+  __syncthreads();  // key-tile bitmaps visible
+  const int ntiles = a.nwords;
+  auto stage_loop = [&](auto plain_tag) __attribute__((always_inline)) {
+    constexpr bool PLAIN = decltype(plain_tag)::value;
+    auto next = [&](int t) { return PLAIN ? min(t, ntiles) : masks.next_live<KU>(t); };
+    int t0 = next(0);
+    issue_loads(min(32 * t0, N - 1), 0);
     wait_dma();
     __syncthreads();
-    if (kt1 >= N) break;
-    kt0 = kt1;
-    kt1 = next_live(kt0 + BK, keep0);
-    issue_loads(min(kt1, N - 1), 0);
-    if (wave_active) compute_stage(1, keep1);
-    wait_dma();
-    __syncthreads();
-    kt0 = kt1;
-  }
+    while (t0 < ntiles) {
+      const int t1 = next(t0 + KU);
+      issue_loads(min(32 * t1, N - 1), 1);
+      compute_stage(plain_tag, 32 * t0, 0);
+      wait_dma();
+      __syncthreads();
+      if (t1 >= ntiles) break;
+      t0 = next(t1 + KU);
+      issue_loads(min(32 * t0, N - 1), 0);
+      compute_stage(plain_tag, 32 * t1, 1);
+      wait_dma();
+      __syncthreads();
+    }
+  };
+  if (masks.all_plain()) stage_loop(std::true_type{});
+  else stage_loop(std::false_type{});
 
   if (!wave_active || j >= N) return;
 #pragma unroll

@@ -129,13 +129,14 @@ float dtype_min(int dtype) {
   }
 }
 
-// workspace layout: keep words | row flags | packq | (backward only) packk | delta | db partials
+// workspace layout: keep words | row flags | packq | (backward only) packk | -delta | lse2 | db partials
 struct Workspace {
   uint32_t* keep;
   uint32_t* rowflag;
   void* packq;
   void* packk;
   float* delta;
+  float* lse2;
   float* dbpart;
   int nwords, np;
 };
@@ -163,6 +164,8 @@ Workspace carve(void* ws, int64_t b, int64_t h, int64_t n, int dtype) {
   w.packk = p;
   p += ws_pack_bytes(b, h, n, dtype);
   w.delta = reinterpret_cast<float*>(p);
+  p += align256(b * h * n * n * 4);
+  w.lse2 = reinterpret_cast<float*>(p);
   p += align256(b * h * n * n * 4);
   w.dbpart = reinterpret_cast<float*>(p);
   w.nwords = (int)nwords;
@@ -296,7 +299,7 @@ int64_t trifast_bwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, 
   (void)d;
   if (b < 1 || h < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
   const int64_t chunks = tri::bwd_b_chunks(n, b * h);
-  return ws_mask_bytes(b, n) + 2 * ws_pack_bytes(b, h, n, dtype) + align256(b * h * n * n * 4) +
+  return ws_mask_bytes(b, n) + 2 * ws_pack_bytes(b, h, n, dtype) + 2 * align256(b * h * n * n * 4) +
          (chunks > 1 ? align256(chunks * b * h * n * n * 4) : 0);
 }
 
@@ -386,7 +389,7 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   a.q = q; a.k = k; a.v = v; a.o = o; a.dout = dout;
   a.packq = w.packq; a.packk = w.packk;
   a.lse = lse;
-  a.keep = w.keep; a.rowflag = w.rowflag; a.delta = w.delta; a.dbpart = w.dbpart;
+  a.keep = w.keep; a.rowflag = w.rowflag; a.delta = w.delta; a.lse2 = w.lse2; a.dbpart = w.dbpart;
   a.BH = (int)(b * h);
   a.nchunks = tri::bwd_b_chunks(n, b * h);
   a.rows_per_chunk = (int)((n + a.nchunks - 1) / a.nchunks);

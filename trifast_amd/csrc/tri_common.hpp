@@ -57,8 +57,16 @@ struct Elem<__bf16> {
   typedef bf16x8 frag;
   typedef bf16x8 vec;
   typedef bf16x4 vec4;
+  // 16 contraction slots of this element sum to a "minus infinity" raw score
+  static constexpr float kMaskElem = -1.0e29f;
   static TRI_DEV f32x16 mfma(frag a, frag b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static TRI_DEV frag splat(float x) {
+    frag f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = (__bf16)x;
+    return f;
   }
   static TRI_DEV frag zero() { return (frag){0, 0, 0, 0, 0, 0, 0, 0}; }
   static TRI_DEV frag pack(const float* x) {
@@ -76,8 +84,16 @@ struct Elem<_Float16> {
   typedef f16x8 frag;
   typedef f16x8 vec;
   typedef f16x4 vec4;
+  // fp16 cannot hold -1e30: 16 slots of -60000 give -9.6e5, far below any raw score
+  static constexpr float kMaskElem = -60000.0f;
   static TRI_DEV f32x16 mfma(frag a, frag b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static TRI_DEV frag splat(float x) {
+    frag f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = (_Float16)x;
+    return f;
   }
   static TRI_DEV frag zero() { return (frag){0, 0, 0, 0, 0, 0, 0, 0}; }
   static TRI_DEV frag pack(const float* x) {
@@ -95,9 +111,11 @@ struct Elem<float> {
   typedef float frag;
   typedef f32x4 vec;
   typedef f32x4 vec4;
+  static constexpr float kMaskElem = -5.0e29f;  // 2 contraction slots
   static TRI_DEV f32x16 mfma(frag a, frag b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
   }
+  static TRI_DEV frag splat(float x) { return x; }
   static TRI_DEV frag zero() { return 0.f; }
   static TRI_DEV frag pack(const float* x) { return x[0]; }
 };

@@ -1,6 +1,6 @@
 // Runtime (dtype, head dim, tile id) -> compile-time instantiation dispatch,
 // shared by the four kernel families.  A family F provides
-//   static constexpr int kNumTiles;                 (at most 4)
+//   static constexpr int kNumTiles;                 (at most 8)
 //   static constexpr int P(int tile, int which);    three ints per tile
 //   template <typename T, int D, int A, int B, int C>
 //   static hipError_t run(const Args&, int bh, hipStream_t, bool dry);
@@ -19,6 +19,10 @@ hipError_t dispatch_tile(const Args& a, int bh, int tile, hipStream_t st, bool d
     case 1: if constexpr (F::kNumTiles > 1) return F::template run<T, D, F::P(1, 0), F::P(1, 1), F::P(1, 2)>(a, bh, st, dry); break;
     case 2: if constexpr (F::kNumTiles > 2) return F::template run<T, D, F::P(2, 0), F::P(2, 1), F::P(2, 2)>(a, bh, st, dry); break;
     case 3: if constexpr (F::kNumTiles > 3) return F::template run<T, D, F::P(3, 0), F::P(3, 1), F::P(3, 2)>(a, bh, st, dry); break;
+    case 4: if constexpr (F::kNumTiles > 4) return F::template run<T, D, F::P(4, 0), F::P(4, 1), F::P(4, 2)>(a, bh, st, dry); break;
+    case 5: if constexpr (F::kNumTiles > 5) return F::template run<T, D, F::P(5, 0), F::P(5, 1), F::P(5, 2)>(a, bh, st, dry); break;
+    case 6: if constexpr (F::kNumTiles > 6) return F::template run<T, D, F::P(6, 0), F::P(6, 1), F::P(6, 2)>(a, bh, st, dry); break;
+    case 7: if constexpr (F::kNumTiles > 7) return F::template run<T, D, F::P(7, 0), F::P(7, 1), F::P(7, 2)>(a, bh, st, dry); break;
   }
   return hipErrorInvalidValue;
 }

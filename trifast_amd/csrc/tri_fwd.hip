@@ -6,7 +6,7 @@ namespace tri {
 namespace {
 
 struct FwdFamily {
-  static constexpr int kNumTiles = 4;
+  static constexpr int kNumTiles = 7;
   // {NW, R, BK}: block of NW*32 queries x R pair rows, K/V streamed BK keys at a time
   static constexpr int P(int tile, int which) {
     constexpr int t[kNumTiles][3] = {
@@ -14,6 +14,9 @@ struct FwdFamily {
         {4, 2, 64},  // 1: 128 queries x 2 rows, 64 keys per stage
         {4, 4, 64},  // 2: 128 queries x 4 rows, 64 keys per stage
         {4, 4, 32},  // 3: 128 queries x 4 rows, 32 keys per stage
+        {4, 2, 32},  // 4: 128 queries x 2 rows, 32 keys per stage (fewer registers: 3 waves per SIMD)
+        {8, 4, 32},  // 5: 256 queries x 4 rows, 32 keys per stage
+        {8, 2, 32},  // 6: 256 queries x 2 rows, 32 keys per stage
     };
     return t[tile][which];
   }
@@ -26,7 +29,7 @@ struct FwdFamily {
     if constexpr (lds <= kMaxLds && (acc_regs <= 160 || R == 1)) {
       if (dry) return hipSuccess;
       dim3 grid((a.N + NW * 32 - 1) / (NW * 32), ((a.N + R - 1) / R + 7) / 8 * 8, bh);
-      const int lds_total = lds + R * a.nwords * 4;  // + keep words of the R rows
+      const int lds_total = lds + KeyTileMasks::lds_bytes(a.nwords);  // + key-tile bitmaps
       if (lds_total > kMaxLds) return hipErrorInvalidConfiguration;
       return launch_dyn(tri_fwd_kernel<T, D, NW, R, BK>, grid, dim3(NW * 64), lds_total, st, a);
     } else {

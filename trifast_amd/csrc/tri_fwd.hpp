@@ -6,8 +6,8 @@
 //   * bias[j, k] does not depend on the row: one packed bias tile (registers) is
 //     reused by the R rows, which divides its L2 traffic by R;
 //   * K[i], V[i] do not depend on the query: they are streamed through LDS in
-//     tiles of BK keys (natural row-major layout, double-buffered) and shared by
-//     the NW waves;
+//     tiles of BK keys (direct global->LDS loads, swizzled, double-buffered) and
+//     shared by the NW waves;
 //   * Q[i, j] and the output accumulator stay in registers for the whole sweep.
 // Scores are computed TRANSPOSED, S^T = K Q^T, so that a lane owns one query
 // (column) and 16 keys of every 32-key tile: the softmax running reference / sum
@@ -19,11 +19,20 @@
 // accumulator init of the score MFMA and is shared by the R rows);
 // p = exp2(acc * c - ref * c) with c = log2(e) / sqrt(d).  `ref` is the running
 // reference of the online softmax: it is raised to the running maximum only when
-// some query of the wave exceeds it by more than kLazy (in log2 units), so the
-// accumulator rescale is rare; p stays below 2^kLazy, which fp32/bf16/fp16 hold.
+// the probabilities of some query of the wave sum to more than 2^kLazy within a
+// tile, so the accumulator rescale is rare and no maximum is searched otherwise;
+// p stays below 2^kLazy, which fp32/bf16/fp16 hold.
+//
+// Masks: a bitmap over the key tiles says which stages are live (others are
+// skipped) and whether all of them are plain (every row attends to every key:
+// the workgroup then runs a loop with no mask work and no per-tile branch).
+// Otherwise a masked key gets a large negative score through one extra MFMA
+// (see mask_operand).
 //
 // Replaces _fwd of reference src/trifast/triton.py:19-132.
 #pragma once
+#include <type_traits>
+
 #include "tri_args.hpp"
 #include "tri_common.hpp"
 #include "tri_tile.hpp"
@@ -31,9 +40,10 @@
 namespace tri {
 
 constexpr float kLazy = 8.0f;
+constexpr float kLazyLimit = 256.0f;  // 2^kLazy
 
 template <typename T, int D, int NW, int R, int BK>
-__global__ __launch_bounds__(NW * 64) void tri_fwd_kernel(const FwdArgs a) {
+__global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd_kernel(const FwdArgs a) {
   using E = Elem<T>;
   using frag = typename E::frag;
   constexpr int KP = E::KP;
@@ -41,21 +51,19 @@ __global__ __launch_bounds__(NW * 64) void tri_fwd_kernel(const FwdArgs a) {
   constexpr int DM = (D + 31) / 32;  // 32-row tiles of O^T
   constexpr int PS = 32 / (2 * KP);  // MFMA steps over a 32-key tile
   constexpr int KU = BK / 32;
-  constexpr int NT = NW * 64;
 
   // One stage: K rows of the R pair rows | V rows | packed bias tiles of the NW waves.
-  // Two stages (double buffer), then the keep words of the R rows.  The tiles are
-  // filled by direct global->LDS loads and read through the swizzle of LdsTile.
+  // Two stages (double buffer), then the key-tile bitmaps.
   using Tile = LdsTile<T, D>;
   constexpr int ROWB = Tile::ROWB;
   constexpr int OFF_K = 0, OFF_V = R * BK * ROWB, OFF_B = 2 * R * BK * ROWB;
   constexpr int BIAS_B = 2 * 64 * 8 * (int)sizeof(T);  // one packed 32 x 32 bias tile
   constexpr int STAGE = OFF_B + NW * KU * BIAS_B;
   extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
-  uint32_t* keep_s = reinterpret_cast<uint32_t*>(tri_smem + 2 * STAGE);
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int jl = lane & 31, g = lane >> 5;
   const int N = a.N;
   int bx, by;
@@ -77,6 +85,8 @@ __global__ __launch_bounds__(NW * 64) void tri_fwd_kernel(const FwdArgs a) {
   // per-row state.  A fully masked row drops the q.k and bias terms (all logits
   // equal): its Q operand is zero and it skips the bias.
   bool flagged[R];
+  bool any_flagged = false;
+  const uint32_t* keep_row[R];
   frag qf[R][DS];
   f32x16 oacc[R][DM];
   float mref[R], mc[R], lrun[R];
@@ -84,7 +94,8 @@ __global__ __launch_bounds__(NW * 64) void tri_fwd_kernel(const FwdArgs a) {
   for (int r = 0; r < R; ++r) {
     const int i = min(i0 + r, N - 1);  // rows past the end repeat the last one and are not stored
     flagged[r] = a.rowflag[(int64_t)b * N + i] != 0;
-    for (int w = tid; w < a.nwords; w += NT) keep_s[r * a.nwords + w] = a.keep[((int64_t)b * N + i) * a.nwords + w];
+    any_flagged |= flagged[r];
+    keep_row[r] = a.keep + ((int64_t)b * N + i) * a.nwords;
 #pragma unroll
     for (int s = 0; s < DS; ++s) {
       if (j < N && !flagged[r])
@@ -98,51 +109,48 @@ __global__ __launch_bounds__(NW * 64) void tri_fwd_kernel(const FwdArgs a) {
 #pragma unroll
     for (int mt = 0; mt < DM; ++mt) oacc[r][mt] = zero16();
   }
-
   const float c = a.c;
 
-  // keep words of the BK keys starting at kt0 for every row; false when no row
-  // attends to any of them (such stages are skipped: their probabilities are zero)
-  auto stage_keep = [&](int kt0, uint32_t (*keepw)[KU]) -> bool {
-    uint32_t any = 0;
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int u = 0; u < KU; ++u) {
-        const int w = kt0 / 32 + u;
-        keepw[r][u] = (w < a.nwords) ? keep_s[r * a.nwords + w] : 0u;
-        any |= keepw[r][u];
-      }
-    return any != 0;
-  };
-  auto next_live = [&](int kt0, uint32_t (*keepw)[KU]) -> int {
-    while (kt0 < N && !stage_keep(kt0, keepw)) kt0 += BK;
-    return kt0;
-  };
+  KeyTileMasks masks;
+  masks.build<R, NW>(reinterpret_cast<uint64_t*>(tri_smem + 2 * STAGE), [&](int r) { return keep_row[r]; }, a.nwords, any_flagged, wave, lane);
 
-  // Stage loads: direct global->LDS, issued unconditionally (indices clamped into
-  // range instead of branching).  A clamped key row duplicates the last valid one;
-  // its keep bit is clear, so it contributes exactly zero.
+  // lane-constant LDS offsets of the operand reads: K rows as natural operands
+  // (tile row m stands for key perm32(m)), V rows through transposing reads
+  OperandOffsets<T, D> ofs;
+  ofs.init(perm32(jl), lane);
+
+  // per-lane source pointers of the K and V stage tiles for keys 0..BK-1
+  TileStream<T, D, R * BK, NW> kstream, vstream;
+  kstream.init([&](int x) { return kbh + min(i0 + x / BK, N - 1) * a.sk.i + (int64_t)(x % BK) * a.sk.j; }, wave, lane);
+  vstream.init([&](int x) { return vbh + min(i0 + x / BK, N - 1) * a.sv.i + (int64_t)(x % BK) * a.sv.j; }, wave, lane);
+
+  // Stage loads: direct global->LDS.  A stage that lies inside the key range adds
+  // one uniform offset to the precomputed pointers; the last, ragged one clamps
+  // key indices instead of branching (a clamped key row duplicates the last valid
+  // one; its keep bit is clear, so it contributes exactly zero).
   const int jt_ld = min(jt, a.NP - 1);
+  const T* bias_lane = pack_bh + ((int64_t)jt_ld * a.NP * 2 * 64 + lane) * 8;
   auto issue_loads = [&](int kt0, int buf) {
     unsigned char* st = tri_smem + buf * STAGE;
-    Tile::template fill<R * BK, NW>(st + OFF_K, [&](int x) {
-      return kbh + min(i0 + x / BK, N - 1) * a.sk.i + (int64_t)min(kt0 + x % BK, N - 1) * a.sk.j; }, wave, lane);
-    Tile::template fill<R * BK, NW>(st + OFF_V, [&](int x) {
-      return vbh + min(i0 + x / BK, N - 1) * a.sv.i + (int64_t)min(kt0 + x % BK, N - 1) * a.sv.j; }, wave, lane);
+    if (kt0 + BK <= N) {
+      kstream.issue(st + OFF_K, (int64_t)kt0 * a.sk.j, wave);
+      vstream.issue(st + OFF_V, (int64_t)kt0 * a.sv.j, wave);
+    } else {
+      Tile::template fill<R * BK, NW>(st + OFF_K, [&](int x) {
+        return kbh + min(i0 + x / BK, N - 1) * a.sk.i + (int64_t)min(kt0 + x % BK, N - 1) * a.sk.j; }, wave, lane);
+      Tile::template fill<R * BK, NW>(st + OFF_V, [&](int x) {
+        return vbh + min(i0 + x / BK, N - 1) * a.sv.i + (int64_t)min(kt0 + x % BK, N - 1) * a.sv.j; }, wave, lane);
+    }
     // each wave fetches the packed bias tiles of its own query tile: 2 x 1 KiB per key tile
 #pragma unroll
     for (int u = 0; u < KU; ++u) {
-      const T* p = pack_bh + (((int64_t)jt_ld * a.NP + min((kt0 >> 5) + u, a.NP - 1)) * 2 * 64 + lane) * 8;
+      const T* p = bias_lane + (int64_t)min((kt0 >> 5) + u, a.NP - 1) * 1024;
 #pragma unroll
       for (int r2 = 0; r2 < 2; ++r2) {
         unsigned char* dst = st + OFF_B + (wave * KU + u) * BIAS_B + r2 * (BIAS_B / 2);
-        if constexpr (sizeof(T) == 2) {
-          __builtin_amdgcn_global_load_lds((const TRI_G1 void*)(p + r2 * 512), (TRI_L3 void*)dst, 16, 0, 0);
-        } else {
-          __builtin_amdgcn_global_load_lds((const TRI_G1 void*)(p + r2 * 512), (TRI_L3 void*)dst, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const TRI_G1 void*)(p + r2 * 512), (TRI_L3 void*)dst, 16, 0, 0);
+        if constexpr (sizeof(T) == 4)
           __builtin_amdgcn_global_load_lds((const TRI_G1 void*)(p + r2 * 512 + 4), (TRI_L3 void*)(dst + 1024), 16, 0, 0);
-        }
       }
     }
   };
@@ -166,138 +174,165 @@ __global__ __launch_bounds__(NW * 64) void tri_fwd_kernel(const FwdArgs a) {
     return bv;
   };
 
-  // one stage of compute from LDS buffer `buf`
-  auto compute_stage = [&](int buf, const uint32_t (*kw)[KU]) {
+  // One stage of compute from LDS buffer `buf`, keys kt0 .. kt0+BK-1.
+  //
+  // The KU*R tiles of the stage run as a software pipeline inside the wave: the
+  // MFMA chain that produces the scores of tile t+1 is issued before the softmax
+  // arithmetic of tile t, so the matrix pipe works on t+1 while the vector ALU
+  // works on t.  K operands are read from LDS two tiles ahead.
+  //
+  // Softmax of a tile: p = exp2(acc * c - ref * c) is computed against the current
+  // reference without looking for the maximum first; only when the rounded
+  // probabilities of some query sum to more than 2^kLazy (which includes the
+  // overflow to +inf of a query that outgrew the reference by a lot, and the very
+  // first tile, whose reference is -1e30) is the reference raised to the running
+  // maximum and the tile recomputed.
+  auto compute_stage = [&](auto plain_tag, int kt0, int buf) __attribute__((always_inline)) {
+    constexpr bool PLAIN = decltype(plain_tag)::value;
     const unsigned char* st = tri_smem + buf * STAGE;
-    if (wave_active) {
-      // The KU*R tiles of the stage run as a software pipeline inside the wave: the
-      // MFMA chain that produces the scores of tile t+1 is issued before the
-      // softmax arithmetic of tile t, so the matrix pipe works on t+1 while the
-      // vector ALU works on t (dependent MFMAs queue in the matrix pipe without
-      // holding up the wave's other instructions).  K operands are read from LDS
-      // two tiles ahead, V^T operands one softmax ahead of their use.
-      constexpr int TS = KU * R;
-      auto k_operand = [&](int t, frag* kf) {
-        const int u = t / R, r = t % R;
+    if (!wave_active) return;
+    constexpr int TS = KU * R;
+    // keep words of the stage's tiles (wave-uniform loads)
+    uint32_t kw[R][KU];
+    if constexpr (!PLAIN) {
 #pragma unroll
-        for (int sd = 0; sd < DS; ++sd) kf[sd] = Tile::operand(st + OFF_K, r * BK + 32 * u + perm32(jl), sd, g);
-      };
-      // The bias tile does not depend on the pair row: it is converted to fp32 in
-      // the raw-score domain once per stage and key tile, and then serves as the
-      // accumulator init (C operand) of the first score MFMA of each of the R rows.
-      f32x16 biasv[KU];
+      for (int r = 0; r < R; ++r)
 #pragma unroll
-      for (int u = 0; u < KU; ++u) biasv[u] = bias_from_lds(buf, u);
-      auto scores = [&](int t, const frag* kf) -> f32x16 {
-        const int u = t / R, r = t % R;
-        f32x16 sc;
-        const bool mixed = kw[r][u] != 0xffffffffu;
-        if (mixed) {
-          sc = mask_tile(kw[r][u], g);
-          if (!flagged[r]) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) sc[v] += biasv[u][v];
-          }
-          sc = E::mfma(kf[0], qf[r][0], sc);
-        } else if (flagged[r]) {
-          sc = E::mfma(kf[0], qf[r][0], zero16());
-        } else {
-          sc = E::mfma(kf[0], qf[r][0], biasv[u]);
+        for (int u = 0; u < KU; ++u) {
+          const int w = (kt0 >> 5) + u;
+          kw[r][u] = (w < a.nwords) ? keep_row[r][w] : 0u;
         }
+    }
+    auto k_operand = [&](int t, frag* kf) {
+      const int u = t / R, r = t % R;
 #pragma unroll
-        for (int sd = 1; sd < DS; ++sd) sc = E::mfma(kf[sd], qf[r][sd], sc);
-        return sc;
-      };
+      for (int sd = 0; sd < DS; ++sd) kf[sd] = ofs.natural(st + OFF_K + (r * BK + 32 * u) * ROWB, sd);
+    };
+    // The bias tile does not depend on the pair row: it is converted to fp32 in
+    // the raw-score domain once per stage and key tile, and then serves as the
+    // accumulator init (C operand) of the first score MFMA of each of the R rows.
+    f32x16 biasv[KU];
+#pragma unroll
+    for (int u = 0; u < KU; ++u) biasv[u] = bias_from_lds(buf, u);
+    auto scores = [&](int t, const frag* kf) -> f32x16 {
+      const int u = t / R, r = t % R;
+      f32x16 sc;
+      if constexpr (PLAIN) {
+        sc = E::mfma(kf[0], qf[r][0], biasv[u]);
+      } else {
+        // a fully masked row has no bias (and a zero Q: all its scores are equal),
+        // but keys past the end of a ragged last tile stay masked for it too
+        f32x16 init;
+        if (flagged[r]) init = zero16();
+        else init = biasv[u];
+        if (kw[r][u] != 0xffffffffu) init = E::mfma(mask_operand<T>(kw[r][u], perm32(jl)), E::splat(1.0f), init);
+        sc = E::mfma(kf[0], qf[r][0], init);
+      }
+#pragma unroll
+      for (int sd = 1; sd < DS; ++sd) sc = E::mfma(kf[sd], qf[r][sd], sc);
+      return sc;
+    };
 
-      frag kf1[DS], kf2[DS];
-      k_operand(0, kf1);
-      if constexpr (TS > 1) k_operand(1, kf2);
-      f32x16 sc = scores(0, kf1);
+    frag kf1[DS], kf2[DS];
+    k_operand(0, kf1);
+    if constexpr (TS > 1) k_operand(1, kf2);
+    f32x16 sc = scores(0, kf1);
 #pragma unroll
-      for (int t = 0; t < TS; ++t) {
-        const int u = t / R, r = t % R;
-        f32x16 sn;
-        if (t + 1 < TS) {
+    for (int t = 0; t < TS; ++t) {
+      const int u = t / R, r = t % R;
+      f32x16 sn;
+      if (t + 1 < TS) {
 #pragma unroll
-          for (int sd = 0; sd < DS; ++sd) kf1[sd] = kf2[sd];
-          if (t + 2 < TS) k_operand(t + 2, kf2);
-          sn = scores(t + 1, kf1);
+        for (int sd = 0; sd < DS; ++sd) kf1[sd] = kf2[sd];
+        if (t + 2 < TS) k_operand(t + 2, kf2);
+        sn = scores(t + 1, kf1);
+      }
+      bool tile_on = true;  // a row that attends to no key of this tile adds nothing
+      if constexpr (!PLAIN) tile_on = kw[r][u] != 0;
+      if (tile_on) {
+        // V^T rows as A operand of the second product
+        frag vf[DM][PS];
+#pragma unroll
+        for (int mt = 0; mt < DM; ++mt)
+#pragma unroll
+          for (int s2 = 0; s2 < PS; ++s2) vf[mt][s2] = ofs.transposed(st + OFF_V + (r * BK + 32 * u) * ROWB, s2, mt);
+        frag pf[PS];
+        float ts = 0.f;
+#pragma unroll
+        for (int s2 = 0; s2 < PS; ++s2) {
+          float p[KP];
+#pragma unroll
+          for (int e = 0; e < KP; ++e) p[e] = fast_exp2(__builtin_fmaf(sc[KP * s2 + e], c, -mc[r]));
+          pf[s2] = E::pack(p);
+          ts = frag_sum(pf[s2], ts);
         }
-        if (kw[r][u] != 0) {  // a row that attends to no key of this tile adds nothing
-          // V^T rows as A operand of the second product
-          frag vf[DM][PS];
+        if (__any(!(ts <= kLazyLimit))) {
+          // some query outgrew the reference: raise it to the running maximum.
+          // (The empty volatile asm keeps the compiler from executing this rare
+          // path speculatively in line with the common one.)
+          asm volatile("" ::);
+          float mx = fmaxf(sc[0], sc[1]);
+#pragma unroll
+          for (int v = 2; v < 16; ++v) mx = fmaxf(mx, sc[v]);
+          mx = half_max(mx);
+          const float mnew = fmaxf(mref[r], mx);
+          const float alpha = fast_exp2((mref[r] - mnew) * c);
+          lrun[r] *= alpha;
 #pragma unroll
           for (int mt = 0; mt < DM; ++mt)
 #pragma unroll
-            for (int s2 = 0; s2 < PS; ++s2) vf[mt][s2] = Tile::tr_operand(st + OFF_V, r * BK + 32 * u, s2, 32 * mt, D, lane);
-          // exponent arguments against the current reference; results of an fma are
-          // canonical floats, so the max below needs no extra canonicalisation
-          float arg[16];
-#pragma unroll
-          for (int v = 0; v < 16; ++v) arg[v] = __builtin_fmaf(sc[v], c, -mc[r]);
-          float amax = fmaxf(arg[0], arg[1]);
-#pragma unroll
-          for (int v = 2; v < 16; v += 2) amax = fmaxf(amax, fmaxf(arg[v], arg[v + 1]));
-          amax = half_max(amax);
-          if (__any(amax > kLazy)) {
-            // some query outgrew the reference: raise it to the running maximum
-            float mx = fmaxf(sc[0], sc[1]);
-#pragma unroll
-            for (int v = 2; v < 16; ++v) mx = fmaxf(mx, sc[v]);
-            mx = half_max(mx);
-            const float mnew = fmaxf(mref[r], mx);
-            const float alpha = fast_exp2((mref[r] - mnew) * c);
-            lrun[r] *= alpha;
-#pragma unroll
-            for (int mt = 0; mt < DM; ++mt)
-#pragma unroll
-              for (int v = 0; v < 16; ++v) oacc[r][mt][v] *= alpha;
-            mref[r] = mnew;
-            mc[r] = mnew * c;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) arg[v] = __builtin_fmaf(sc[v], c, -mc[r]);
-          }
-          float p[16];
-#pragma unroll
-          for (int v = 0; v < 16; ++v) p[v] = fast_exp2(arg[v]);
+            for (int v = 0; v < 16; ++v) oacc[r][mt][v] *= alpha;
+          mref[r] = mnew;
+          mc[r] = mnew * c;
+          ts = 0.f;
 #pragma unroll
           for (int s2 = 0; s2 < PS; ++s2) {
-            const frag pf = E::pack(&p[KP * s2]);
-            lrun[r] = frag_sum(pf, lrun[r]);
+            float p[KP];
 #pragma unroll
-            for (int mt = 0; mt < DM; ++mt) oacc[r][mt] = E::mfma(vf[mt][s2], pf, oacc[r][mt]);
+            for (int e = 0; e < KP; ++e) p[e] = fast_exp2(__builtin_fmaf(sc[KP * s2 + e], c, -mc[r]));
+            pf[s2] = E::pack(p);
+            ts = frag_sum(pf[s2], ts);
           }
         }
-        if (t + 1 < TS) sc = sn;
+        lrun[r] += ts;
+#pragma unroll
+        for (int s2 = 0; s2 < PS; ++s2)
+#pragma unroll
+          for (int mt = 0; mt < DM; ++mt) oacc[r][mt] = E::mfma(vf[mt][s2], pf[s2], oacc[r][mt]);
       }
+      if (t + 1 < TS) sc = sn;
     }
-
   };
-
-  // The stage loop is unrolled by two so that the two sets of keep words swap
-  // roles without being copied.
-  uint32_t keep0[R][KU], keep1[R][KU];
-  __syncthreads();  // keep words visible
-  int kt0 = next_live(0, keep0);
-  issue_loads(min(kt0, N - 1), 0);
-  wait_dma();
-  __syncthreads();
-  while (kt0 < N) {
-    // past the last live stage the prefetch re-reads a valid stage that nobody uses
-    int kt1 = next_live(kt0 + BK, keep1);
-    issue_loads(min(kt1, N - 1), 1);
-    compute_stage(0, keep0);
+  // Stage loop over the live stages, unrolled by two for the two LDS buffers.  A
+  // workgroup whose rows attend to every key runs the loop specialised for plain
+  // stages; any other one runs the general loop for all of its stages (mixing the
+  // two inside one loop would copy the accumulators where the versions meet).
+  __syncthreads();  // key-tile bitmaps visible
+  const int ntiles = a.nwords;
+  auto stage_loop = [&](auto plain_tag) __attribute__((always_inline)) {
+    constexpr bool PLAIN = decltype(plain_tag)::value;
+    auto next = [&](int t) { return PLAIN ? min(t, ntiles) : masks.next_live<KU>(t); };
+    int t0 = next(0);
+    issue_loads(min(32 * t0, N - 1), 0);
     wait_dma();
     __syncthreads();
-    if (kt1 >= N) break;
-    kt0 = kt1;
-    kt1 = next_live(kt0 + BK, keep0);
-    issue_loads(min(kt1, N - 1), 0);
-    compute_stage(1, keep1);
-    wait_dma();
-    __syncthreads();
-    kt0 = kt1;
-  }
+    while (t0 < ntiles) {
+      // past the last live stage the prefetch re-reads a valid stage that nobody uses
+      const int t1 = next(t0 + KU);
+      issue_loads(min(32 * t1, N - 1), 1);
+      compute_stage(plain_tag, 32 * t0, 0);
+      wait_dma();
+      __syncthreads();
+      if (t1 >= ntiles) break;
+      t0 = next(t1 + KU);
+      issue_loads(min(32 * t0, N - 1), 0);
+      compute_stage(plain_tag, 32 * t1, 1);
+      wait_dma();
+      __syncthreads();
+    }
+  };
+  if (masks.all_plain()) stage_loop(std::true_type{});
+  else stage_loop(std::false_type{});
 
   if (!wave_active) return;
 #pragma unroll

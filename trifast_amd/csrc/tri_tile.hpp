@@ -17,29 +17,6 @@ TRI_DEV void xcd_remap(int gx, int& x, int& y) {
   y = 8 * (slot / gx) + xcd;
 }
 
-// Cooperative copy of a [ROWS x D] row-major tile (row stride `stride` elements,
-// rows >= nrows read as zero) into LDS in natural layout.
-template <typename T, int D, int ROWS, int LD, int NT>
-TRI_DEV void lds_load_natural(T (*dst)[LD], const T* src, int64_t stride, int nrows, int tid) {
-  using E = Elem<T>;
-  constexpr int VEC = E::VEC;
-  constexpr int CPR = D / VEC;  // 16-byte chunks per row
-#pragma unroll
-  for (int c0 = 0; c0 < ROWS * CPR; c0 += NT) {
-    const int c = c0 + tid;
-    if ((ROWS * CPR) % NT != 0 && c >= ROWS * CPR) break;
-    const int row = c / CPR, col = (c % CPR) * VEC;
-    typename E::vec val;
-    if (row < nrows) {
-      val = *reinterpret_cast<const typename E::vec*>(src + (int64_t)row * stride + col);
-    } else {
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) val[e] = (T)0.f;
-    }
-    *reinterpret_cast<typename E::vec*>(&dst[row][col]) = val;
-  }
-}
-
 // ---------------------------------------------------------------------------
 // Swizzled LDS tiles filled by direct global->LDS loads.
 //
@@ -113,6 +90,90 @@ struct LdsTile {
   }
 };
 
+// Lane-constant byte offsets of the operand reads of one wave.  Tiles start at
+// rows that are multiples of 32 and MFMA steps move by 16 rows; neither changes
+// the swizzle, so an operand read is (tile base + compile-time offset) + one of
+// these registers.  fp32 operands are single elements with many steps: their
+// offsets are computed where they are used.
+template <typename T, int D>
+struct OperandOffsets {
+  using Tile = LdsTile<T, D>;
+  using frag = typename Elem<T>::frag;
+  static constexpr int KP = Elem<T>::KP;
+  static constexpr int DS = D / (2 * KP);
+  static constexpr int DM = (D + 31) / 32;
+  static constexpr bool PRE = sizeof(T) == 2;
+  int nat[PRE ? DS : 1];
+  int tlo[PRE ? DM : 1], thi[PRE ? DM : 1];
+  int row, lane;
+  // `row_in_tile`: the row of a 32-row tile this lane reads as a natural operand
+  TRI_DEV void init(int row_in_tile, int lane_) {
+    row = row_in_tile;
+    lane = lane_;
+    if constexpr (PRE) {
+      const int g = lane >> 5, L = lane & 15, chalf = (lane >> 4) & 1;
+#pragma unroll
+      for (int s = 0; s < DS; ++s) nat[s] = Tile::off(row, (2 * KP * s + KP * g) * (int)sizeof(T));
+#pragma unroll
+      for (int mt = 0; mt < DM; ++mt) {
+        const int col = 32 * mt + 16 * chalf + 4 * (L & 3);
+        tlo[mt] = Tile::off(8 * g + (L >> 2), col * 2);
+        thi[mt] = Tile::off(8 * g + 4 + (L >> 2), col * 2);
+      }
+    }
+  }
+  // natural operand (head-dim index in-lane), MFMA step s, of the 32-row tile at `tile`
+  TRI_DEV frag natural(const unsigned char* tile, int s) const {
+    if constexpr (PRE) return *reinterpret_cast<const frag*>(tile + nat[s]);
+    else return Tile::operand(tile, row, s, lane >> 5);
+  }
+  // transposed operand (row index in-lane): rows cidx(KP*step.., g), column 32*mt + lane%32
+  TRI_DEV frag transposed(const unsigned char* tile, int step, int mt) const {
+    if constexpr (PRE) {
+      if (D % 32 != 0 && 32 * mt + (lane & 31) >= D) return Elem<T>::zero();
+      const unsigned char* p = tile + 16 * step * Tile::ROWB;
+      const auto lo = lds_tr4(reinterpret_cast<const T*>(p + tlo[mt]));
+      const auto hi = lds_tr4(reinterpret_cast<const T*>(p + thi[mt]));
+      frag f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { f[e] = lo[e]; f[4 + e] = hi[e]; }
+      return f;
+    } else {
+      return Tile::tr_operand(tile, 0, step, 32 * mt, D, lane);
+    }
+  }
+};
+
+// A tile of ROWS rows that is re-filled stage after stage from rows that move
+// along one tensor index: the per-lane source pointers are computed once for
+// position 0 and a stage adds one wave-uniform element offset to them.
+template <typename T, int D, int ROWS, int NW>
+struct TileStream {
+  using Tile = LdsTile<T, D>;
+  static constexpr int GROUPS = ROWS * Tile::CPR / 64;
+  static constexpr int XN = (GROUPS + NW - 1) / NW;
+  static_assert(ROWS * Tile::CPR % 64 == 0, "tile must be a whole number of 1 KiB wave loads");
+  const T* p0[XN];
+  template <typename RowPtr>
+  TRI_DEV void init(RowPtr row_ptr, int wave, int lane) {
+#pragma unroll
+    for (int x = 0; x < XN; ++x) {
+      const int gi = (GROUPS % NW == 0) ? x * NW + wave : min(x * NW + wave, GROUPS - 1);
+      const int p = gi * 64 + lane;
+      const int r = p / Tile::CPR, c = (p % Tile::CPR) ^ Tile::swz(r);
+      p0[x] = row_ptr(r) + c * Tile::VEC;
+    }
+  }
+  TRI_DEV void issue(unsigned char* base, int64_t elem_offset, int wave) const {
+#pragma unroll
+    for (int x = 0; x < XN; ++x) {
+      const int gi = x * NW + wave;
+      if (GROUPS % NW == 0 || gi < GROUPS)
+        __builtin_amdgcn_global_load_lds((const TRI_G1 void*)(p0[x] + elem_offset), (TRI_L3 void*)(base + gi * 1024), 16, 0, 0);
+    }
+  }
+};
+
 // 4-byte-per-lane variant for rows of floats (lse, delta): 64 floats per wave load
 template <int COUNT, int NW, typename Ptr>
 TRI_DEV void fill_floats(float* base, Ptr elem_ptr, int wave, int lane) {
@@ -125,63 +186,6 @@ TRI_DEV void fill_floats(float* base, Ptr elem_ptr, int wave, int lane) {
       __builtin_amdgcn_global_load_lds((const TRI_G1 void*)elem_ptr(gi * 64 + lane), (TRI_L3 void*)(base + gi * 64), 4, 0, 0);
   }
 }
-
-// Two-phase version of the same copy, for software pipelining: the global loads
-// of the next tile are issued into registers before the current tile is computed
-// and written to LDS afterwards.
-template <typename T, int D, int ROWS, int NT>
-struct TileRegs {
-  using vec = typename Elem<T>::vec;
-  static constexpr int VEC = Elem<T>::VEC;
-  static constexpr int CPR = D / VEC;
-  static constexpr int CNT = (ROWS * CPR + NT - 1) / NT;
-  vec v[CNT];
-  TRI_DEV void load(const T* src, int64_t stride, int nrows, int tid) {
-#pragma unroll
-    for (int x = 0; x < CNT; ++x) {
-      const int c = x * NT + tid;
-      const int row = c / CPR, col = (c % CPR) * VEC;
-      if (c < ROWS * CPR && row < nrows) {
-        v[x] = *reinterpret_cast<const vec*>(src + (int64_t)row * stride + col);
-      } else {
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) v[x][e] = (T)0.f;
-      }
-    }
-  }
-  template <int LD>
-  TRI_DEV void store(T (*dst)[LD], int tid) const {
-#pragma unroll
-    for (int x = 0; x < CNT; ++x) {
-      const int c = x * NT + tid;
-      const int row = c / CPR, col = (c % CPR) * VEC;
-      if (c < ROWS * CPR) *reinterpret_cast<vec*>(&dst[row][col]) = v[x];
-    }
-  }
-};
-
-// The packed bias operand of tile (jt, kt) for one lane: 2 x 8 elements.
-template <typename T>
-struct BiasRegs {
-  typename Elem<T>::vec v[2 * (sizeof(T) == 2 ? 1 : 2)];
-  TRI_DEV void load(const T* pack_bh, int NP, int jt, int kt, int lane_q) {
-    const T* p = pack_bh + ((((int64_t)jt * NP + kt) * 2) * 64 + lane_q) * 8;
-    if constexpr (sizeof(T) == 2) {
-      v[0] = *reinterpret_cast<const typename Elem<T>::vec*>(p);
-      v[1] = *reinterpret_cast<const typename Elem<T>::vec*>(p + 512);
-    } else {
-      v[0] = *reinterpret_cast<const f32x4*>(p);
-      v[1] = *reinterpret_cast<const f32x4*>(p + 4);
-      v[2] = *reinterpret_cast<const f32x4*>(p + 512);
-      v[3] = *reinterpret_cast<const f32x4*>(p + 516);
-    }
-  }
-  // element x (0..15) as float
-  TRI_DEV float at(int x) const {
-    if constexpr (sizeof(T) == 2) return (float)v[x / 8][x % 8];
-    else return v[x / 4][x % 4];
-  }
-};
 
 // The 16 bias values of one lane for tile (jt, kt), in the raw-score domain
 // (times sqrt(d)) plus a per-lane additive term, from a packed bias array.
@@ -208,109 +212,97 @@ TRI_DEV f32x16 bias_tile(const T* pack_bh, int NP, int jt, int kt, int lane, flo
   return s;
 }
 
-// The bias enters the raw scores through the matrix pipe rather than the vector
-// ALU: S^T[key, j] += sum_k' (sqrt(d) * I)[key, k'] * bias^T[k', j].  The packed
-// bias tile is the B operand as stored (no conversion); the A operand is the
-// scaled identity, whose row m stands for key perm32(m).  sqrt(d) is split into
-// hi + lo parts of the operand type so the product is exact to ~2^-17 (for d a
-// power of 4 the lo part is zero and is skipped).  fp32 needs no split.
+// Additive key mask through the matrix pipe.  One extra MFMA adds, to every score
+// of a masked key, the sum over all contraction slots of kMaskElem * 1: the
+// operand returned here holds kMaskElem in every slot when key `key_in_tile` of
+// the tile is masked (bit clear in keepw) and zeros otherwise; the other operand
+// is Elem<T>::splat(1).  The lane passes the key its operand row / column stands
+// for.
 template <typename T>
-struct BiasIdentity {
-  using frag = typename Elem<T>::frag;
-  static constexpr int KP = Elem<T>::KP;
-  static constexpr int PS = 32 / (2 * KP);
-  frag hi[PS], lo[PS];
-  bool has_lo;
-  TRI_DEV void init(float sqrt_d, int lane) {
-    const int m = perm32(lane & 31), g = lane >> 5;
-    const T h = (T)sqrt_d;
-    const T l = (T)(sqrt_d - (float)h);
-    has_lo = (float)l != 0.f;
+TRI_DEV typename Elem<T>::frag mask_operand(uint32_t keepw, int key_in_tile) {
+  return ((keepw >> key_in_tile) & 1u) ? Elem<T>::zero() : Elem<T>::splat(Elem<T>::kMaskElem);
+}
+
+// Which 32-key tiles matter to the R pair rows of a workgroup, as bitmaps over
+// the key tiles, one 64-bit word per 64 tiles, built once into LDS:
+//   live  = some row attends to some key of the tile (other tiles are skipped:
+//           their probabilities are exactly zero),
+//   plain = every row attends to every key of the tile (no mask work at all).
+// The words of the 64-tile chunk in use are cached in scalar registers, so the
+// per-stage queries are scalar bit operations.
+struct KeyTileMasks {
+  const uint64_t* words;  // LDS: [nchunks] live, then [nchunks] plain
+  int nchunks, ntiles, cur;
+  uint64_t live, plain;
+
+  static constexpr int lds_bytes(int nwords) { return 16 * ((nwords + 63) / 64); }
+
+  // keep_row(r) = pointer to the keep words of row r.  Every wave calls this; the
+  // caller synchronises the workgroup before the first query.
+  template <int R, int NW, typename KeepRow>
+  TRI_DEV void build(uint64_t* lds, KeepRow keep_row, int nwords, bool force_not_plain, int wave, int lane) {
+    words = lds;
+    ntiles = nwords;
+    nchunks = (nwords + 63) / 64;
+    cur = -1;
+    live = plain = 0;
+    for (int ch = wave; ch < nchunks; ch += NW) {
+      const int w = ch * 64 + lane;
+      uint32_t any = 0, all = 0xffffffffu;
 #pragma unroll
-    for (int s = 0; s < PS; ++s) {
-      if constexpr (KP == 1) {
-        hi[s] = (cidx(s, g) == m) ? sqrt_d : 0.f;
-        lo[s] = 0.f;
-      } else {
-#pragma unroll
-        for (int e = 0; e < KP; ++e) {
-          const bool on = cidx(KP * s + e, g) == m;
-          hi[s][e] = on ? h : (T)0.f;
-          lo[s][e] = on ? l : (T)0.f;
-        }
+      for (int r = 0; r < R; ++r) {
+        const uint32_t x = (w < nwords) ? keep_row(r)[w] : 0u;
+        any |= x;
+        all &= x;
+      }
+      const uint64_t lv = __ballot(any != 0);
+      const uint64_t pl = force_not_plain ? 0 : __ballot(all == 0xffffffffu);
+      if (lane == 0) {
+        lds[ch] = lv;
+        lds[nchunks + ch] = pl;
       }
     }
+  }
+  TRI_DEV void select(int ch) {
+    if (ch == cur) return;
+    cur = ch;
+    const uint64_t lv = words[ch], pl = words[nchunks + ch];
+    live = ((uint64_t)__builtin_amdgcn_readfirstlane((uint32_t)(lv >> 32)) << 32) | __builtin_amdgcn_readfirstlane((uint32_t)lv);
+    plain = ((uint64_t)__builtin_amdgcn_readfirstlane((uint32_t)(pl >> 32)) << 32) | __builtin_amdgcn_readfirstlane((uint32_t)pl);
+  }
+  // first stage of KU tiles at or after tile t (t % KU == 0) with a live tile; ntiles if none
+  template <int KU>
+  TRI_DEV int next_live(int t) {
+    while (t < ntiles) {
+      select(t >> 6);
+      const uint64_t m = live >> (t & 63);
+      if (m != 0) {
+        const int pos = __builtin_ctzll(m);
+        return t + pos - pos % KU;
+      }
+      t = ((t >> 6) + 1) << 6;
+    }
+    return ntiles;
+  }
+  // every key tile is plain (wave-uniform; reads the bitmaps from LDS)
+  TRI_DEV bool all_plain() const {
+    bool all = true;
+    for (int ch = 0; ch < nchunks; ++ch) {
+      const int nt = min(64, ntiles - 64 * ch);
+      const uint64_t want = nt == 64 ? ~0ull : ((1ull << nt) - 1);
+      const uint64_t pl = words[nchunks + ch];
+      const uint64_t u = ((uint64_t)__builtin_amdgcn_readfirstlane((uint32_t)(pl >> 32)) << 32) | __builtin_amdgcn_readfirstlane((uint32_t)pl);
+      all = all && (u & want) == want;
+    }
+    return all;
+  }
+  // every tile of the stage at tile t (in the chunk last selected) is plain
+  template <int KU>
+  TRI_DEV bool stage_plain(int t) const {
+    constexpr uint64_t kMask = (1ull << KU) - 1;
+    return ((plain >> (t & 63)) & kMask) == kMask;
   }
 };
-
-// Adds sqrt(d) * bias tile (jt, kt) to the raw-score accumulator.  `lane_q` is
-// the lane whose packed slot this lane reads: its own in the transposed-score
-// kernels (the bias is the B operand), the row-permuted one in the dk/dv kernel
-// (the bias is the A operand and the identity the B operand).
-template <typename T, bool BIAS_IS_B>
-TRI_DEV f32x16 add_bias_mfma(f32x16 acc, const BiasIdentity<T>& id, const T* pack_bh, int NP, int jt, int kt, int lane_q) {
-  using E = Elem<T>;
-  using frag = typename E::frag;
-  constexpr int KP = E::KP;
-  constexpr int PS = 32 / (2 * KP);
-  const T* p = pack_bh + ((((int64_t)jt * NP + kt) * 2) * 64 + lane_q) * 8;
-  frag bf[PS];
-  if constexpr (KP == 1) {
-#pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      const f32x4 x0 = *reinterpret_cast<const f32x4*>(p + r * 512);
-      const f32x4 x1 = *reinterpret_cast<const f32x4*>(p + r * 512 + 4);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) { bf[8 * r + e] = x0[e]; bf[8 * r + 4 + e] = x1[e]; }
-    }
-  } else {
-#pragma unroll
-    for (int r = 0; r < 2; ++r) bf[r] = *reinterpret_cast<const frag*>(p + r * 512);
-  }
-#pragma unroll
-  for (int s = 0; s < PS; ++s) {
-    if constexpr (BIAS_IS_B) acc = E::mfma(id.hi[s], bf[s], acc);
-    else acc = E::mfma(bf[s], id.hi[s], acc);
-  }
-  if constexpr (KP > 1) {
-    if (id.has_lo) {
-#pragma unroll
-      for (int s = 0; s < PS; ++s) {
-        if constexpr (BIAS_IS_B) acc = E::mfma(id.lo[s], bf[s], acc);
-        else acc = E::mfma(bf[s], id.lo[s], acc);
-      }
-    }
-  }
-  return acc;
-}
-
-// Same, from bias operands already in registers.
-template <typename T, bool BIAS_IS_B>
-TRI_DEV f32x16 add_bias_mfma(f32x16 acc, const BiasIdentity<T>& id, const BiasRegs<T>& b) {
-  using E = Elem<T>;
-  static_assert(E::KP > 1, "the fp32 path adds the bias on the vector ALU");
-#pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    if constexpr (BIAS_IS_B) acc = E::mfma(id.hi[s], b.v[s], acc);
-    else acc = E::mfma(b.v[s], id.hi[s], acc);
-  }
-  if (id.has_lo) {
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      if constexpr (BIAS_IS_B) acc = E::mfma(id.lo[s], b.v[s], acc);
-      else acc = E::mfma(b.v[s], id.lo[s], acc);
-    }
-  }
-  return acc;
-}
-
-template <typename T>
-TRI_DEV f32x16 bias_tile(const BiasRegs<T>& b, float sqrt_d, float add) {
-  f32x16 s;
-#pragma unroll
-  for (int x = 0; x < 16; ++x) s[x] = __builtin_fmaf(b.at(x), sqrt_d, add);
-  return s;
-}
 
 // Additive key mask of one 32-key tile in the transposed-score layout: value v
 // of lane group g is 0 when key cidx(v, g) is attended to and kNeg otherwise.
@@ -320,23 +312,6 @@ TRI_DEV f32x16 mask_tile(uint32_t keepw, int g) {
 #pragma unroll
   for (int v = 0; v < 16; ++v) m[v] = ((myw >> (16 * (v / 8) + (v % 8))) & 1u) ? 0.f : kNeg;
   return m;
-}
-
-// Operand whose contraction index is in-lane, from a natural LDS tile
-// tile[contraction index][column]: 16-bit types use the transposing read, fp32
-// operands are single elements.  `step` is the MFMA step within a 32-wide block
-// of contraction indices starting at row `base`; the lane's column is col0 + lane%32
-// (columns >= ncols read as zero).
-template <typename T, int LD>
-TRI_DEV typename Elem<T>::frag tr_operand(const T (*tile)[LD], int base, int step, int col0, int ncols, int lane) {
-  constexpr int KP = Elem<T>::KP;
-  const int g = lane >> 5;
-  if (col0 + (lane & 31) >= ncols) return Elem<T>::zero();
-  if constexpr (KP == 1) {
-    return tile[base + cidx(step, g)][col0 + (lane & 31)];
-  } else {
-    return lds_tr_frag<T, LD>(tile, base + cidx(KP * step, g), col0, lane);
-  }
 }
 
 // Store a 32-row tile of an [n x D] output held transposed in registers
