@@ -4,17 +4,22 @@
 // owns one tile of 32 keys for all R rows: its K and V rows (B operands) and the
 // dk, dv accumulators stay in registers, and the queries of the rows are streamed
 // through LDS in tiles of BJ (direct global->LDS loads, double-buffered, swizzled;
-// rows of Q and dO, the saved log-sum-exp and delta, and the packed bias tiles).
-// Scores are computed UN-transposed here, S = Q K^T, so that a lane owns one key
-// (column) and 16 queries of every 32-query tile: P and dS are then already in
-// B-operand layout for the two products that contract over queries,
+// rows of Q and dO, lse*log2e and -delta as left by the dq kernel, and the packed
+// bias tiles).  Scores are computed UN-transposed here, S = Q K^T, so that a lane
+// owns one key (column) and 16 queries of every 32-query tile: P and dS are then
+// already in B-operand layout for the two products that contract over queries,
 //   dv^T += dO^T P,   dk^T += Q^T dS,   dk = dk^T / sqrt(d),
 // whose A operands dO^T, Q^T come from the natural tiles through transposing LDS
-// reads.  The bias tile (fp32, raw-score domain) is converted once per stage and
-// shared by the R rows as the accumulator init of the score MFMA.
+// reads.  Two accumulator inits do work for free: the bias tile (fp32, raw-score
+// domain, converted once per stage and shared by the R rows) starts the score
+// MFMA, and the -delta values of the tile's 16 queries start the dP MFMA, so
+// dS = P * (dP - delta) is one multiply.  Masked keys get a large negative score
+// through one extra MFMA (see mask_operand), which makes their P and dS zero.
 //
 // Replaces _bwd_kv of reference src/trifast/triton.py:143-263.
 #pragma once
+#include <type_traits>
+
 #include "tri_args.hpp"
 #include "tri_common.hpp"
 #include "tri_tile.hpp"
@@ -22,7 +27,7 @@
 namespace tri {
 
 template <typename T, int D, int NW, int R, int BJ, int NBUF>
-__global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void tri_bwd_kv_kernel(const BwdArgs a) {
   using E = Elem<T>;
   using frag = typename E::frag;
   using Tile = LdsTile<T, D>;
@@ -32,7 +37,7 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
   constexpr int PS = 32 / (2 * KP);
   constexpr int JU = BJ / 32;
   constexpr int ROWB = Tile::ROWB;
-  // one stage: Q rows of the R pair rows | dO rows | lse | delta | packed bias tiles
+  // one stage: Q rows of the R pair rows | dO rows | lse2 | -delta | packed bias tiles
   constexpr int OFF_Q = 0, OFF_DO = R * BJ * ROWB, OFF_LSE = 2 * R * BJ * ROWB;
   constexpr int OFF_DELTA = OFF_LSE + R * BJ * 4, OFF_B = OFF_DELTA + R * BJ * 4;
   constexpr int BIAS_B = 2 * 64 * 8 * (int)sizeof(T);
@@ -41,7 +46,8 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kl = lane & 31, g = lane >> 5;
   const int N = a.N;
   int bx, by;
@@ -60,12 +66,14 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
   const T* vbh = reinterpret_cast<const T*>(a.v) + b * a.sv.b + h * a.sv.h;
   const T* dobh = reinterpret_cast<const T*>(a.dout) + b * a.sdo.b + h * a.sdo.h;
   const T* pack_bh = reinterpret_cast<const T*>(a.packk) + (int64_t)bh * a.NP * a.NP * 1024;
-  const float* lse_bh = a.lse + (int64_t)bh * N * N;
+  const float* lse2_bh = a.lse2 + (int64_t)bh * N * N;
   const float* delta_bh = a.delta + (int64_t)bh * N * N;
 
-  // per-row state: K and V tiles as B operands (lane owns key k_wave + kl)
-  bool flagged[R], kept[R], tile_live[R], tile_mixed[R];
-  frag kf[R][DS], vf[R][DS];
+  // per-row state: K and V tiles as B operands (lane owns key k_wave + kl).  A
+  // fully masked row drops the q.k and bias terms from its scores: its K operand
+  // is zero here (K itself is not needed for dk, dv) and it skips the bias.
+  bool flagged[R], tile_live[R], tile_mixed[R];
+  frag kf[R][DS], vf[R][DS], maskf[R];
   f32x16 dkacc[R][DM], dvacc[R][DM];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -75,12 +83,12 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
     const uint32_t word = (wave_active && w < a.nwords) ? a.keep[((int64_t)b * N + i) * a.nwords + w] : 0u;
     tile_live[r] = word != 0;
     tile_mixed[r] = word != 0xffffffffu;
-    kept[r] = (word >> kl) & 1u;
+    maskf[r] = mask_operand<T>(word, kl);
 #pragma unroll
     for (int s = 0; s < DS; ++s) {
       const int dofs = 2 * KP * s + KP * g;
       const int kc = min(key, N - 1);
-      kf[r][s] = *reinterpret_cast<const frag*>(kbh + i * a.sk.i + (int64_t)kc * a.sk.j + dofs);
+      kf[r][s] = flagged[r] ? E::zero() : *reinterpret_cast<const frag*>(kbh + i * a.sk.i + (int64_t)kc * a.sk.j + dofs);
       vf[r][s] = *reinterpret_cast<const frag*>(vbh + i * a.sv.i + (int64_t)kc * a.sv.j + dofs);
     }
 #pragma unroll
@@ -90,22 +98,44 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
     }
   }
 
-  // Stage loads: direct global->LDS, issued unconditionally with clamped indices.
-  // A clamped query row duplicates the last valid one (with its dO, lse and
-  // delta); the duplicate's P and dS are zeroed below, so queries >= N add nothing.
+  // lane-constant LDS offsets: Q and dO rows as natural operands (tile row m stands
+  // for query perm32(m)) and again through transposing reads
+  OperandOffsets<T, D> ofs;
+  ofs.init(perm32(kl), lane);
+
+  // per-lane source pointers of the stage tiles for queries 0..BJ-1
+  TileStream<T, D, R * BJ, NW> qstream, dostream;
+  qstream.init([&](int x) { return qbh + min(i0 + x / BJ, N - 1) * a.sq.i + (int64_t)(x % BJ) * a.sq.j; }, wave, lane);
+  dostream.init([&](int x) { return dobh + min(i0 + x / BJ, N - 1) * a.sdo.i + (int64_t)(x % BJ) * a.sdo.j; }, wave, lane);
+  FloatStream<R * BJ, NW> lstream, dstream;
+  lstream.init([&](int x) { return lse2_bh + (int64_t)min(i0 + x / BJ, N - 1) * N + x % BJ; }, wave, lane);
+  dstream.init([&](int x) { return delta_bh + (int64_t)min(i0 + x / BJ, N - 1) * N + x % BJ; }, wave, lane);
+  const T* bias_lane = pack_bh + ((int64_t)kt * 2 * 64 + lane) * 8;
+
+  // Stage loads: direct global->LDS.  A ragged last stage clamps query indices: a
+  // clamped row duplicates the last valid one, and the compute of that stage gives
+  // the duplicates P = dS = 0.
   auto issue_loads = [&](int jt0, int buf) {
     unsigned char* st = tri_smem + buf * STAGE;
-    Tile::template fill<R * BJ, NW>(st + OFF_Q, [&](int x) {
-      return qbh + min(i0 + x / BJ, N - 1) * a.sq.i + (int64_t)min(jt0 + x % BJ, N - 1) * a.sq.j; }, wave, lane);
-    Tile::template fill<R * BJ, NW>(st + OFF_DO, [&](int x) {
-      return dobh + min(i0 + x / BJ, N - 1) * a.sdo.i + (int64_t)min(jt0 + x % BJ, N - 1) * a.sdo.j; }, wave, lane);
-    fill_floats<R * BJ, NW>(reinterpret_cast<float*>(st + OFF_LSE), [&](int x) {
-      return lse_bh + (int64_t)min(i0 + x / BJ, N - 1) * N + min(jt0 + x % BJ, N - 1); }, wave, lane);
-    fill_floats<R * BJ, NW>(reinterpret_cast<float*>(st + OFF_DELTA), [&](int x) {
-      return delta_bh + (int64_t)min(i0 + x / BJ, N - 1) * N + min(jt0 + x % BJ, N - 1); }, wave, lane);
+    if (jt0 + BJ <= N) {
+      qstream.issue(st + OFF_Q, (int64_t)jt0 * a.sq.j, wave);
+      dostream.issue(st + OFF_DO, (int64_t)jt0 * a.sdo.j, wave);
+      lstream.issue(reinterpret_cast<float*>(st + OFF_LSE), jt0, wave);
+      dstream.issue(reinterpret_cast<float*>(st + OFF_DELTA), jt0, wave);
+    } else {
+      asm volatile("" ::);  // keeps this rare path a real branch
+      Tile::template fill<R * BJ, NW>(st + OFF_Q, [&](int x) {
+        return qbh + min(i0 + x / BJ, N - 1) * a.sq.i + (int64_t)min(jt0 + x % BJ, N - 1) * a.sq.j; }, wave, lane);
+      Tile::template fill<R * BJ, NW>(st + OFF_DO, [&](int x) {
+        return dobh + min(i0 + x / BJ, N - 1) * a.sdo.i + (int64_t)min(jt0 + x % BJ, N - 1) * a.sdo.j; }, wave, lane);
+      fill_floats<R * BJ, NW>(reinterpret_cast<float*>(st + OFF_LSE), [&](int x) {
+        return lse2_bh + (int64_t)min(i0 + x / BJ, N - 1) * N + min(jt0 + x % BJ, N - 1); }, wave, lane);
+      fill_floats<R * BJ, NW>(reinterpret_cast<float*>(st + OFF_DELTA), [&](int x) {
+        return delta_bh + (int64_t)min(i0 + x / BJ, N - 1) * N + min(jt0 + x % BJ, N - 1); }, wave, lane);
+    }
 #pragma unroll
     for (int u = 0; u < JU; ++u) {
-      const T* p = pack_bh + (((int64_t)min((jt0 >> 5) + u, a.NP - 1) * a.NP + kt) * 2 * 64 + lane) * 8;
+      const T* p = bias_lane + (int64_t)min((jt0 >> 5) + u, a.NP - 1) * a.NP * 1024;
 #pragma unroll
       for (int r2 = 0; r2 < 2; ++r2) {
         unsigned char* dst = st + OFF_B + (wave * JU + u) * BIAS_B + r2 * (BIAS_B / 2);
@@ -133,15 +163,31 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
     }
     return bv;
   };
+  // the 16 per-query values (lse2 or -delta) of tile (r, u) that this lane's C
+  // layout pairs with its 16 scores: two runs of 8 queries
+  auto query_values = [&](const unsigned char* st, int off, int r, int u) -> f32x16 {
+    const float* src = reinterpret_cast<const float*>(st + off) + r * BJ + 32 * u + 8 * g;
+    f32x16 x;
+#pragma unroll
+    for (int r2 = 0; r2 < 2; ++r2)
+#pragma unroll
+      for (int e4 = 0; e4 < 2; ++e4) {
+        const f32x4 y = *reinterpret_cast<const f32x4*>(src + 16 * r2 + 4 * e4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[8 * r2 + 4 * e4 + e] = y[e];
+      }
+    return x;
+  };
 
   const float c = a.c;
-  const float lse2_flagged = fast_log2((float)N);
 
-  auto compute_stage = [&](int jt0, int buf) {
+  // One stage of compute.  The JU*R tiles run as a software pipeline inside the
+  // wave: the two MFMA chains (scores, dP) of tile t+1 are issued before the
+  // exponentials of tile t.  EDGE stages hold queries past the end.
+  auto compute_stage = [&](auto edge_tag, int jt0, int buf) __attribute__((always_inline)) {
+    constexpr bool EDGE = decltype(edge_tag)::value;
     const unsigned char* st = tri_smem + buf * STAGE;
-    // The JU*R tiles of the stage run as a software pipeline inside the wave: the
-    // two MFMA chains (scores, dP) of tile t+1 are issued before the exponentials
-    // of tile t.
+    if (!wave_active) return;
     constexpr int TS = JU * R;
     f32x16 biasv[JU];
 #pragma unroll
@@ -149,15 +195,25 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
 
     auto chains = [&](int t, f32x16& sc, f32x16& dp) {
       const int u = t / R, r = t % R;
-      // query rows as A operands; tile row m stands for query perm32(m)
-      const int row = r * BJ + 32 * u + perm32(kl);
-      if (flagged[r]) sc = zero16();
-      else sc = E::mfma(Tile::operand(st + OFF_Q, row, 0, g), kf[r][0], biasv[u]);
-      dp = E::mfma(Tile::operand(st + OFF_DO, row, 0, g), vf[r][0], zero16());
+      const unsigned char* qt = st + OFF_Q + (r * BJ + 32 * u) * ROWB;
+      const unsigned char* dot = st + OFF_DO + (r * BJ + 32 * u) * ROWB;
+      if (!flagged[r] && !tile_mixed[r]) {
+        sc = E::mfma(ofs.natural(qt, 0), kf[r][0], biasv[u]);
+      } else {
+        // rare: kept a real branch so that the common case starts from the bias
+        // tile in place (a select between the two inits would copy 16 registers)
+        asm volatile("" ::);
+        f32x16 init;
+        if (flagged[r]) init = zero16();
+        else init = biasv[u];
+        if (tile_mixed[r]) init = E::mfma(E::splat(1.0f), maskf[r], init);
+        sc = E::mfma(ofs.natural(qt, 0), kf[r][0], init);
+      }
+      dp = E::mfma(ofs.natural(dot, 0), vf[r][0], query_values(st, OFF_DELTA, r, u));
 #pragma unroll
       for (int sd = 1; sd < DS; ++sd) {
-        if (!flagged[r]) sc = E::mfma(Tile::operand(st + OFF_Q, row, sd, g), kf[r][sd], sc);
-        dp = E::mfma(Tile::operand(st + OFF_DO, row, sd, g), vf[r][sd], dp);
+        sc = E::mfma(ofs.natural(qt, sd), kf[r][sd], sc);
+        dp = E::mfma(ofs.natural(dot, sd), vf[r][sd], dp);
       }
     };
 
@@ -168,34 +224,18 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
       const int u = t / R, r = t % R;
       f32x16 sn, dn;
       if (t + 1 < TS) chains(t + 1, sn, dn);
-      if (tile_live[r] && jt0 + 32 * u < N) {
-        // per-query statistics of the 16 queries this lane sees: two runs of 8
-        const float* lse_s = reinterpret_cast<const float*>(st + OFF_LSE) + r * BJ + 32 * u;
-        const float* del_s = reinterpret_cast<const float*>(st + OFF_DELTA) + r * BJ + 32 * u;
+      if (tile_live[r] && (!EDGE || jt0 + 32 * u < N)) {
+        f32x16 l2 = query_values(st, OFF_LSE, r, u);
+        if constexpr (EDGE) {
+          // queries past the end: an infinite lse makes their P and dS zero
+#pragma unroll
+          for (int v = 0; v < 16; ++v) l2[v] = (jt0 + 32 * u + cidx(v, g) < N) ? l2[v] : 1.0e30f;
+        }
         float p[16], ds[16];
 #pragma unroll
-        for (int r2 = 0; r2 < 2; ++r2)
-#pragma unroll
-          for (int e4 = 0; e4 < 2; ++e4) {
-            const f32x4 x = *reinterpret_cast<const f32x4*>(lse_s + 16 * r2 + 8 * g + 4 * e4);
-            const f32x4 y = *reinterpret_cast<const f32x4*>(del_s + 16 * r2 + 8 * g + 4 * e4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int v = 8 * r2 + 4 * e4 + e;
-              const float l2 = flagged[r] ? lse2_flagged : x[e] * kLog2e;
-              p[v] = fast_exp2(__builtin_fmaf(sc[v], c, -l2));
-              ds[v] = p[v] * (dp[v] + y[e]);  // the workspace holds -delta
-            }
-          }
-        // masked keys (this lane's column) and queries past the end contribute nothing
-        const bool edge = jt0 + 32 * u + 32 > N;
-        if (tile_mixed[r] || edge) {
-#pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const bool on = kept[r] && (!edge || jt0 + 32 * u + cidx(v, g) < N);
-            p[v] = on ? p[v] : 0.f;
-            ds[v] = on ? ds[v] : 0.f;
-          }
+        for (int v = 0; v < 16; ++v) {
+          p[v] = fast_exp2(__builtin_fmaf(sc[v], c, -l2[v]));
+          ds[v] = p[v] * dp[v];
         }
 #pragma unroll
         for (int s2 = 0; s2 < PS; ++s2) {
@@ -203,8 +243,8 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
           const frag dsf = E::pack(&ds[KP * s2]);
 #pragma unroll
           for (int mt = 0; mt < DM; ++mt) {
-            dvacc[r][mt] = E::mfma(Tile::tr_operand(st + OFF_DO, r * BJ + 32 * u, s2, 32 * mt, D, lane), pf, dvacc[r][mt]);
-            dkacc[r][mt] = E::mfma(Tile::tr_operand(st + OFF_Q, r * BJ + 32 * u, s2, 32 * mt, D, lane), dsf, dkacc[r][mt]);
+            dvacc[r][mt] = E::mfma(ofs.transposed(st + OFF_DO + (r * BJ + 32 * u) * ROWB, s2, mt), pf, dvacc[r][mt]);
+            dkacc[r][mt] = E::mfma(ofs.transposed(st + OFF_Q + (r * BJ + 32 * u) * ROWB, s2, mt), dsf, dkacc[r][mt]);
           }
         }
       }
@@ -212,29 +252,51 @@ __global__ __launch_bounds__(NW * 64) void tri_bwd_kv_kernel(const BwdArgs a) {
     }
   };
 
+  // Stages that lie inside the query range run in the main loop; a ragged last
+  // stage runs after it with the edge handling.
+  const int nfull = N / BJ;  // whole stages
+  const bool ragged = N % BJ != 0;
   if constexpr (NBUF == 2) {
     issue_loads(0, 0);
     wait_dma();
     __syncthreads();
-    for (int jt0 = 0; jt0 < N; jt0 += 2 * BJ) {
-      issue_loads(min(jt0 + BJ, N - 1), 1);
-      if (wave_active) compute_stage(jt0, 0);
+    int s = 0;
+    for (; s + 1 < nfull; s += 2) {
+      issue_loads((s + 1) * BJ, 1);
+      compute_stage(std::false_type{}, s * BJ, 0);
       wait_dma();
       __syncthreads();
-      if (jt0 + BJ >= N) break;
-      issue_loads(min(jt0 + 2 * BJ, N - 1), 0);
-      if (wave_active) compute_stage(jt0 + BJ, 1);
+      if ((s + 2) * BJ < N) issue_loads((s + 2) * BJ, 0);
+      compute_stage(std::false_type{}, (s + 1) * BJ, 1);
       wait_dma();
       __syncthreads();
     }
+    // buffer 0 now holds stage s: the last whole one, the ragged one, or a spare
+    if (s < nfull) {
+      if (ragged) issue_loads((s + 1) * BJ, 1);
+      compute_stage(std::false_type{}, s * BJ, 0);
+      if (ragged) {
+        wait_dma();
+        __syncthreads();
+        compute_stage(std::true_type{}, (s + 1) * BJ, 1);
+      }
+    } else if (ragged) {
+      compute_stage(std::true_type{}, s * BJ, 0);
+    }
   } else {
     // one stage only (the double buffer does not fit in LDS): load, then compute
-    for (int jt0 = 0; jt0 < N; jt0 += BJ) {
-      issue_loads(jt0, 0);
+    for (int s = 0; s < nfull; ++s) {
+      issue_loads(s * BJ, 0);
       wait_dma();
       __syncthreads();
-      if (wave_active) compute_stage(jt0, 0);
+      compute_stage(std::false_type{}, s * BJ, 0);
       __syncthreads();
+    }
+    if (ragged) {
+      issue_loads(nfull * BJ, 0);
+      wait_dma();
+      __syncthreads();
+      compute_stage(std::true_type{}, nfull * BJ, 0);
     }
   }
 

@@ -136,6 +136,7 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
       kstream.issue(st + OFF_K, (int64_t)kt0 * a.sk.j, wave);
       vstream.issue(st + OFF_V, (int64_t)kt0 * a.sv.j, wave);
     } else {
+      asm volatile("" ::);  // keeps this rare path a real branch (no speculation into the common one)
       Tile::template fill<R * BK, NW>(st + OFF_K, [&](int x) {
         return kbh + min(i0 + x / BK, N - 1) * a.sk.i + (int64_t)min(kt0 + x % BK, N - 1) * a.sk.j; }, wave, lane);
       Tile::template fill<R * BK, NW>(st + OFF_V, [&](int x) {

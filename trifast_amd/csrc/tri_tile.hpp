@@ -165,6 +165,11 @@ struct TileStream {
     }
   }
   TRI_DEV void issue(unsigned char* base, int64_t elem_offset, int wave) const {
+    // the offset is wave-uniform: pin it to scalar registers so that a stage costs
+    // one 64-bit add per load
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)elem_offset);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)elem_offset >> 32));
+    elem_offset = (int64_t)(((uint64_t)hi << 32) | lo);
 #pragma unroll
     for (int x = 0; x < XN; ++x) {
       const int gi = x * NW + wave;
@@ -186,6 +191,34 @@ TRI_DEV void fill_floats(float* base, Ptr elem_ptr, int wave, int lane) {
       __builtin_amdgcn_global_load_lds((const TRI_G1 void*)elem_ptr(gi * 64 + lane), (TRI_L3 void*)(base + gi * 64), 4, 0, 0);
   }
 }
+
+// The same for COUNT floats that move along one index (lse, delta of a query tile).
+template <int COUNT, int NW>
+struct FloatStream {
+  static constexpr int GROUPS = COUNT / 64;
+  static constexpr int XN = (GROUPS + NW - 1) / NW;
+  static_assert(COUNT % 64 == 0, "whole wave loads only");
+  const float* p0[XN];
+  template <typename Ptr>
+  TRI_DEV void init(Ptr elem_ptr, int wave, int lane) {
+#pragma unroll
+    for (int x = 0; x < XN; ++x) {
+      const int gi = (GROUPS % NW == 0) ? x * NW + wave : min(x * NW + wave, GROUPS - 1);
+      p0[x] = elem_ptr(gi * 64 + lane);
+    }
+  }
+  TRI_DEV void issue(float* base, int64_t elem_offset, int wave) const {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)elem_offset);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)elem_offset >> 32));
+    elem_offset = (int64_t)(((uint64_t)hi << 32) | lo);
+#pragma unroll
+    for (int x = 0; x < XN; ++x) {
+      const int gi = x * NW + wave;
+      if (GROUPS % NW == 0 || gi < GROUPS)
+        __builtin_amdgcn_global_load_lds((const TRI_G1 void*)(p0[x] + elem_offset), (TRI_L3 void*)(base + gi * 64), 4, 0, 0);
+    }
+  }
+};
 
 // The 16 bias values of one lane for tile (jt, kt), in the raw-score domain
 // (times sqrt(d)) plus a per-lane additive term, from a packed bias array.
