@@ -104,7 +104,7 @@ def test_every_tile(n, h, d, dtype, monkeypatch):
     ref = orc.forward_backward(*(t.float() for t in low), m, do.to(dtype).float())
     pt = orc.forward_backward(*low, m, do.to(dtype))
     ran = 0
-    for tile in range(4):
+    for tile in range(8):
         tiles = {kern: tile if lib.trifast_supports(kern, tile, n, h, d, code) else None for kern in range(4)}
         if all(t is None for t in tiles.values()):
             continue

@@ -6,33 +6,36 @@ namespace tri {
 namespace {
 
 struct BwdBFamily {
-  static constexpr int kNumTiles = 3;
-  // {WJ, WK, unused}: each wave owns WJ x WK tiles of 32 x 32; 2 x 2 waves per workgroup
+  static constexpr int kNumTiles = 6;
+  // {WJ, WK, 16 * GJ + GK}: GJ x GK waves per workgroup, each owning WJ x WK tiles of 32 x 32
   static constexpr int P(int tile, int which) {
     constexpr int t[kNumTiles][3] = {
-        {2, 2, 0},  // 0: 128 queries x 128 keys per workgroup
-        {1, 2, 0},  // 1:  64 queries x 128 keys
-        {1, 1, 0},  // 2:  64 queries x  64 keys
+        {2, 2, 16 * 2 + 2},  // 0: 128 queries x 128 keys,  4 waves
+        {1, 2, 16 * 2 + 2},  // 1:  64 queries x 128 keys,  4 waves
+        {1, 1, 16 * 2 + 2},  // 2:  64 queries x  64 keys,  4 waves (fits every dtype / head dim)
+        {1, 2, 16 * 4 + 2},  // 3: 128 queries x 128 keys,  8 waves
+        {1, 1, 16 * 4 + 4},  // 4: 128 queries x 128 keys, 16 waves
+        {2, 2, 16 * 4 + 2},  // 5: 256 queries x 128 keys,  8 waves
     };
     return t[tile][which];
   }
-  template <typename T, int D, int WJ, int WK>
-  static constexpr int stage_bytes() {
-    return (2 * 2 * WJ * 32 + 2 * 2 * WK * 32) * D * (int)sizeof(T) + 2 * (2 * WJ * 32) * 4 + 256;
-  }
-  template <typename T, int D, int WJ, int WK, int>
+  template <typename T, int D, int WJ, int WK, int G>
   static hipError_t run(const BwdArgs& a, int bh, hipStream_t st, bool dry) {
+    constexpr int GJ = G / 16, GK = G % 16;
+    constexpr int BJ = GJ * WJ * 32, BKB = GK * WK * 32;
     // registers of one row's operands, the db accumulators and the bias tiles
     constexpr int frag_regs = (2 * WJ + 2 * WK) * (D / 2) * (int)sizeof(T) / 4;
-    constexpr int stage = stage_bytes<T, D, WJ, WK>();
-    constexpr int nbuf = 2 * stage <= kMaxLds ? 2 : 1;
+    constexpr int stage = (2 * BJ + 2 * BKB) * D * (int)sizeof(T) + 2 * BJ * 4 + 256;
+    // ring of row buffers: up to 4 (loads run 3 rows ahead), as many as fit
+    constexpr int nbuf = 4 * stage <= kMaxLds ? 4 : (3 * stage <= kMaxLds ? 3 : (2 * stage <= kMaxLds ? 2 : 1));
     // the smallest tile always runs (at the price of register spills for large head dims)
-    constexpr bool fits = stage <= kMaxLds && (2 * WJ * WK * 16 + frag_regs <= 320 || WJ * WK == 1);
+    constexpr bool fits = stage <= kMaxLds && (2 * WJ * WK * 16 + frag_regs <= 320 || (WJ * WK == 1 && GJ * GK == 4));
     if constexpr (fits) {
       if (dry) return hipSuccess;
       const int lds = nbuf * stage;
-      dim3 grid((a.N + 2 * WJ * 32 - 1) / (2 * WJ * 32), (a.N + 2 * WK * 32 - 1) / (2 * WK * 32), bh * a.nchunks);
-      hipError_t e = launch_dyn(tri_bwd_b_kernel<T, D, WJ, WK, nbuf>, grid, dim3(256), lds, st, a);
+      const int groups = bh * a.nchunks;
+      dim3 grid((a.N + BJ - 1) / BJ, (a.N + BKB - 1) / BKB, (groups + 7) / 8 * 8);
+      hipError_t e = launch_dyn(tri_bwd_b_kernel<T, D, GJ, GK, WJ, WK, nbuf>, grid, dim3(GJ * GK * 64), lds, st, a);
       if (e != hipSuccess || a.nchunks == 1) return e;
       const int64_t count = (int64_t)bh * a.N * a.N;
       hipLaunchKernelGGL(tri_bwd_b_reduce_kernel<T>, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st,
@@ -49,7 +52,8 @@ struct BwdBFamily {
 int bwd_b_num_tiles() { return BwdBFamily::kNumTiles; }
 
 TileInfo bwd_b_tile_info(int tile) {
-  return TileInfo{2 * BwdBFamily::P(tile, 0) * 32, 2 * BwdBFamily::P(tile, 1) * 32, 4};
+  const int gj = BwdBFamily::P(tile, 2) / 16, gk = BwdBFamily::P(tile, 2) % 16;
+  return TileInfo{gj * BwdBFamily::P(tile, 0) * 32, gk * BwdBFamily::P(tile, 1) * 32, gj * gk};
 }
 
 bool bwd_b_supports(int tile, int64_t n, int d, int dtype) {

@@ -1,54 +1,78 @@
 // Backward kernel 3 of 3: db[j, k] = sum over rows i of dS[i, j, k].
 //
-// Work unit: (batch*head, block of 2*WJ*32 queries j, block of 2*WK*32 keys k,
-// chunk of pair rows i).  The 2 x 2 waves of a workgroup each own WJ x WK tiles of
-// 32 x 32 and keep their db tiles in fp32 registers while the workgroup walks its
-// rows, so the reduction over i has one fixed order and needs no atomics.  The
-// bias tiles (register-resident, fp32, raw-score domain) are the accumulator init
-// of the score MFMA of every row.  Per row the workgroup stages the Q, dO rows of
-// its queries and the K, V rows of its keys in LDS (direct global->LDS loads,
-// double-buffered, swizzled), and each wave recomputes for its tiles
-//   S^T = K Q^T (+bias), P^T = exp2(S^T c - lse), dP^T = V dO^T, dS^T = P^T (dP^T - delta)
-// with every operand in its natural row-major layout, adding dS^T into db.
-// When the rows are split into several chunks (to fill the GPU at small n), each
-// chunk writes an fp32 partial and a second kernel adds the partials in order.
+// Work unit: (batch*head, chunk of pair rows i, block of GJ*WJ*32 queries j, block
+// of GK*WK*32 keys k).  The GJ x GK waves of a workgroup each own WJ x WK tiles of
+// 32 x 32 and keep their db tiles in fp32 registers while the workgroup walks the
+// rows of its chunk, so the reduction over i has one fixed order and needs no
+// atomics.  Per row the workgroup stages the Q, dO rows of its queries and the K,
+// V rows of its keys in LDS (direct global->LDS loads into a ring of row buffers
+// that runs several rows ahead of the compute, swizzled tiles) together with
+// lse*log2e and -delta as left by the dq kernel, and each wave
+// recomputes for its tiles
+//   S^T = K Q^T (+bias), P^T = exp2(S^T c - lse2), dP^T = V dO^T, dS^T = P^T (dP^T - delta)
+// with every operand in its natural row-major layout: a lane owns one query
+// (column) and 16 keys of each tile, so lse2 and delta are per-lane scalars.  (The
+// other orientation would take -delta and lse2 as 16 values per lane from LDS,
+// which costs more LDS bandwidth than this kernel has to spare: every row brings
+// fresh Q, dO, K, V operands.)  The bias tiles (register-resident, fp32, raw-score
+// domain) are the accumulator init of every row's score MFMA.  Masked keys get a
+// large negative score through one extra MFMA (see mask_operand).
+//
+// All workgroups of one (batch*head, chunk) read the same rows at about the same
+// time; the block index is remapped so that they run on one XCD and share its L2.
+// When the rows are split into several chunks (to fill the GPU), each chunk writes
+// an fp32 partial and a second kernel adds the partials in chunk order.
 //
 // Replaces _bwd_b of reference src/trifast/triton.py:394-501.
 #pragma once
+#include <type_traits>
+
 #include "tri_args.hpp"
 #include "tri_common.hpp"
 #include "tri_tile.hpp"
 
 namespace tri {
 
-template <typename T, int D, int WJ, int WK, int NBUF>
-__global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
+template <typename T, int D, int GJ, int GK, int WJ, int WK, int NBUF>
+__global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a) {
   using E = Elem<T>;
   using frag = typename E::frag;
   using Tile = LdsTile<T, D>;
   constexpr int KP = E::KP;
   constexpr int DS = D / (2 * KP);
-  constexpr int NW = 4;
-  constexpr int BJ = 2 * WJ * 32, BKB = 2 * WK * 32;  // queries / keys per workgroup
+  constexpr int NW = GJ * GK;
+  constexpr int BJ = GJ * WJ * 32, BKB = GK * WK * 32;  // queries / keys per workgroup
   constexpr int ROWB = Tile::ROWB;
-  // one stage: Q rows | dO rows | K rows | V rows | lse[BJ] | delta[BJ] | row meta
+  // one stage: Q rows | dO rows | K rows | V rows | lse2[BJ] | -delta[BJ] | row meta
   // (64 words: the WKW keep words of the key block, then the row's flag)
   constexpr int OFF_Q = 0, OFF_DO = BJ * ROWB, OFF_K = 2 * BJ * ROWB, OFF_V = OFF_K + BKB * ROWB;
   constexpr int OFF_LSE = OFF_V + BKB * ROWB, OFF_DELTA = OFF_LSE + BJ * 4;
   constexpr int OFF_META = OFF_DELTA + BJ * 4;
   constexpr int STAGE = OFF_META + 256;
   constexpr int WKW = BKB / 32;
+  static_assert(WKW < 64, "keep words and the row flag share one 64-lane load");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int jl = lane & 31, g = lane >> 5;
   const int N = a.N;
-  const int bh = blockIdx.z % a.BH, chunk = blockIdx.z / a.BH;
+
+  // Linear block id L = 8 * slot + xcd (workgroups go to the 8 XCDs round-robin).
+  // Every XCD walks its own sequence of (batch*head, chunk) groups; the launcher
+  // pads the group count to a multiple of 8.
+  const int per_group = gridDim.x * gridDim.y;
+  const int L = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const int slot = L >> 3;
+  const int group = 8 * (slot / per_group) + (L & 7);
+  if (group >= a.BH * a.nchunks) return;
+  const int within = slot % per_group;
+  const int bh = group % a.BH, chunk = group / a.BH;
   const int b = bh / a.H, h = bh % a.H;
-  const int j_blk = blockIdx.x * BJ, k_blk = blockIdx.y * BKB;
-  const int wj = wave & 1, wk = wave >> 1;
+  const int j_blk = (within % gridDim.x) * BJ, k_blk = (within / gridDim.x) * BKB;
+  const int wj = wave % GJ, wk = wave / GJ;
   const int j_wave = j_blk + wj * (WJ * 32), k_wave = k_blk + wk * (WK * 32);
   const int i_begin = chunk * a.rows_per_chunk;
   const int i_end = min(N, i_begin + a.rows_per_chunk);
@@ -59,7 +83,7 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
   const T* vbase = reinterpret_cast<const T*>(a.v) + b * a.sv.b + h * a.sv.h;
   const T* dobase = reinterpret_cast<const T*>(a.dout) + b * a.sdo.b + h * a.sdo.h;
   const T* pack_bh = reinterpret_cast<const T*>(a.packq) + (int64_t)bh * a.NP * a.NP * 1024;
-  const float* lse_bh = a.lse + (int64_t)bh * N * N;
+  const float* lse2_bh = a.lse2 + (int64_t)bh * N * N;
   const float* delta_bh = a.delta + (int64_t)bh * N * N;
 
   // bias tiles in the raw-score domain: accumulator init of every row's score MFMA
@@ -76,120 +100,189 @@ __global__ __launch_bounds__(256) void tri_bwd_b_kernel(const BwdArgs a) {
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk) dbacc[tj][tk] = zero16();
 
-  // issue the loads of row i into stage buffer `buf` (indices clamped, never branched)
-  auto issue_row = [&](int i, int buf) {
+  // The loads of one row, as a flat list of wave-sized items: 1 KiB pieces of the Q,
+  // dO, K, V tiles (16 bytes per lane), 64-float pieces of lse2 and -delta, and the
+  // 64-word row meta (4 bytes per lane).  Wave w takes items w, w + NW, ...; every
+  // wave issues exactly XN loads per row (a wave that runs out repeats the last
+  // item, which rewrites the same bytes), so "all but the newest K rows have
+  // landed" is one s_waitcnt vmcnt(K * XN) for every wave.  Queries and keys past
+  // the end are clamped (they feed db entries that are never stored).
+  constexpr int CPR = Tile::CPR;
+  constexpr int GQ = BJ * CPR / 64, GKK = BKB * CPR / 64, GF = BJ / 64;
+  constexpr int TOT = 2 * GQ + 2 * GKK + 2 * GF + 1;
+  constexpr int XN = (TOT + NW - 1) / NW;
+  static_assert(BJ * CPR % 64 == 0 && BKB * CPR % 64 == 0 && BJ % 64 == 0, "whole wave loads only");
+  const char* item_ptr[XN];   // source of the next row to load (per lane)
+  int64_t item_step[XN];      // bytes from one pair row to the next (per lane: the meta item mixes two arrays)
+  int item_lds[XN];           // destination offset inside a stage (wave-uniform)
+  bool item_wide[XN];         // 16-byte (tile) or 4-byte (float / meta) lanes
+  {
+    const int es = (int)sizeof(T);
+    auto tile_item = [&](int x, int gi, const T* base, int64_t srow, int64_t si, int blk, int off) {
+      const int p = gi * 64 + lane;
+      const int r = p / CPR, cc = (p % CPR) ^ Tile::swz(r);
+      item_ptr[x] = reinterpret_cast<const char*>(base + (int64_t)min(blk + r, N - 1) * srow + cc * Tile::VEC) + (int64_t)i_begin * si * es;
+      item_step[x] = si * es;
+      item_lds[x] = off + gi * 1024;
+      item_wide[x] = true;
+    };
+#pragma unroll
+    for (int x = 0; x < XN; ++x) {
+      int it = __builtin_amdgcn_readfirstlane(min(x * NW + wave, TOT - 1));
+      if (it < GQ) {
+        tile_item(x, it, qbase, a.sq.j, a.sq.i, j_blk, OFF_Q);
+      } else if (it < 2 * GQ) {
+        tile_item(x, it - GQ, dobase, a.sdo.j, a.sdo.i, j_blk, OFF_DO);
+      } else if (it < 2 * GQ + GKK) {
+        tile_item(x, it - 2 * GQ, kbase, a.sk.j, a.sk.i, k_blk, OFF_K);
+      } else if (it < 2 * GQ + 2 * GKK) {
+        tile_item(x, it - 2 * GQ - GKK, vbase, a.sv.j, a.sv.i, k_blk, OFF_V);
+      } else if (it < 2 * GQ + 2 * GKK + 2 * GF) {
+        const int f = it - 2 * GQ - 2 * GKK;
+        const int gi = f % GF;
+        const float* base = (f < GF) ? lse2_bh : delta_bh;
+        item_ptr[x] = reinterpret_cast<const char*>(base + (int64_t)i_begin * N + min(j_blk + gi * 64 + lane, N - 1));
+        item_step[x] = (int64_t)N * 4;
+        item_lds[x] = ((f < GF) ? OFF_LSE : OFF_DELTA) + gi * 256;
+        item_wide[x] = false;
+      } else {
+        // lanes 0..WKW-1: keep words of this key block; lane WKW (and up): the row flag
+        const bool is_flag = lane >= WKW;
+        const uint32_t* src = is_flag ? a.rowflag + (int64_t)b * N + i_begin
+                                      : a.keep + ((int64_t)b * N + i_begin) * a.nwords + min(k_blk / 32 + lane, a.nwords - 1);
+        item_ptr[x] = reinterpret_cast<const char*>(src);
+        item_step[x] = is_flag ? 4 : (int64_t)a.nwords * 4;
+        item_lds[x] = OFF_META;
+        item_wide[x] = false;
+      }
+    }
+  }
+  // issue the loads of the next row into stage buffer `buf`; past the last row of
+  // the chunk the pointers stop and the last row is loaded again (never used)
+  int rows_issued = 0;
+  auto issue_row = [&](int buf) {
     unsigned char* st = tri_smem + buf * STAGE;
-    i = min(i, N - 1);
-    Tile::template fill<BJ, NW>(st + OFF_Q, [&](int r) { return qbase + i * a.sq.i + (int64_t)min(j_blk + r, N - 1) * a.sq.j; }, wave, lane);
-    Tile::template fill<BJ, NW>(st + OFF_DO, [&](int r) { return dobase + i * a.sdo.i + (int64_t)min(j_blk + r, N - 1) * a.sdo.j; }, wave, lane);
-    Tile::template fill<BKB, NW>(st + OFF_K, [&](int r) { return kbase + i * a.sk.i + (int64_t)min(k_blk + r, N - 1) * a.sk.j; }, wave, lane);
-    Tile::template fill<BKB, NW>(st + OFF_V, [&](int r) { return vbase + i * a.sv.i + (int64_t)min(k_blk + r, N - 1) * a.sv.j; }, wave, lane);
-    fill_floats<BJ, NW>(reinterpret_cast<float*>(st + OFF_LSE), [&](int x) { return lse_bh + (int64_t)i * N + min(j_blk + x, N - 1); }, wave, lane);
-    fill_floats<BJ, NW>(reinterpret_cast<float*>(st + OFF_DELTA), [&](int x) { return delta_bh + (int64_t)i * N + min(j_blk + x, N - 1); }, wave, lane);
-    if (wave == NW - 1) {
-      // lanes 0..WKW-1: keep words of this key block; lane WKW: the row flag
-      const uint32_t* src = (lane == WKW) ? a.rowflag + (int64_t)b * N + i
-                                          : a.keep + ((int64_t)b * N + i) * a.nwords + min(k_blk / 32 + min(lane, WKW - 1), a.nwords - 1);
-      __builtin_amdgcn_global_load_lds((const TRI_G1 void*)src, (TRI_L3 void*)(st + OFF_META), 4, 0, 0);
+    const bool advance = rows_issued + 1 < nrows;
+    ++rows_issued;
+#pragma unroll
+    for (int x = 0; x < XN; ++x) {
+      if (item_wide[x]) __builtin_amdgcn_global_load_lds((const TRI_G1 void*)item_ptr[x], (TRI_L3 void*)(st + item_lds[x]), 16, 0, 0);
+      else __builtin_amdgcn_global_load_lds((const TRI_G1 void*)item_ptr[x], (TRI_L3 void*)(st + item_lds[x]), 4, 0, 0);
+      if (advance) item_ptr[x] += item_step[x];
     }
   };
+  // wait until at most the newest `K` rows of this wave's loads are in flight and
+  // every LDS read has returned, then meet the other waves
+  auto sync_rows = [&](auto k_tag) {
+    constexpr int K = decltype(k_tag)::value * XN;
+    static_assert(K <= 63, "vmcnt has 6 bits");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(K) : "memory");
+  };
+
+  // lane-constant LDS offsets: K, V rows as A operands (tile row m stands for key
+  // perm32(m)); Q, dO rows as B operands (the lane's own query)
+  OperandOffsets<T, D> ofk, ofq;
+  ofk.init(perm32(jl), lane);
+  ofq.init(jl, lane);
 
   const float c = a.c;
-  const float lse2_flagged = fast_log2((float)N);
   const bool wave_live = j_wave < N && k_wave < N;
 
-  auto compute_row = [&](int buf) {
+  auto compute_row = [&](int buf) __attribute__((always_inline)) {
     const unsigned char* st = tri_smem + buf * STAGE;
     const uint32_t* meta = reinterpret_cast<const uint32_t*>(st + OFF_META);
-    const bool flagged = meta[WKW] != 0;
-    // operands of this wave's tiles; tile row m of the key tiles stands for key perm32(m)
+    // (wave-uniform values are pinned to scalar registers so that the branches on
+    // them are real branches and not lane masks)
+    const bool flagged = __builtin_amdgcn_readfirstlane(meta[WKW]) != 0;
     frag qf[WJ][DS], dof[WJ][DS], kf[WK][DS], vf[WK][DS];
-    float lse2[WJ], delta[WJ];
+    float l2[WJ], nd[WJ];
 #pragma unroll
     for (int tj = 0; tj < WJ; ++tj) {
-      const int r = wj * (WJ * 32) + 32 * tj + jl;
 #pragma unroll
       for (int s = 0; s < DS; ++s) {
-        // a fully masked row ignores q.k as well as the bias
-        qf[tj][s] = flagged ? E::zero() : Tile::operand(st + OFF_Q, r, s, g);
-        dof[tj][s] = Tile::operand(st + OFF_DO, r, s, g);
+        qf[tj][s] = ofq.natural(st + OFF_Q + (wj * WJ + tj) * 32 * ROWB, s);
+        dof[tj][s] = ofq.natural(st + OFF_DO + (wj * WJ + tj) * 32 * ROWB, s);
       }
-      lse2[tj] = flagged ? lse2_flagged : reinterpret_cast<const float*>(st + OFF_LSE)[r] * kLog2e;
-      delta[tj] = reinterpret_cast<const float*>(st + OFF_DELTA)[r];
+      l2[tj] = reinterpret_cast<const float*>(st + OFF_LSE)[(wj * WJ + tj) * 32 + jl];
+      nd[tj] = reinterpret_cast<const float*>(st + OFF_DELTA)[(wj * WJ + tj) * 32 + jl];
     }
 #pragma unroll
-    for (int tk = 0; tk < WK; ++tk) {
-      const int r = wk * (WK * 32) + 32 * tk + perm32(jl);
+    for (int tk = 0; tk < WK; ++tk)
 #pragma unroll
       for (int s = 0; s < DS; ++s) {
-        kf[tk][s] = Tile::operand(st + OFF_K, r, s, g);
-        vf[tk][s] = Tile::operand(st + OFF_V, r, s, g);
+        kf[tk][s] = ofk.natural(st + OFF_K + (wk * WK + tk) * 32 * ROWB, s);
+        vf[tk][s] = ofk.natural(st + OFF_V + (wk * WK + tk) * 32 * ROWB, s);
       }
-    }
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk) {
       // a key tile past the last word of the row has no attended key
-      const uint32_t keepw = (k_wave / 32 + tk < a.nwords) ? meta[wk * WK + tk] : 0u;
+      const uint32_t keepw = __builtin_amdgcn_readfirstlane((k_wave / 32 + tk < a.nwords) ? meta[wk * WK + tk] : 0u);
       if (keepw == 0) continue;  // no attended key in this tile: dS = 0
-      const bool mixed = keepw != 0xffffffffu;
 #pragma unroll
       for (int tj = 0; tj < WJ; ++tj) {
         f32x16 s;
-        if (mixed) {
-          s = mask_tile(keepw, g);
+        if (!flagged && keepw == 0xffffffffu) {
+          s = E::mfma(kf[tk][0], qf[tj][0], biasr[tj][tk]);
+#pragma unroll
+          for (int sd = 1; sd < DS; ++sd) s = E::mfma(kf[tk][sd], qf[tj][sd], s);
+        } else {
+          // rare: a fully masked row ignores q.k and the bias; masked keys get a
+          // large negative score.  (Kept a real branch: a select between the two
+          // accumulator inits would copy 16 registers in the common case.)
+          asm volatile("" ::);
+          if (flagged) s = zero16();
+          else s = biasr[tj][tk];
+          if (keepw != 0xffffffffu) s = E::mfma(mask_operand<T>(keepw, perm32(jl)), E::splat(1.0f), s);
           if (!flagged) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) s[v] += biasr[tj][tk][v];
+            for (int sd = 0; sd < DS; ++sd) s = E::mfma(kf[tk][sd], qf[tj][sd], s);
           }
-          s = E::mfma(kf[tk][0], qf[tj][0], s);
-        } else if (flagged) {
-          s = E::mfma(kf[tk][0], qf[tj][0], zero16());
-        } else {
-          s = E::mfma(kf[tk][0], qf[tj][0], biasr[tj][tk]);
         }
         f32x16 dp = E::mfma(vf[tk][0], dof[tj][0], zero16());
 #pragma unroll
-        for (int sd = 1; sd < DS; ++sd) {
-          s = E::mfma(kf[tk][sd], qf[tj][sd], s);
-          dp = E::mfma(vf[tk][sd], dof[tj][sd], dp);
-        }
+        for (int sd = 1; sd < DS; ++sd) dp = E::mfma(vf[tk][sd], dof[tj][sd], dp);
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const float p = fast_exp2(__builtin_fmaf(s[v], c, -lse2[tj]));
-          dbacc[tj][tk][v] = __builtin_fmaf(p, dp[v] + delta[tj], dbacc[tj][tk][v]);  // the workspace holds -delta
+          const float p = fast_exp2(__builtin_fmaf(s[v], c, -l2[tj]));
+          dbacc[tj][tk][v] = __builtin_fmaf(p, dp[v] + nd[tj], dbacc[tj][tk][v]);
         }
       }
     }
   };
 
-  if constexpr (NBUF == 2) {
-    issue_row(i_begin, 0);
-    wait_dma();
-    __syncthreads();
-    for (int ir = 0; ir < nrows; ir += 2) {
-      issue_row(i_begin + ir + 1, 1);
-      if (wave_live) compute_row(0);
-      wait_dma();
-      __syncthreads();
-      if (ir + 1 >= nrows) break;
-      issue_row(i_begin + ir + 2, 0);
-      if (wave_live) compute_row(1);
-      wait_dma();
-      __syncthreads();
+  if constexpr (NBUF >= 2) {
+    // Ring of NBUF row buffers: the loads run NBUF-1 rows ahead of the compute, which
+    // hides the memory latency behind several rows of work.  Row q lives in buffer
+    // q % NBUF; the buffer that row q + NBUF - 1 goes to was last read for row q - 1,
+    // which every wave finished before the barrier that ended that row.
+    constexpr int P = NBUF - 1;
+#pragma unroll
+    for (int u = 0; u < P; ++u) issue_row(u);
+    sync_rows(std::integral_constant<int, P - 1>{});  // row 0 has landed
+    for (int r = 0; r < nrows; r += NBUF) {
+#pragma unroll
+      for (int u = 0; u < NBUF; ++u) {
+        if (r + u < nrows) {
+          issue_row((u + P) % NBUF);
+          if (wave_live) compute_row(u);
+          sync_rows(std::integral_constant<int, P - 1>{});  // the next row has landed
+        }
+      }
     }
   } else {
-    // one stage only (the double buffer does not fit in LDS): load, then compute
+    // one stage only (two do not fit in LDS): load, then compute
     for (int ir = 0; ir < nrows; ++ir) {
-      issue_row(i_begin + ir, 0);
-      wait_dma();
-      __syncthreads();
+      issue_row(0);
+      sync_rows(std::integral_constant<int, 0>{});
       if (wave_live) compute_row(0);
-      __syncthreads();
+      sync_rows(std::integral_constant<int, 0>{});
     }
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the spare rows loaded past the end
   if (!wave_live) return;
 
-  // a single chunk writes db itself; several chunks write fp32 partials
+  // a single chunk writes db itself; several chunks write fp32 partials.  The lane
+  // owns query j; its 16 values are two runs of 8 consecutive keys.
   const bool direct = a.nchunks == 1;
   T* db_bh = reinterpret_cast<T*>(a.db) + (int64_t)bh * N * N;
   float* part = a.dbpart + ((int64_t)chunk * a.BH + bh) * N * N;

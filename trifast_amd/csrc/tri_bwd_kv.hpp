@@ -78,9 +78,11 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int i = min(i0 + r, N - 1);  // rows past the end repeat the last one and are not stored
-    flagged[r] = a.rowflag[(int64_t)b * N + i] != 0;
+    // (wave-uniform values, pinned to scalar registers so that the branches on
+    // them are real branches and not lane masks)
+    flagged[r] = __builtin_amdgcn_readfirstlane(a.rowflag[(int64_t)b * N + i]) != 0;
     const int w = k_wave >> 5;
-    const uint32_t word = (wave_active && w < a.nwords) ? a.keep[((int64_t)b * N + i) * a.nwords + w] : 0u;
+    const uint32_t word = __builtin_amdgcn_readfirstlane((wave_active && w < a.nwords) ? a.keep[((int64_t)b * N + i) * a.nwords + w] : 0u);
     tile_live[r] = word != 0;
     tile_mixed[r] = word != 0xffffffffu;
     maskf[r] = mask_operand<T>(word, kl);

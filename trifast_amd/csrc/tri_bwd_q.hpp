@@ -79,7 +79,7 @@ __global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(co
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int i = min(i0 + r, N - 1);  // rows past the end repeat the last one and are not stored
-    flagged[r] = a.rowflag[(int64_t)b * N + i] != 0;
+    flagged[r] = __builtin_amdgcn_readfirstlane(a.rowflag[(int64_t)b * N + i]) != 0;  // pinned to a scalar register
     any_flagged |= flagged[r];
     keep_row[r] = a.keep + ((int64_t)b * N + i) * a.nwords;
     const int jc = min(j, N - 1);
@@ -184,7 +184,7 @@ __global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(co
 #pragma unroll
         for (int u = 0; u < KU; ++u) {
           const int w = (kt0 >> 5) + u;
-          kw[r][u] = (w < a.nwords) ? keep_row[r][w] : 0u;
+          kw[r][u] = __builtin_amdgcn_readfirstlane((w < a.nwords) ? keep_row[r][w] : 0u);
         }
     }
     f32x16 biasv[KU];
