@@ -43,7 +43,7 @@ def test_tile_tables():
         assert 1 <= nt <= 8
         for t in range(nt):
             info = _lib.tile_info(kernel, t)
-            assert info["BLOCK_J"] % 32 == 0 and info["BLOCK_K"] % 32 == 0 and info["num_waves"] in (1, 2, 4, 8)
+            assert info["BLOCK_J"] % 32 == 0 and info["BLOCK_K"] % 32 == 0 and info["num_waves"] in (1, 2, 4, 8, 16)
         with pytest.raises(ValueError):
             _lib.tile_info(kernel, nt)
     assert lib.trifast_num_tiles(99) < 0

@@ -49,8 +49,12 @@ struct BwdArgs {
   const float* lse;
   const uint32_t* keep;
   const uint32_t* rowflag;
-  float* delta;              // [b*h, n, n] fp32 workspace, indexed [i, j]: MINUS rowsum(o * do)
-  float* lse2;               // [b*h, n, n] fp32 workspace: lse * log2(e); log2(n) for fully masked rows
+  // [b*h, n, n] 32-bit workspaces indexed [i, j], written by the dq kernel for the
+  // other two: the per-query terms of the backward as rank-1 MFMA operand words
+  // (see split_word): delta = -rowsum(o * do); lse2 = -lse * sqrt(d), the
+  // log-sum-exp in the raw-score domain (ln n instead of lse for fully masked rows)
+  uint32_t* delta;
+  uint32_t* lse2;
   float* dbpart;             // [nchunks, b*h, n, n] fp32 partial db (nchunks > 1 only)
   void *dq, *dk, *dv, *db;
   Str5 sq, sk, sv, sdo;

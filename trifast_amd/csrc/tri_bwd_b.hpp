@@ -7,16 +7,16 @@
 // atomics.  Per row the workgroup stages the Q, dO rows of its queries and the K,
 // V rows of its keys in LDS (direct global->LDS loads into a ring of row buffers
 // that runs several rows ahead of the compute, swizzled tiles) together with
-// lse*log2e and -delta as left by the dq kernel, and each wave
+// the lse and delta operand words left by the dq kernel, and each wave
 // recomputes for its tiles
-//   S^T = K Q^T (+bias), P^T = exp2(S^T c - lse2), dP^T = V dO^T, dS^T = P^T (dP^T - delta)
+//   S^T = K Q^T + bias - lse, P^T = exp2(c S^T), dP^T = V dO^T - delta, dS^T = P^T dP^T
 // with every operand in its natural row-major layout: a lane owns one query
-// (column) and 16 keys of each tile, so lse2 and delta are per-lane scalars.  (The
-// other orientation would take -delta and lse2 as 16 values per lane from LDS,
-// which costs more LDS bandwidth than this kernel has to spare: every row brings
-// fresh Q, dO, K, V operands.)  The bias tiles (register-resident, fp32, raw-score
-// domain) are the accumulator init of every row's score MFMA.  Masked keys get a
-// large negative score through one extra MFMA (see mask_operand).
+// (column) and 16 keys of each tile.  The additive terms ride on the matrix pipe:
+// the bias tiles (register-resident, fp32, raw-score domain) are the accumulator
+// init of every row's score MFMA, and the per-query terms -lse*sqrt(d) and -delta
+// enter through one extra MFMA each (see rank1_operand), which leaves one
+// multiply, one exp2 and one fma per element to the vector ALU.  Masked keys get a
+// large negative score through one more MFMA (see mask_operand).
 //
 // All workgroups of one (batch*head, chunk) read the same rows at about the same
 // time; the block index is remapped so that they run on one XCD and share its L2.
@@ -83,8 +83,8 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   const T* vbase = reinterpret_cast<const T*>(a.v) + b * a.sv.b + h * a.sv.h;
   const T* dobase = reinterpret_cast<const T*>(a.dout) + b * a.sdo.b + h * a.sdo.h;
   const T* pack_bh = reinterpret_cast<const T*>(a.packq) + (int64_t)bh * a.NP * a.NP * 1024;
-  const float* lse2_bh = a.lse2 + (int64_t)bh * N * N;
-  const float* delta_bh = a.delta + (int64_t)bh * N * N;
+  const float* lse2_bh = reinterpret_cast<const float*>(a.lse2) + (int64_t)bh * N * N;    // 32-bit words, moved as floats
+  const float* delta_bh = reinterpret_cast<const float*>(a.delta) + (int64_t)bh * N * N;
 
   // bias tiles in the raw-score domain: accumulator init of every row's score MFMA
   f32x16 biasr[WJ][WK];
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     // them are real branches and not lane masks)
     const bool flagged = __builtin_amdgcn_readfirstlane(meta[WKW]) != 0;
     frag qf[WJ][DS], dof[WJ][DS], kf[WK][DS], vf[WK][DS];
-    float l2[WJ], nd[WJ];
+    frag lf[WJ], df[WJ];  // per-query terms -lse*sqrt(d) and -delta as rank-1 MFMA operands
 #pragma unroll
     for (int tj = 0; tj < WJ; ++tj) {
 #pragma unroll
@@ -203,8 +203,8 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
         qf[tj][s] = ofq.natural(st + OFF_Q + (wj * WJ + tj) * 32 * ROWB, s);
         dof[tj][s] = ofq.natural(st + OFF_DO + (wj * WJ + tj) * 32 * ROWB, s);
       }
-      l2[tj] = reinterpret_cast<const float*>(st + OFF_LSE)[(wj * WJ + tj) * 32 + jl];
-      nd[tj] = reinterpret_cast<const float*>(st + OFF_DELTA)[(wj * WJ + tj) * 32 + jl];
+      lf[tj] = rank1_operand<T>(reinterpret_cast<const uint32_t*>(st + OFF_LSE)[(wj * WJ + tj) * 32 + jl], g);
+      df[tj] = rank1_operand<T>(reinterpret_cast<const uint32_t*>(st + OFF_DELTA)[(wj * WJ + tj) * 32 + jl], g);
     }
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk)
@@ -221,10 +221,11 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
 #pragma unroll
       for (int tj = 0; tj < WJ; ++tj) {
         f32x16 s;
+        const frag ones = E::splat(1.0f);
         if (!flagged && keepw == 0xffffffffu) {
-          s = E::mfma(kf[tk][0], qf[tj][0], biasr[tj][tk]);
+          s = E::mfma(ones, lf[tj], biasr[tj][tk]);
 #pragma unroll
-          for (int sd = 1; sd < DS; ++sd) s = E::mfma(kf[tk][sd], qf[tj][sd], s);
+          for (int sd = 0; sd < DS; ++sd) s = E::mfma(kf[tk][sd], qf[tj][sd], s);
         } else {
           // rare: a fully masked row ignores q.k and the bias; masked keys get a
           // large negative score.  (Kept a real branch: a select between the two
@@ -232,19 +233,20 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
           asm volatile("" ::);
           if (flagged) s = zero16();
           else s = biasr[tj][tk];
-          if (keepw != 0xffffffffu) s = E::mfma(mask_operand<T>(keepw, perm32(jl)), E::splat(1.0f), s);
+          if (keepw != 0xffffffffu) s = E::mfma(mask_operand<T>(keepw, perm32(jl)), ones, s);
+          s = E::mfma(ones, lf[tj], s);
           if (!flagged) {
 #pragma unroll
             for (int sd = 0; sd < DS; ++sd) s = E::mfma(kf[tk][sd], qf[tj][sd], s);
           }
         }
-        f32x16 dp = E::mfma(vf[tk][0], dof[tj][0], zero16());
+        f32x16 dp = E::mfma(ones, df[tj], zero16());
 #pragma unroll
-        for (int sd = 1; sd < DS; ++sd) dp = E::mfma(vf[tk][sd], dof[tj][sd], dp);
+        for (int sd = 0; sd < DS; ++sd) dp = E::mfma(vf[tk][sd], dof[tj][sd], dp);
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const float p = fast_exp2(__builtin_fmaf(s[v], c, -l2[tj]));
-          dbacc[tj][tk][v] = __builtin_fmaf(p, dp[v] + nd[tj], dbacc[tj][tk][v]);
+          const float p = fast_exp2(s[v] * c);
+          dbacc[tj][tk][v] = __builtin_fmaf(p, dp[v], dbacc[tj][tk][v]);
         }
       }
     }

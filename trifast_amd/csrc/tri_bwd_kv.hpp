@@ -4,17 +4,19 @@
 // owns one tile of 32 keys for all R rows: its K and V rows (B operands) and the
 // dk, dv accumulators stay in registers, and the queries of the rows are streamed
 // through LDS in tiles of BJ (direct global->LDS loads, double-buffered, swizzled;
-// rows of Q and dO, lse*log2e and -delta as left by the dq kernel, and the packed
+// rows of Q and dO, the lse and delta operand words left by the dq kernel, and the packed
 // bias tiles).  Scores are computed UN-transposed here, S = Q K^T, so that a lane
 // owns one key (column) and 16 queries of every 32-query tile: P and dS are then
 // already in B-operand layout for the two products that contract over queries,
 //   dv^T += dO^T P,   dk^T += Q^T dS,   dk = dk^T / sqrt(d),
 // whose A operands dO^T, Q^T come from the natural tiles through transposing LDS
-// reads.  Two accumulator inits do work for free: the bias tile (fp32, raw-score
-// domain, converted once per stage and shared by the R rows) starts the score
-// MFMA, and the -delta values of the tile's 16 queries start the dP MFMA, so
-// dS = P * (dP - delta) is one multiply.  Masked keys get a large negative score
-// through one extra MFMA (see mask_operand), which makes their P and dS zero.
+// reads.  The per-element additive terms ride on the matrix pipe: the bias tile
+// (fp32, raw-score domain, converted once per stage and shared by the R rows) is
+// the accumulator init of the score MFMA, and the per-query terms -lse*sqrt(d) and
+// -delta enter through one extra MFMA each (see rank1_operand), so that
+// P = exp2(c * acc) and dS = P * dP' are one multiply each.  Masked keys get a
+// large negative score through one more MFMA (see mask_operand), which makes
+// their P and dS zero.
 //
 // Replaces _bwd_kv of reference src/trifast/triton.py:143-263.
 #pragma once
@@ -66,8 +68,8 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
   const T* vbh = reinterpret_cast<const T*>(a.v) + b * a.sv.b + h * a.sv.h;
   const T* dobh = reinterpret_cast<const T*>(a.dout) + b * a.sdo.b + h * a.sdo.h;
   const T* pack_bh = reinterpret_cast<const T*>(a.packk) + (int64_t)bh * a.NP * a.NP * 1024;
-  const float* lse2_bh = a.lse2 + (int64_t)bh * N * N;
-  const float* delta_bh = a.delta + (int64_t)bh * N * N;
+  const float* lse2_bh = reinterpret_cast<const float*>(a.lse2) + (int64_t)bh * N * N;    // 32-bit words, moved as floats
+  const float* delta_bh = reinterpret_cast<const float*>(a.delta) + (int64_t)bh * N * N;
 
   // per-row state: K and V tiles as B operands (lane owns key k_wave + kl).  A
   // fully masked row drops the q.k and bias terms from its scores: its K operand
@@ -165,20 +167,10 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
     }
     return bv;
   };
-  // the 16 per-query values (lse2 or -delta) of tile (r, u) that this lane's C
-  // layout pairs with its 16 scores: two runs of 8 queries
-  auto query_values = [&](const unsigned char* st, int off, int r, int u) -> f32x16 {
-    const float* src = reinterpret_cast<const float*>(st + off) + r * BJ + 32 * u + 8 * g;
-    f32x16 x;
-#pragma unroll
-    for (int r2 = 0; r2 < 2; ++r2)
-#pragma unroll
-      for (int e4 = 0; e4 < 2; ++e4) {
-        const f32x4 y = *reinterpret_cast<const f32x4*>(src + 16 * r2 + 4 * e4);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) x[8 * r2 + 4 * e4 + e] = y[e];
-      }
-    return x;
+  // the per-query operand word (lse or delta term) of the query this lane's A
+  // operand row stands for, in tile (r, u)
+  auto query_word = [&](const unsigned char* st, int off, int r, int u) -> uint32_t {
+    return reinterpret_cast<const uint32_t*>(st + off)[r * BJ + 32 * u + perm32(kl)];
   };
 
   const float c = a.c;
@@ -195,12 +187,20 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
 #pragma unroll
     for (int u = 0; u < JU; ++u) biasv[u] = bias_from_lds(st, u);
 
+    // scores: bias tile (accumulator init) - lse*sqrt(d) (per query, one MFMA) + Q K^T;
+    // dP - delta: -delta (per query, one MFMA) + dO V^T
     auto chains = [&](int t, f32x16& sc, f32x16& dp) {
       const int u = t / R, r = t % R;
       const unsigned char* qt = st + OFF_Q + (r * BJ + 32 * u) * ROWB;
       const unsigned char* dot = st + OFF_DO + (r * BJ + 32 * u) * ROWB;
+      uint32_t lw = query_word(st, OFF_LSE, r, u);
+      if constexpr (EDGE) {
+        // queries past the end: a huge lse makes their P and dS zero
+        if (jt0 + 32 * u + perm32(kl) >= N) lw = split_word<T>(E::kMaskElem);
+      }
+      const frag ones = E::splat(1.0f);
       if (!flagged[r] && !tile_mixed[r]) {
-        sc = E::mfma(ofs.natural(qt, 0), kf[r][0], biasv[u]);
+        sc = E::mfma(rank1_operand<T>(lw, g), ones, biasv[u]);
       } else {
         // rare: kept a real branch so that the common case starts from the bias
         // tile in place (a select between the two inits would copy 16 registers)
@@ -208,12 +208,12 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
         f32x16 init;
         if (flagged[r]) init = zero16();
         else init = biasv[u];
-        if (tile_mixed[r]) init = E::mfma(E::splat(1.0f), maskf[r], init);
-        sc = E::mfma(ofs.natural(qt, 0), kf[r][0], init);
+        if (tile_mixed[r]) init = E::mfma(ones, maskf[r], init);
+        sc = E::mfma(rank1_operand<T>(lw, g), ones, init);
       }
-      dp = E::mfma(ofs.natural(dot, 0), vf[r][0], query_values(st, OFF_DELTA, r, u));
+      dp = E::mfma(rank1_operand<T>(query_word(st, OFF_DELTA, r, u), g), ones, zero16());
 #pragma unroll
-      for (int sd = 1; sd < DS; ++sd) {
+      for (int sd = 0; sd < DS; ++sd) {
         sc = E::mfma(ofs.natural(qt, sd), kf[r][sd], sc);
         dp = E::mfma(ofs.natural(dot, sd), vf[r][sd], dp);
       }
@@ -227,16 +227,10 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
       f32x16 sn, dn;
       if (t + 1 < TS) chains(t + 1, sn, dn);
       if (tile_live[r] && (!EDGE || jt0 + 32 * u < N)) {
-        f32x16 l2 = query_values(st, OFF_LSE, r, u);
-        if constexpr (EDGE) {
-          // queries past the end: an infinite lse makes their P and dS zero
-#pragma unroll
-          for (int v = 0; v < 16; ++v) l2[v] = (jt0 + 32 * u + cidx(v, g) < N) ? l2[v] : 1.0e30f;
-        }
         float p[16], ds[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          p[v] = fast_exp2(__builtin_fmaf(sc[v], c, -l2[v]));
+          p[v] = fast_exp2(sc[v] * c);
           ds[v] = p[v] * dp[v];
         }
 #pragma unroll

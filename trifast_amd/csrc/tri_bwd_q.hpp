@@ -15,8 +15,8 @@
 // so the subtraction costs nothing.  Masked keys get a large negative score
 // through one extra MFMA (see mask_operand), which makes their P and dS zero.
 //
-// This kernel runs first: it writes -delta and lse*log2e (log2 n for fully
-// masked rows) in fp32 for the dk/dv and db kernels.
+// This kernel runs first: it writes -delta and -lse*sqrt(d) (ln n for lse in fully
+// masked rows) per query, as rank-1 MFMA operand words, for the dk/dv and db kernels.
 //
 // Replaces _bwd_q of reference src/trifast/triton.py:274-383.
 #pragma once
@@ -101,8 +101,9 @@ __global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(co
     dsum = half_sum(dsum);
     lse2[r] = (j >= N) ? 0.f : (flagged[r] ? fast_log2((float)N) : a.lse[((int64_t)bh * N + i) * N + jc] * kLog2e);
     if (j < N && i0 + r < N && g == 0) {
-      a.delta[((int64_t)bh * N + i) * N + j] = -dsum;
-      a.lse2[((int64_t)bh * N + i) * N + j] = lse2[r];
+      // the per-query terms of the other two backward kernels, as rank-1 MFMA operand words
+      a.delta[((int64_t)bh * N + i) * N + j] = split_word<T>(-dsum);
+      a.lse2[((int64_t)bh * N + i) * N + j] = split_word<T>(-lse2[r] * (kLn2 * a.sqrt_d));
     }
 #pragma unroll
     for (int v = 0; v < 16; ++v) ndelta[r][v] = -dsum;
@@ -267,7 +268,8 @@ __global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(co
       __syncthreads();
     }
   };
-  if (masks.all_plain()) stage_loop(std::true_type{});
+  // (a last stage with fewer than KU key tiles is not plain: its missing tiles are masked)
+  if (masks.all_plain() && ntiles % KU == 0) stage_loop(std::true_type{});
   else stage_loop(std::false_type{});
 
   if (!wave_active || j >= N) return;

@@ -135,8 +135,8 @@ struct Workspace {
   uint32_t* rowflag;
   void* packq;
   void* packk;
-  float* delta;
-  float* lse2;
+  uint32_t* delta;
+  uint32_t* lse2;
   float* dbpart;
   int nwords, np;
 };
@@ -163,9 +163,9 @@ Workspace carve(void* ws, int64_t b, int64_t h, int64_t n, int dtype) {
   p += ws_pack_bytes(b, h, n, dtype);
   w.packk = p;
   p += ws_pack_bytes(b, h, n, dtype);
-  w.delta = reinterpret_cast<float*>(p);
+  w.delta = reinterpret_cast<uint32_t*>(p);
   p += align256(b * h * n * n * 4);
-  w.lse2 = reinterpret_cast<float*>(p);
+  w.lse2 = reinterpret_cast<uint32_t*>(p);
   p += align256(b * h * n * n * 4);
   w.dbpart = reinterpret_cast<float*>(p);
   w.nwords = (int)nwords;
@@ -270,13 +270,14 @@ int trifast_supports(int kernel, int tile, int64_t n, int64_t h, int64_t d, int 
 int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype) {
   (void)h;
   // Picks measured on MI355X at d = 32; anything that does not fit the shape
-  // falls back to tile 0, which every dtype and head dim supports.
+  // falls back to tile 0 and then to the first tile that supports it.
   int pick = 0;
   switch (kernel) {
     case TRIFAST_KERNEL_FWD: pick = n <= 64 ? 0 : 3; break;     // 4 pair rows share a bias tile
-    case TRIFAST_KERNEL_BWD_Q: pick = n <= 64 ? 0 : 2; break;   // 2 pair rows, 32 keys per stage
-    case TRIFAST_KERNEL_BWD_KV: pick = n <= 64 ? 0 : 2; break;  // 2 pair rows, 64 queries per stage
-    case TRIFAST_KERNEL_BWD_B: pick = 2; break;                 // 64 x 64 block, most workgroups per CU
+    case TRIFAST_KERNEL_BWD_Q: pick = n <= 64 ? 0 : 1; break;   // 2 pair rows, 64 keys per stage
+    case TRIFAST_KERNEL_BWD_KV: pick = n <= 64 ? 0 : 1; break;  // 2 pair rows, 32 queries per stage
+    case TRIFAST_KERNEL_BWD_B: pick = n <= 128 ? 2 : 4; break;  // 128 x 128 block of 16 waves; 64 x 64 at small n
+
     default: return fail(TRIFAST_EINVAL, "unknown kernel id %d", kernel);
   }
   if (!trifast_supports(kernel, pick, n, h, d, dtype)) pick = 0;

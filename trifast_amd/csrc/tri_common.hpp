@@ -192,6 +192,36 @@ TRI_DEV void half_pair(float x, float& a, float& b) {
 TRI_DEV float half_max(float x) { float a, b; half_pair(x, a, b); return fmaxf(a, b); }
 TRI_DEV float half_sum(float x) { float a, b; half_pair(x, a, b); return a + b; }
 
+// Per-row (or per-column) additive terms through the matrix pipe: acc[m][n] += x[m]
+// is one extra MFMA whose A operand holds x[m] in its first contraction slots and
+// whose B operand is all ones (or the other way round for a per-column term).
+// For the 16-bit types x is split into hi + lo parts (two slots), which keeps
+// 16 / 22 significant bits; fp32 needs one slot.  split_word() packs the parts
+// into one 32-bit word (so they can be stored per query by one kernel and loaded
+// by another); rank1_operand() turns the word into the operand of the lane that
+// owns row / column m: lanes of group 0 supply the first slots, group 1 zeros.
+template <typename T>
+TRI_DEV uint32_t split_word(float x) {
+  if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(uint32_t, x);
+  } else {
+    const T hi = (T)x;
+    const T lo = (T)(x - (float)hi);
+    return (uint32_t)__builtin_bit_cast(uint16_t, hi) | ((uint32_t)__builtin_bit_cast(uint16_t, lo) << 16);
+  }
+}
+template <typename T>
+TRI_DEV typename Elem<T>::frag rank1_operand(uint32_t word, int g) {
+  const uint32_t w = g ? 0u : word;
+  if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(float, w);
+  } else {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 v = {w, 0u, 0u, 0u};
+    return __builtin_bit_cast(typename Elem<T>::frag, v);
+  }
+}
+
 TRI_DEV f32x16 zero16() {
   f32x16 z;
 #pragma unroll

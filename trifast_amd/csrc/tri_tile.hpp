@@ -33,6 +33,17 @@ TRI_DEV void xcd_remap(int gx, int& x, int& y) {
 
 TRI_DEV void wait_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// Stage hand-over for a ring of LDS buffers: wait until at most the newest
+// IN_FLIGHT loads of this wave are outstanding (loads complete in issue order, so
+// everything issued before them has landed in LDS) and every LDS read of the wave
+// has returned, then meet the other waves.  A plain barrier instruction: the
+// fence of __syncthreads() would wait for every load in flight.
+template <int IN_FLIGHT>
+TRI_DEV void ring_sync() {
+  static_assert(IN_FLIGHT >= 0 && IN_FLIGHT <= 63, "vmcnt has 6 bits");
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(IN_FLIGHT) : "memory");
+}
+
 template <typename T, int D>
 struct LdsTile {
   static constexpr int ROWB = D * (int)sizeof(T);  // bytes per row
@@ -164,6 +175,11 @@ struct TileStream {
       p0[x] = row_ptr(r) + c * Tile::VEC;
     }
   }
+  // EVERY = true: a wave whose share of the tile is empty repeats the tile's last
+  // piece instead of skipping it, so that every wave issues exactly XN loads (a
+  // fixed count is what lets a later s_waitcnt vmcnt(k) stand for "all but the
+  // newest stages have landed")
+  template <bool EVERY = false>
   TRI_DEV void issue(unsigned char* base, int64_t elem_offset, int wave) const {
     // the offset is wave-uniform: pin it to scalar registers so that a stage costs
     // one 64-bit add per load
@@ -172,8 +188,8 @@ struct TileStream {
     elem_offset = (int64_t)(((uint64_t)hi << 32) | lo);
 #pragma unroll
     for (int x = 0; x < XN; ++x) {
-      const int gi = x * NW + wave;
-      if (GROUPS % NW == 0 || gi < GROUPS)
+      const int gi = EVERY ? min(x * NW + wave, GROUPS - 1) : x * NW + wave;
+      if (EVERY || GROUPS % NW == 0 || gi < GROUPS)
         __builtin_amdgcn_global_load_lds((const TRI_G1 void*)(p0[x] + elem_offset), (TRI_L3 void*)(base + gi * 1024), 16, 0, 0);
     }
   }
@@ -207,14 +223,15 @@ struct FloatStream {
       p0[x] = elem_ptr(gi * 64 + lane);
     }
   }
+  template <bool EVERY = false>
   TRI_DEV void issue(float* base, int64_t elem_offset, int wave) const {
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)elem_offset);
     const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)elem_offset >> 32));
     elem_offset = (int64_t)(((uint64_t)hi << 32) | lo);
 #pragma unroll
     for (int x = 0; x < XN; ++x) {
-      const int gi = x * NW + wave;
-      if (GROUPS % NW == 0 || gi < GROUPS)
+      const int gi = EVERY ? min(x * NW + wave, GROUPS - 1) : x * NW + wave;
+      if (EVERY || GROUPS % NW == 0 || gi < GROUPS)
         __builtin_amdgcn_global_load_lds((const TRI_G1 void*)(p0[x] + elem_offset), (TRI_L3 void*)(base + gi * 64), 4, 0, 0);
     }
   }
