@@ -31,6 +31,17 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA
 PEAK_F32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch (fetch + write) of the kernels of workload M with the tiles the
+# tuner picks there, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
+# profiles/bench_M_hbm_traffic.txt (readings scaled by a plain 256 MiB copy).  Reported
+# as roofline.traffic when the benchmark runs that workload with that tile.
+MEASURED_TRAFFIC_MIB = {
+    ("M", "_fwd", (128, 32, 4)): 1516.8,
+    ("M", "_bwd_q", (128, 32, 4)): 2264.8,
+    ("M", "_bwd_kv", (32, 128, 4)): 2091.4,
+    ("M", "_bwd_b", (128, 128, 16)): 1649.0,
+}
+
 # name -> (dtype, b, n, h, d, description)
 WORKLOADS = {
     "C1": (torch.float32, 1, 32, 4, 32, "fp32 b1 n32 h4 d32, 10% random mask"),
@@ -264,6 +275,9 @@ def main():
     for name, rec in kern.items():
         rec["tflops"] = gemms[name] * 2 * b * h * n**3 * d / rec["ms"] / 1e9
     dom = max(kern, key=lambda key: kern[key]["ms"])
+    tile = kern[dom]["tile"]
+    mib = MEASURED_TRAFFIC_MIB.get((args.workload, dom, (tile["BLOCK_J"], tile["BLOCK_K"], tile["num_waves"])))
+    traffic = None if mib is None else mib * 2**20
     roofline = {
         "kernel": dom,
         "bound": "mfma",
@@ -271,7 +285,7 @@ def main():
         "peak": peak,
         "unit": "TFLOP/s",
         "frac": kern[dom]["tflops"] / peak,
-        "traffic": None,
+        "traffic": traffic,
         "launch_ms": kern[dom]["ms"],
         "flop_per_launch": gemms[dom] * 2 * b * h * n**3 * d,
     }
