@@ -72,6 +72,12 @@ int bwd_b_chunks(int64_t n, int64_t bh) {
   if (chunks > max_chunks) chunks = max_chunks;
   if (chunks > 8) chunks = 8;
   if (chunks < 1) chunks = 1;
+  // The kernel runs each (batch*head, chunk) group on one XCD: make the number of
+  // groups a multiple of the 8 XCDs when the row count allows it.
+  int64_t g = bh % 8 == 0 ? 8 : (bh % 4 == 0 ? 4 : (bh % 2 == 0 ? 2 : 1));
+  const int64_t m = 8 / g;  // chunks must be a multiple of m
+  const int64_t rounded = (chunks + m - 1) / m * m;
+  if (rounded <= max_chunks && rounded <= 8) chunks = rounded;
   return (int)chunks;
 }
 

@@ -1,0 +1,122 @@
+"""Runtime and peak-memory sweeps over the sequence length, written in the layout the
+reference keeps its own results in (``benchmark/<device>/runtime/*.csv``,
+``benchmark/<device>/memory/memory.parquet``), so that MI355X results sit beside the
+A100 / RTX 3090 files.
+
+    python -m trifast_amd.sweep runtime [--out benchmark] [--n-max 2048] [--step 32]
+    python -m trifast_amd.sweep memory  [--out benchmark] [--n-max 2048] [--step 32]
+
+Same protocol as reference scripts/benchmark.py:13-105 and scripts/memory.py:25-131:
+bf16, h=4, d=32, 50 % random mask, n = 32..2048 in steps of 32; "fwd" times the forward,
+"bwd" times ``o.sum().backward()`` alone (retain_graph), median of the timed calls in
+milliseconds; memory is ``torch.cuda.max_memory_allocated`` around one forward
+(+ backward) in MiB.  Only the "Trifast" column is produced: the other columns of the
+reference's tables are other implementations.
+"""
+
+from __future__ import annotations
+
+import argparse
+import statistics
+from pathlib import Path
+
+import torch
+
+from .torch import triangle_attention
+from .utils import gen_tensors
+
+H, D = 4, 32
+DTYPE = torch.bfloat16
+
+
+def device_name() -> str:
+    # reference src/trifast/autotune_helpers.py:19
+    return torch.cuda.get_device_name().replace(" ", "-")
+
+
+def _median_ms(fn, warmup: int = 5, rep_ms: float = 100.0, min_calls: int = 10, max_calls: int = 200) -> float:
+    """Median duration of fn() in ms: `warmup` untimed calls, then calls timed one by one
+    with events until `rep_ms` of GPU time or `max_calls` (mirrors triton's do_bench)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    times, total = [], 0.0
+    while len(times) < min_calls or (total < rep_ms and len(times) < max_calls):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        fn()
+        end.record()
+        end.synchronize()
+        times.append(start.elapsed_time(end))
+        total += times[-1]
+    return statistics.median(times)
+
+
+def runtime(out: Path, ns: list[int]) -> None:
+    out = out / device_name() / "runtime"
+    out.mkdir(parents=True, exist_ok=True)
+    rows = {"fwd": [], "bwd": []}
+    for n in ns:
+        q, k, v, bias, mask = gen_tensors(n, D, H, True, torch.device("cuda"), DTYPE)
+        fwd = lambda: triangle_attention(q, k, v, bias, mask)
+        ms_fwd = _median_ms(fwd)
+        s = fwd().sum()
+        ms_bwd = _median_ms(lambda: s.backward(retain_graph=True))
+        q.grad = k.grad = v.grad = bias.grad = None
+        rows["fwd"].append((n, ms_fwd))
+        rows["bwd"].append((n, ms_bwd))
+        print(f"n={n:5d} fwd {ms_fwd:8.4f} ms  bwd {ms_bwd:8.4f} ms", flush=True)
+    for mode, data in rows.items():
+        path = out / f"tri_attn_{mode}_{DTYPE}.csv"
+        with open(path, "w") as f:
+            f.write("n,Trifast\n")
+            for n, ms in data:
+                f.write(f"{float(n):.6f},{ms:.6f}\n")
+        print(f"wrote {path}")
+
+
+def memory(out: Path, ns: list[int], repeat: int = 3) -> None:
+    import pandas as pd
+
+    out = out / device_name() / "memory"
+    out.mkdir(parents=True, exist_ok=True)
+    rows = []
+    for n in ns:
+        for mode in ("fwd", "bwd"):
+            for it in range(1 + repeat):  # the first pass warms the tile cache and is not recorded
+                torch.cuda.synchronize()
+                torch.cuda.reset_peak_memory_stats()
+                q, k, v, bias, mask = gen_tensors(n, D, H, True, torch.device("cuda"), DTYPE)
+                base = torch.cuda.max_memory_allocated() / 1024**2
+                o = triangle_attention(q, k, v, bias, mask)
+                torch.cuda.synchronize()
+                if mode == "bwd":
+                    o.sum().backward()
+                    torch.cuda.synchronize()
+                peak = torch.cuda.max_memory_allocated() / 1024**2
+                if it > 0:
+                    rows.append({"n": n, "base_memory": base, "peak_memory": peak, "model": "trifast", "mode": mode, "dtype": str(DTYPE)})
+                del q, k, v, bias, mask, o
+        print(f"n={n:5d} peak fwd {rows[-1 - repeat]['peak_memory']:10.1f} MiB  bwd {rows[-1]['peak_memory']:10.1f} MiB", flush=True)
+    df = pd.DataFrame(rows)
+    df.to_parquet(out / "memory.parquet")
+    pivot = df.groupby(["n", "mode"])[["base_memory", "peak_memory"]].mean().reset_index()
+    pivot.to_csv(out / "memory.csv", index=False, float_format="%.3f")
+    print(f"wrote {out / 'memory.parquet'} and {out / 'memory.csv'}")
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("what", choices=["runtime", "memory"])
+    ap.add_argument("--out", default="benchmark")
+    ap.add_argument("--n-max", type=int, default=2048)
+    ap.add_argument("--step", type=int, default=32)
+    args = ap.parse_args()
+    if not torch.cuda.is_available():
+        raise SystemExit("the sweeps need a GPU: the operator has no CPU path")
+    ns = list(range(args.step, args.n_max + 1, args.step))
+    (runtime if args.what == "runtime" else memory)(Path(args.out), ns)
+
+
+if __name__ == "__main__":
+    main()
