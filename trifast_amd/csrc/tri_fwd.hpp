@@ -188,8 +188,9 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
   // overflow to +inf of a query that outgrew the reference by a lot, and the very
   // first tile, whose reference is -1e30) is the reference raised to the running
   // maximum and the tile recomputed.
-  auto compute_stage = [&](auto plain_tag, int kt0, int buf) __attribute__((always_inline)) {
-    constexpr bool PLAIN = decltype(plain_tag)::value;
+  auto compute_stage = [&](auto mode_tag, int kt0, int buf) __attribute__((always_inline)) {
+    constexpr int MODE = decltype(mode_tag)::value;
+    constexpr bool PLAIN = MODE == kPlain;
     const unsigned char* st = tri_smem + buf * STAGE;
     if (!wave_active) return;
     constexpr int TS = KU * R;
@@ -221,13 +222,24 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
       if constexpr (PLAIN) {
         sc = E::mfma(kf[0], qf[r][0], biasv[u]);
       } else {
-        // a fully masked row has no bias (and a zero Q: all its scores are equal),
-        // but keys past the end of a ragged last tile stay masked for it too
-        f32x16 init;
-        if (flagged[r]) init = zero16();
-        else init = biasv[u];
-        if (kw[r][u] != 0xffffffffu) init = E::mfma(mask_operand<T>(kw[r][u], perm32(jl)), E::splat(1.0f), init);
-        sc = E::mfma(kf[0], qf[r][0], init);
+        // Each case ends in the MFMA that defines sc, so that the bias tile is used
+        // in place as an accumulator init (a select between inits copies 16 registers).
+        if (MODE == kMasked) {
+          // no fully masked row in the workgroup: the mask MFMA runs for every tile
+          // (its operand is zero where nothing is masked) and nothing branches
+          sc = E::mfma(kf[0], qf[r][0], E::mfma(mask_operand<T>(kw[r][u], perm32(jl)), E::splat(1.0f), biasv[u]));
+        } else if (!flagged[r]) {
+          if (kw[r][u] != 0xffffffffu)
+            sc = E::mfma(kf[0], qf[r][0], E::mfma(mask_operand<T>(kw[r][u], perm32(jl)), E::splat(1.0f), biasv[u]));
+          else
+            sc = E::mfma(kf[0], qf[r][0], biasv[u]);
+        } else {
+          // a fully masked row has no bias (and a zero Q: all its scores are equal),
+          // but keys past the end of a ragged last tile stay masked for it too
+          asm volatile("" ::);
+          sc = E::mfma(mask_operand<T>(kw[r][u], perm32(jl)), E::splat(1.0f), zero16());
+          sc = E::mfma(kf[0], qf[r][0], sc);
+        }
       }
 #pragma unroll
       for (int sd = 1; sd < DS; ++sd) sc = E::mfma(kf[sd], qf[r][sd], sc);
@@ -310,8 +322,8 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
   // two inside one loop would copy the accumulators where the versions meet).
   __syncthreads();  // key-tile bitmaps visible
   const int ntiles = a.nwords;
-  auto stage_loop = [&](auto plain_tag) __attribute__((always_inline)) {
-    constexpr bool PLAIN = decltype(plain_tag)::value;
+  auto stage_loop = [&](auto mode_tag) __attribute__((always_inline)) {
+    constexpr bool PLAIN = decltype(mode_tag)::value == kPlain;
     auto next = [&](int t) { return PLAIN ? min(t, ntiles) : masks.next_live<KU>(t); };
     int t0 = next(0);
     issue_loads(min(32 * t0, N - 1), 0);
@@ -321,20 +333,21 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
       // past the last live stage the prefetch re-reads a valid stage that nobody uses
       const int t1 = next(t0 + KU);
       issue_loads(min(32 * t1, N - 1), 1);
-      compute_stage(plain_tag, 32 * t0, 0);
+      compute_stage(mode_tag, 32 * t0, 0);
       wait_dma();
       __syncthreads();
       if (t1 >= ntiles) break;
       t0 = next(t1 + KU);
       issue_loads(min(32 * t0, N - 1), 0);
-      compute_stage(plain_tag, 32 * t1, 1);
+      compute_stage(mode_tag, 32 * t1, 1);
       wait_dma();
       __syncthreads();
     }
   };
   // (a last stage with fewer than KU key tiles is not plain: its missing tiles are masked)
-  if (masks.all_plain() && ntiles % KU == 0) stage_loop(std::true_type{});
-  else stage_loop(std::false_type{});
+  if (masks.all_plain() && ntiles % KU == 0) stage_loop(std::integral_constant<int, kPlain>{});
+  else if (!any_flagged) stage_loop(std::integral_constant<int, kMasked>{});
+  else stage_loop(std::integral_constant<int, kGeneral>{});
 
   if (!wave_active) return;
 #pragma unroll

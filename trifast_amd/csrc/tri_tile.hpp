@@ -354,6 +354,11 @@ struct KeyTileMasks {
   }
 };
 
+// Compile-time versions of a stage loop, chosen per workgroup: every row attends to
+// every key (no mask work, no per-tile branch); some keys are masked but no row is
+// fully masked (one mask MFMA per tile, dead tiles skipped); anything.
+constexpr int kPlain = 0, kMasked = 1, kGeneral = 2;
+
 // Additive key mask of one 32-key tile in the transposed-score layout: value v
 // of lane group g is 0 when key cidx(v, g) is attended to and kNeg otherwise.
 TRI_DEV f32x16 mask_tile(uint32_t keepw, int g) {
