@@ -6,7 +6,7 @@ namespace tri {
 namespace {
 
 struct BwdBFamily {
-  static constexpr int kNumTiles = 6;
+  static constexpr int kNumTiles = 5;
   // {WJ, WK, 16 * GJ + GK}: GJ x GK waves per workgroup, each owning WJ x WK tiles of 32 x 32
   static constexpr int P(int tile, int which) {
     constexpr int t[kNumTiles][3] = {
@@ -15,7 +15,6 @@ struct BwdBFamily {
         {1, 1, 16 * 2 + 2},  // 2:  64 queries x  64 keys,  4 waves (fits every dtype / head dim)
         {1, 2, 16 * 4 + 2},  // 3: 128 queries x 128 keys,  8 waves
         {1, 1, 16 * 4 + 4},  // 4: 128 queries x 128 keys, 16 waves
-        {2, 2, 16 * 4 + 2},  // 5: 256 queries x 128 keys,  8 waves
     };
     return t[tile][which];
   }
