@@ -184,6 +184,14 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   OperandOffsets<T, D> ofk, ofq;
   ofk.init(perm32(jl), lane);
   ofq.init(jl, lane);
+  // the wave's own tiles inside the workgroup's rows: folded into the offsets once
+  ofk.shift(wk * WK * 32 * ROWB);
+  ofq.shift(wj * WJ * 32 * ROWB);
+  const int scalar_off = ((wj * WJ) * 32 + jl) * 4;  // this lane's query in the lse / delta words
+  const frag ones = resident_ones<T>();
+  Rank1<T> lrank[WJ], drank[WJ];
+#pragma unroll
+  for (int tj = 0; tj < WJ; ++tj) { lrank[tj].init(); drank[tj].init(); }
 
   const float c = a.c;
   const bool wave_live = j_wave < N && k_wave < N;
@@ -200,18 +208,18 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     for (int tj = 0; tj < WJ; ++tj) {
 #pragma unroll
       for (int s = 0; s < DS; ++s) {
-        qf[tj][s] = ofq.natural(st + OFF_Q + (wj * WJ + tj) * 32 * ROWB, s);
-        dof[tj][s] = ofq.natural(st + OFF_DO + (wj * WJ + tj) * 32 * ROWB, s);
+        qf[tj][s] = ofq.natural(st + OFF_Q + tj * 32 * ROWB, s);
+        dof[tj][s] = ofq.natural(st + OFF_DO + tj * 32 * ROWB, s);
       }
-      lf[tj] = rank1_operand<T>(reinterpret_cast<const uint32_t*>(st + OFF_LSE)[(wj * WJ + tj) * 32 + jl], g);
-      df[tj] = rank1_operand<T>(reinterpret_cast<const uint32_t*>(st + OFF_DELTA)[(wj * WJ + tj) * 32 + jl], g);
+      lf[tj] = lrank[tj].set(*reinterpret_cast<const uint32_t*>(st + OFF_LSE + tj * 128 + scalar_off), g);
+      df[tj] = drank[tj].set(*reinterpret_cast<const uint32_t*>(st + OFF_DELTA + tj * 128 + scalar_off), g);
     }
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk)
 #pragma unroll
       for (int s = 0; s < DS; ++s) {
-        kf[tk][s] = ofk.natural(st + OFF_K + (wk * WK + tk) * 32 * ROWB, s);
-        vf[tk][s] = ofk.natural(st + OFF_V + (wk * WK + tk) * 32 * ROWB, s);
+        kf[tk][s] = ofk.natural(st + OFF_K + tk * 32 * ROWB, s);
+        vf[tk][s] = ofk.natural(st + OFF_V + tk * 32 * ROWB, s);
       }
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk) {
@@ -221,7 +229,6 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
 #pragma unroll
       for (int tj = 0; tj < WJ; ++tj) {
         f32x16 s;
-        const frag ones = E::splat(1.0f);
         if (!flagged && keepw == 0xffffffffu) {
           s = E::mfma(ones, lf[tj], biasr[tj][tk]);
 #pragma unroll

@@ -135,6 +135,15 @@ TRI_DEV f16x4 lds_tr4(const _Float16* p) {
   const s16x4v r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TRI_LDS s16x4v*)(p));
   return __builtin_bit_cast(f16x4, r);
 }
+// the same from pointers that are already in the LDS address space
+TRI_DEV bf16x4 lds_tr4(TRI_LDS const __bf16* p) {
+  const s16x4v r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TRI_LDS s16x4v*)(p));
+  return __builtin_bit_cast(bf16x4, r);
+}
+TRI_DEV f16x4 lds_tr4(TRI_LDS const _Float16* p) {
+  const s16x4v r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TRI_LDS s16x4v*)(p));
+  return __builtin_bit_cast(f16x4, r);
+}
 
 // Operand with the contraction index in-lane, read from a natural row-major LDS
 // tile[rows = contraction index][cols]: the lane gets tile[row0 .. row0+7][col0 + lane%32]
@@ -210,16 +219,40 @@ TRI_DEV uint32_t split_word(float x) {
     return (uint32_t)__builtin_bit_cast(uint16_t, hi) | ((uint32_t)__builtin_bit_cast(uint16_t, lo) << 16);
   }
 }
+// The operand is kept in one variable whose first dword is replaced per use
+// (rank1_set), so that the zero slots are written once and not per tile.
+template <typename T>
+struct Rank1 {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  u32x4 v;
+  TRI_DEV void init() { v = u32x4{0u, 0u, 0u, 0u}; }
+  TRI_DEV typename Elem<T>::frag set(uint32_t word, int g) {
+    v[0] = g ? 0u : word;
+    if constexpr (sizeof(T) == 4) return __builtin_bit_cast(float, v[0]);
+    else return __builtin_bit_cast(typename Elem<T>::frag, v);
+  }
+};
 template <typename T>
 TRI_DEV typename Elem<T>::frag rank1_operand(uint32_t word, int g) {
-  const uint32_t w = g ? 0u : word;
+  Rank1<T> r;
+  r.init();
+  return r.set(word, g);
+}
+
+// A fragment of ones that the compiler keeps in registers (it would otherwise
+// rebuild the four registers from a constant at every use).
+template <typename T>
+TRI_DEV typename Elem<T>::frag resident_ones() {
+  typename Elem<T>::frag f = Elem<T>::splat(1.0f);
   if constexpr (sizeof(T) == 4) {
-    return __builtin_bit_cast(float, w);
+    asm volatile("" : "+v"(f));
   } else {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    const u32x4 v = {w, 0u, 0u, 0u};
-    return __builtin_bit_cast(typename Elem<T>::frag, v);
+    u32x4 v = __builtin_bit_cast(u32x4, f);
+    asm volatile("" : "+v"(v));
+    f = __builtin_bit_cast(typename Elem<T>::frag, v);
   }
+  return f;
 }
 
 TRI_DEV f32x16 zero16() {

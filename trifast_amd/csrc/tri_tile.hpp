@@ -133,6 +133,17 @@ struct OperandOffsets {
       }
     }
   }
+  // move every offset by a whole number of 32-row tiles (a wave's own part of a larger tile)
+  TRI_DEV void shift(int bytes) {
+    if constexpr (PRE) {
+#pragma unroll
+      for (int s = 0; s < DS; ++s) nat[s] += bytes;
+#pragma unroll
+      for (int mt = 0; mt < DM; ++mt) { tlo[mt] += bytes; thi[mt] += bytes; }
+    } else {
+      row += bytes / Tile::ROWB;
+    }
+  }
   // natural operand (head-dim index in-lane), MFMA step s, of the 32-row tile at `tile`
   TRI_DEV frag natural(const unsigned char* tile, int s) const {
     if constexpr (PRE) return *reinterpret_cast<const frag*>(tile + nat[s]);
