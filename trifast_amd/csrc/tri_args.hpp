@@ -52,9 +52,12 @@ struct BwdArgs {
   // [b*h, n, n] 32-bit workspaces indexed [i, j], written by the dq kernel for the
   // other two: the per-query terms of the backward as rank-1 MFMA operand words
   // (see split_word): delta = -rowsum(o * do); lse2 = -lse * sqrt(d), the
-  // log-sum-exp in the raw-score domain (ln n instead of lse for fully masked rows)
+  // log-sum-exp in the raw-score domain (ln n instead of lse for fully masked rows),
+  // for the db kernel; lse2l = -lse * log2(e), the same in the base-2 domain, for
+  // the dk/dv kernel
   uint32_t* delta;
   uint32_t* lse2;
+  uint32_t* lse2l;
   float* dbpart;             // [nchunks, b*h, n, n] fp32 partial db (nchunks > 1 only)
   void *dq, *dk, *dv, *db;
   Str5 sq, sk, sv, sdo;

@@ -11,10 +11,11 @@
 //   dv^T += dO^T P,   dk^T += Q^T dS,   dk = dk^T / sqrt(d),
 // whose A operands dO^T, Q^T come from the natural tiles through transposing LDS
 // reads.  The per-element additive terms ride on the matrix pipe: the bias tile
-// (fp32, raw-score domain, converted once per stage and shared by the R rows) is
-// the accumulator init of the score MFMA, and the per-query terms -lse*sqrt(d) and
-// -delta enter through one extra MFMA each (see rank1_operand), so that
-// P = exp2(c * acc) and dS = P * dP' are one multiply each.  Masked keys get a
+// (fp32, times log2(e), converted once per stage and shared by the R rows) is
+// the accumulator init of the score MFMA, the resident K operand is scaled by
+// log2(e)/sqrt(d) once, and the per-query terms -lse*log2(e) and -delta enter
+// through one extra MFMA each (see rank1_operand), so that P = exp2(acc) needs no
+// arithmetic before the exponential and dS = P * dP' is one multiply.  Masked keys get a
 // large negative score through one more MFMA (see mask_operand), which makes
 // their P and dS zero.
 //
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
   const T* vbh = reinterpret_cast<const T*>(a.v) + b * a.sv.b + h * a.sv.h;
   const T* dobh = reinterpret_cast<const T*>(a.dout) + b * a.sdo.b + h * a.sdo.h;
   const T* pack_bh = reinterpret_cast<const T*>(a.packk) + (int64_t)bh * a.NP * a.NP * 1024;
-  const float* lse2_bh = reinterpret_cast<const float*>(a.lse2) + (int64_t)bh * N * N;    // 32-bit words, moved as floats
+  const float* lse2_bh = reinterpret_cast<const float*>(a.lse2l) + (int64_t)bh * N * N;    // 32-bit words, moved as floats
   const float* delta_bh = reinterpret_cast<const float*>(a.delta) + (int64_t)bh * N * N;
 
   // per-row state: K and V tiles as B operands (lane owns key k_wave + kl).  A
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
     for (int s = 0; s < DS; ++s) {
       const int dofs = 2 * KP * s + KP * g;
       const int kc = min(key, N - 1);
-      kf[r][s] = flagged[r] ? E::zero() : *reinterpret_cast<const frag*>(kbh + i * a.sk.i + (int64_t)kc * a.sk.j + dofs);
+      kf[r][s] = flagged[r] ? E::zero() : scale_frag<T>(*reinterpret_cast<const frag*>(kbh + i * a.sk.i + (int64_t)kc * a.sk.j + dofs), a.c);
       vf[r][s] = *reinterpret_cast<const frag*>(vbh + i * a.sv.i + (int64_t)kc * a.sv.j + dofs);
     }
 #pragma unroll
@@ -157,12 +158,12 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
       if constexpr (sizeof(T) == 2) {
         const typename E::vec x = *reinterpret_cast<const typename E::vec*>(src + r2 * (BIAS_B / 2) + lane * 16);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) bv[8 * r2 + e] = (float)x[e] * a.sqrt_d;
+        for (int e = 0; e < 8; ++e) bv[8 * r2 + e] = (float)x[e] * kLog2e;
       } else {
         const f32x4 x0 = *reinterpret_cast<const f32x4*>(src + r2 * (BIAS_B / 2) + lane * 16);
         const f32x4 x1 = *reinterpret_cast<const f32x4*>(src + r2 * (BIAS_B / 2) + 1024 + lane * 16);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { bv[8 * r2 + e] = x0[e] * a.sqrt_d; bv[8 * r2 + 4 + e] = x1[e] * a.sqrt_d; }
+        for (int e = 0; e < 4; ++e) { bv[8 * r2 + e] = x0[e] * kLog2e; bv[8 * r2 + 4 + e] = x1[e] * kLog2e; }
       }
     }
     return bv;
@@ -172,8 +173,6 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
   auto query_word = [&](const unsigned char* st, int off, int r, int u) -> uint32_t {
     return reinterpret_cast<const uint32_t*>(st + off)[r * BJ + 32 * u + perm32(kl)];
   };
-
-  const float c = a.c;
 
   // One stage of compute.  The JU*R tiles run as a software pipeline inside the
   // wave: the two MFMA chains (scores, dP) of tile t+1 are issued before the
@@ -187,7 +186,7 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
 #pragma unroll
     for (int u = 0; u < JU; ++u) biasv[u] = bias_from_lds(st, u);
 
-    // scores: bias tile (accumulator init) - lse*sqrt(d) (per query, one MFMA) + Q K^T;
+    // base-2 scores: bias tile (accumulator init) - lse*log2(e) (per query, one MFMA) + Q (cK)^T;
     // dP - delta: -delta (per query, one MFMA) + dO V^T
     auto chains = [&](int t, f32x16& sc, f32x16& dp) {
       const int u = t / R, r = t % R;
@@ -230,7 +229,7 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
         float p[16], ds[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          p[v] = fast_exp2(sc[v] * c);
+          p[v] = fast_exp2(sc[v]);
           ds[v] = p[v] * dp[v];
         }
 #pragma unroll

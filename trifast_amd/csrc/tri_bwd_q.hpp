@@ -104,6 +104,7 @@ __global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(co
       // the per-query terms of the other two backward kernels, as rank-1 MFMA operand words
       a.delta[((int64_t)bh * N + i) * N + j] = split_word<T>(-dsum);
       a.lse2[((int64_t)bh * N + i) * N + j] = split_word<T>(-lse2[r] * (kLn2 * a.sqrt_d));
+      a.lse2l[((int64_t)bh * N + i) * N + j] = split_word<T>(-lse2[r]);
     }
 #pragma unroll
     for (int v = 0; v < 16; ++v) ndelta[r][v] = -dsum;

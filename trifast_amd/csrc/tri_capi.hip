@@ -129,7 +129,7 @@ float dtype_min(int dtype) {
   }
 }
 
-// workspace layout: keep words | row flags | packq | (backward only) packk | -delta | lse2 | db partials
+// workspace layout: keep words | row flags | packq | (backward only) packk | -delta | lse2 | lse2l | db partials
 struct Workspace {
   uint32_t* keep;
   uint32_t* rowflag;
@@ -137,6 +137,7 @@ struct Workspace {
   void* packk;
   uint32_t* delta;
   uint32_t* lse2;
+  uint32_t* lse2l;
   float* dbpart;
   int nwords, np;
 };
@@ -166,6 +167,8 @@ Workspace carve(void* ws, int64_t b, int64_t h, int64_t n, int dtype) {
   w.delta = reinterpret_cast<uint32_t*>(p);
   p += align256(b * h * n * n * 4);
   w.lse2 = reinterpret_cast<uint32_t*>(p);
+  p += align256(b * h * n * n * 4);
+  w.lse2l = reinterpret_cast<uint32_t*>(p);
   p += align256(b * h * n * n * 4);
   w.dbpart = reinterpret_cast<float*>(p);
   w.nwords = (int)nwords;
@@ -300,7 +303,7 @@ int64_t trifast_bwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, 
   (void)d;
   if (b < 1 || h < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
   const int64_t chunks = tri::bwd_b_chunks(n, b * h);
-  return ws_mask_bytes(b, n) + 2 * ws_pack_bytes(b, h, n, dtype) + 2 * align256(b * h * n * n * 4) +
+  return ws_mask_bytes(b, n) + 2 * ws_pack_bytes(b, h, n, dtype) + 3 * align256(b * h * n * n * 4) +
          (chunks > 1 ? align256(chunks * b * h * n * n * 4) : 0);
 }
 
@@ -390,7 +393,7 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   a.q = q; a.k = k; a.v = v; a.o = o; a.dout = dout;
   a.packq = w.packq; a.packk = w.packk;
   a.lse = lse;
-  a.keep = w.keep; a.rowflag = w.rowflag; a.delta = w.delta; a.lse2 = w.lse2; a.dbpart = w.dbpart;
+  a.keep = w.keep; a.rowflag = w.rowflag; a.delta = w.delta; a.lse2 = w.lse2; a.lse2l = w.lse2l; a.dbpart = w.dbpart;
   a.BH = (int)(b * h);
   a.nchunks = tri::bwd_b_chunks(n, b * h);
   a.rows_per_chunk = (int)((n + a.nchunks - 1) / a.nchunks);

@@ -255,6 +255,19 @@ TRI_DEV typename Elem<T>::frag resident_ones() {
   return f;
 }
 
+// every element of an operand fragment times s, rounded back to T
+template <typename T>
+TRI_DEV typename Elem<T>::frag scale_frag(typename Elem<T>::frag f, float s) {
+  if constexpr (sizeof(T) == 4) {
+    return f * s;
+  } else {
+    float x[Elem<T>::KP];
+#pragma unroll
+    for (int e = 0; e < Elem<T>::KP; ++e) x[e] = (float)f[e] * s;
+    return Elem<T>::pack(x);
+  }
+}
+
 TRI_DEV f32x16 zero16() {
   f32x16 z;
 #pragma unroll
