@@ -24,7 +24,7 @@ struct BwdBFamily {
     constexpr int BJ = GJ * WJ * 32, BKB = GK * WK * 32;
     // registers of one row's operands, the db accumulators and the bias tiles
     constexpr int frag_regs = (2 * WJ + 2 * WK) * (D / 2) * (int)sizeof(T) / 4;
-    constexpr int stage = (2 * BJ + 2 * BKB) * D * (int)sizeof(T) + 2 * BJ * 4 + 256;
+    constexpr int stage = bwd_b_stage_bytes(BJ, BKB, LdsTile<T, D>::ROWB);
     // ring of row buffers: up to 4 (loads run 3 rows ahead), as many as fit
     constexpr int nbuf = 4 * stage <= kMaxLds ? 4 : (3 * stage <= kMaxLds ? 3 : (2 * stage <= kMaxLds ? 2 : 1));
     // the smallest tile always runs (at the price of register spills for large head dims)

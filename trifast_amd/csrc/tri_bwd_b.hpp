@@ -33,6 +33,9 @@
 
 namespace tri {
 
+// LDS bytes of one stage (one pair row) of the kernel below
+constexpr int bwd_b_stage_bytes(int BJ, int BKB, int ROWB) { return 2 * (BJ * 4 + 256) + 512 + (2 * BJ + 2 * BKB) * ROWB; }
+
 template <typename T, int D, int GJ, int GK, int WJ, int WK, int NBUF>
 __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a) {
   using E = Elem<T>;
@@ -43,14 +46,18 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   constexpr int NW = GJ * GK;
   constexpr int BJ = GJ * WJ * 32, BKB = GK * WK * 32;  // queries / keys per workgroup
   constexpr int ROWB = Tile::ROWB;
-  // one stage: Q rows | dO rows | K rows | V rows | lse2[BJ] | -delta[BJ] | row meta
-  // (64 words: the WKW keep words of the key block, then the row's flag)
-  constexpr int OFF_Q = 0, OFF_DO = BJ * ROWB, OFF_K = 2 * BJ * ROWB, OFF_V = OFF_K + BKB * ROWB;
-  constexpr int OFF_LSE = OFF_V + BKB * ROWB, OFF_DELTA = OFF_LSE + BJ * 4;
-  constexpr int OFF_META = OFF_DELTA + BJ * 4;
-  constexpr int STAGE = OFF_META + 256;
+  // one stage: lse2[BJ] | 64 zero words | -delta[BJ] | 64 zero words | keep words of the
+  // key block (64 words) | the row's flag (64 copies) | Q rows | dO rows | K rows | V rows.
+  // The small arrays come first so that their offsets in every ring buffer fit the
+  // 16-bit immediate of an LDS read; the zero words are what lanes 32..63 read as
+  // their (empty) half of a rank-1 operand.
+  constexpr int OFF_LSE = 0, OFF_DELTA = OFF_LSE + BJ * 4 + 256;
+  constexpr int OFF_META = OFF_DELTA + BJ * 4 + 256, OFF_FLAG = OFF_META + 256;
+  constexpr int OFF_Q = OFF_FLAG + 256, OFF_DO = OFF_Q + BJ * ROWB, OFF_K = OFF_DO + BJ * ROWB, OFF_V = OFF_K + BKB * ROWB;
+  constexpr int STAGE = OFF_V + BKB * ROWB;
+  static_assert(STAGE == bwd_b_stage_bytes(BJ, BKB, ROWB), "the launcher sizes LDS with bwd_b_stage_bytes");
   constexpr int WKW = BKB / 32;
-  static_assert(WKW < 64, "keep words and the row flag share one 64-lane load");
+  static_assert(WKW <= 64, "the keep words of the key block are one 64-lane load");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
 
@@ -101,19 +108,23 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     for (int tk = 0; tk < WK; ++tk) dbacc[tj][tk] = zero16();
 
   // The loads of one row, as a flat list of wave-sized items: 1 KiB pieces of the Q,
-  // dO, K, V tiles (16 bytes per lane), 64-float pieces of lse2 and -delta, and the
-  // 64-word row meta (4 bytes per lane).  Wave w takes items w, w + NW, ...; every
+  // dO, K, V tiles (16 bytes per lane), 64-float pieces of lse2 and -delta, the keep
+  // words of the key block and the row's flag (4 bytes per lane).  Wave w takes items w, w + NW, ...; every
   // wave issues exactly XN loads per row (a wave that runs out repeats the last
   // item, which rewrites the same bytes), so "all but the newest K rows have
   // landed" is one s_waitcnt vmcnt(K * XN) for every wave.  Queries and keys past
   // the end are clamped (they feed db entries that are never stored).
   constexpr int CPR = Tile::CPR;
   constexpr int GQ = BJ * CPR / 64, GKK = BKB * CPR / 64, GF = BJ / 64;
-  constexpr int TOT = 2 * GQ + 2 * GKK + 2 * GF + 1;
+  constexpr int TOT = 2 * GQ + 2 * GKK + 2 * GF + 2;
   constexpr int XN = (TOT + NW - 1) / NW;
   static_assert(BJ * CPR % 64 == 0 && BKB * CPR % 64 == 0 && BJ % 64 == 0, "whole wave loads only");
+  auto uniform64 = [](int64_t x) -> int64_t {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)x), hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)x >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+  };
   const char* item_ptr[XN];   // source of the next row to load (per lane)
-  int64_t item_step[XN];      // bytes from one pair row to the next (per lane: the meta item mixes two arrays)
+  int64_t item_step[XN];      // bytes from one pair row to the next (wave-uniform, in scalar registers)
   int item_lds[XN];           // destination offset inside a stage (wave-uniform)
   bool item_wide[XN];         // 16-byte (tile) or 4-byte (float / meta) lanes
   {
@@ -122,7 +133,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
       const int p = gi * 64 + lane;
       const int r = p / CPR, cc = (p % CPR) ^ Tile::swz(r);
       item_ptr[x] = reinterpret_cast<const char*>(base + (int64_t)min(blk + r, N - 1) * srow + cc * Tile::VEC) + (int64_t)i_begin * si * es;
-      item_step[x] = si * es;
+      item_step[x] = uniform64(si * es);
       item_lds[x] = off + gi * 1024;
       item_wide[x] = true;
     };
@@ -142,17 +153,20 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
         const int gi = f % GF;
         const float* base = (f < GF) ? lse2_bh : delta_bh;
         item_ptr[x] = reinterpret_cast<const char*>(base + (int64_t)i_begin * N + min(j_blk + gi * 64 + lane, N - 1));
-        item_step[x] = (int64_t)N * 4;
+        item_step[x] = uniform64((int64_t)N * 4);
         item_lds[x] = ((f < GF) ? OFF_LSE : OFF_DELTA) + gi * 256;
         item_wide[x] = false;
-      } else {
-        // lanes 0..WKW-1: keep words of this key block; lane WKW (and up): the row flag
-        const bool is_flag = lane >= WKW;
-        const uint32_t* src = is_flag ? a.rowflag + (int64_t)b * N + i_begin
-                                      : a.keep + ((int64_t)b * N + i_begin) * a.nwords + min(k_blk / 32 + lane, a.nwords - 1);
-        item_ptr[x] = reinterpret_cast<const char*>(src);
-        item_step[x] = is_flag ? 4 : (int64_t)a.nwords * 4;
+      } else if (it < TOT - 1) {
+        // the keep words of this key block (lanes past the block repeat the last word)
+        item_ptr[x] = reinterpret_cast<const char*>(a.keep + ((int64_t)b * N + i_begin) * a.nwords + min(k_blk / 32 + min(lane, WKW - 1), a.nwords - 1));
+        item_step[x] = uniform64((int64_t)a.nwords * 4);
         item_lds[x] = OFF_META;
+        item_wide[x] = false;
+      } else {
+        // the row's flag, the same word for every lane
+        item_ptr[x] = reinterpret_cast<const char*>(a.rowflag + (int64_t)b * N + i_begin);
+        item_step[x] = 4;
+        item_lds[x] = OFF_FLAG;
         item_wide[x] = false;
       }
     }
@@ -168,7 +182,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     for (int x = 0; x < XN; ++x) {
       if (item_wide[x]) __builtin_amdgcn_global_load_lds((const TRI_G1 void*)item_ptr[x], (TRI_L3 void*)(st + item_lds[x]), 16, 0, 0);
       else __builtin_amdgcn_global_load_lds((const TRI_G1 void*)item_ptr[x], (TRI_L3 void*)(st + item_lds[x]), 4, 0, 0);
-      if (advance) item_ptr[x] += item_step[x];
+      item_ptr[x] += advance ? item_step[x] : 0;
     }
   };
   // wait until at most the newest `K` rows of this wave's loads are in flight and
@@ -187,7 +201,37 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   // the wave's own tiles inside the workgroup's rows: folded into the offsets once
   ofk.shift(wk * WK * 32 * ROWB);
   ofq.shift(wj * WJ * 32 * ROWB);
-  const int scalar_off = ((wj * WJ) * 32 + jl) * 4;  // this lane's query in the lse / delta words
+  // (absolute LDS addresses from here on: the block's address is folded in once)
+  ofk.make_absolute(tri_smem);
+  ofq.make_absolute(tri_smem);
+  ofk.pin();
+  ofq.pin();
+  // this lane's query in the lse / delta words (lanes 32..63: the zero words behind
+  // them), as an absolute LDS address
+  int scalar_off = (g ? BJ * 4 : ((wj * WJ) * 32 + jl) * 4) + (int)(uintptr_t)(TRI_L3 const unsigned char*)tri_smem;
+  asm volatile("" : "+v"(scalar_off));
+  if (wave == 0) {
+#pragma unroll
+    for (int u = 0; u < NBUF; ++u) {
+      reinterpret_cast<uint32_t*>(tri_smem + u * STAGE + OFF_LSE + BJ * 4)[lane] = 0u;
+      reinterpret_cast<uint32_t*>(tri_smem + u * STAGE + OFF_DELTA + BJ * 4)[lane] = 0u;
+    }
+  }
+  // LDS reads take a 16-bit immediate offset: for ring buffers past the first 64 KiB a
+  // second set of lane offsets, moved up by two stages, keeps the buffer's offset an
+  // immediate (the reads of those buffers would otherwise each need an address add)
+  constexpr bool kHighSet = NBUF > 2 && sizeof(T) == 2;
+  constexpr int HIGH = kHighSet ? 2 * STAGE : 0;
+  OperandOffsets<T, D> ofk_hi = ofk, ofq_hi = ofq;
+  int scalar_off_hi = scalar_off;
+  if constexpr (kHighSet) {
+    ofk_hi.shift(HIGH);
+    ofq_hi.shift(HIGH);
+    ofk_hi.pin();
+    ofq_hi.pin();
+    scalar_off_hi += HIGH;
+    asm volatile("" : "+v"(scalar_off_hi));
+  }
   const frag ones = resident_ones<T>();
   Rank1<T> lrank[WJ], drank[WJ];
 #pragma unroll
@@ -199,27 +243,32 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   auto compute_row = [&](int buf) __attribute__((always_inline)) {
     const unsigned char* st = tri_smem + buf * STAGE;
     const uint32_t* meta = reinterpret_cast<const uint32_t*>(st + OFF_META);
+    const bool high = kHighSet && buf >= 2;  // (a constant once the ring loop is unrolled)
+    const int sl = buf * STAGE - (high ? HIGH : 0);  // offset of the buffer for reads through the lane offsets
+    const OperandOffsets<T, D>& oq = high ? ofq_hi : ofq;
+    const OperandOffsets<T, D>& ok = high ? ofk_hi : ofk;
+    const int soff = high ? scalar_off_hi : scalar_off;
     // (wave-uniform values are pinned to scalar registers so that the branches on
     // them are real branches and not lane masks)
-    const bool flagged = __builtin_amdgcn_readfirstlane(meta[WKW]) != 0;
+    const bool flagged = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const uint32_t*>(st + OFF_FLAG)) != 0;
     frag qf[WJ][DS], dof[WJ][DS], kf[WK][DS], vf[WK][DS];
     frag lf[WJ], df[WJ];  // per-query terms -lse*sqrt(d) and -delta as rank-1 MFMA operands
 #pragma unroll
     for (int tj = 0; tj < WJ; ++tj) {
 #pragma unroll
       for (int s = 0; s < DS; ++s) {
-        qf[tj][s] = ofq.natural(st + OFF_Q + tj * 32 * ROWB, s);
-        dof[tj][s] = ofq.natural(st + OFF_DO + tj * 32 * ROWB, s);
+        qf[tj][s] = oq.natural_at(sl + OFF_Q + tj * 32 * ROWB, s);
+        dof[tj][s] = oq.natural_at(sl + OFF_DO + tj * 32 * ROWB, s);
       }
-      lf[tj] = lrank[tj].set(*reinterpret_cast<const uint32_t*>(st + OFF_LSE + tj * 128 + scalar_off), g);
-      df[tj] = drank[tj].set(*reinterpret_cast<const uint32_t*>(st + OFF_DELTA + tj * 128 + scalar_off), g);
+      lf[tj] = lrank[tj].set(*reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_LSE + tj * 128 + soff)));
+      df[tj] = drank[tj].set(*reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_DELTA + tj * 128 + soff)));
     }
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk)
 #pragma unroll
       for (int s = 0; s < DS; ++s) {
-        kf[tk][s] = ofk.natural(st + OFF_K + tk * 32 * ROWB, s);
-        vf[tk][s] = ofk.natural(st + OFF_V + tk * 32 * ROWB, s);
+        kf[tk][s] = ok.natural_at(sl + OFF_K + tk * 32 * ROWB, s);
+        vf[tk][s] = ok.natural_at(sl + OFF_V + tk * 32 * ROWB, s);
       }
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk) {

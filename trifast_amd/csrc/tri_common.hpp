@@ -226,8 +226,10 @@ struct Rank1 {
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   u32x4 v;
   TRI_DEV void init() { v = u32x4{0u, 0u, 0u, 0u}; }
-  TRI_DEV typename Elem<T>::frag set(uint32_t word, int g) {
-    v[0] = g ? 0u : word;
+  TRI_DEV typename Elem<T>::frag set(uint32_t word, int g) { return set(g ? 0u : word); }
+  // `word` is already zero in lanes 32..63
+  TRI_DEV typename Elem<T>::frag set(uint32_t word) {
+    v[0] = word;
     if constexpr (sizeof(T) == 4) return __builtin_bit_cast(float, v[0]);
     else return __builtin_bit_cast(typename Elem<T>::frag, v);
   }

@@ -117,6 +117,7 @@ struct OperandOffsets {
   int nat[PRE ? DS : 1];
   int tlo[PRE ? DM : 1], thi[PRE ? DM : 1];
   int row, lane;
+  const unsigned char* base = nullptr;
   // `row_in_tile`: the row of a 32-row tile this lane reads as a natural operand
   TRI_DEV void init(int row_in_tile, int lane_) {
     row = row_in_tile;
@@ -143,6 +144,29 @@ struct OperandOffsets {
     } else {
       row += bytes / Tile::ROWB;
     }
+  }
+  // make the offsets opaque to the compiler: it then keeps them in registers as they
+  // are instead of rebuilding them from another instance plus a constant
+  TRI_DEV void pin() {
+    if constexpr (PRE) {
+#pragma unroll
+      for (int s = 0; s < DS; ++s) asm volatile("" : "+v"(nat[s]));
+    }
+  }
+  // Fold the address of the workgroup's LDS block into the offsets: natural_at() then
+  // reads from absolute LDS addresses, one register plus an immediate per read.
+  TRI_DEV void make_absolute(const unsigned char* lds_base) {
+    base = lds_base;
+    if constexpr (PRE) {
+      const int b0 = (int)(uintptr_t)(TRI_L3 const unsigned char*)lds_base;
+#pragma unroll
+      for (int s = 0; s < DS; ++s) nat[s] += b0;
+    }
+  }
+  // natural operand of the 32-row tile `byte_offset` bytes into the block (after make_absolute)
+  TRI_DEV frag natural_at(int byte_offset, int s) const {
+    if constexpr (PRE) return *reinterpret_cast<TRI_L3 const frag*>((uintptr_t)(uint32_t)(nat[s] + byte_offset));
+    else return Tile::operand(base + byte_offset, row, s, lane >> 5);
   }
   // natural operand (head-dim index in-lane), MFMA step s, of the 32-row tile at `tile`
   TRI_DEV frag natural(const unsigned char* tile, int s) const {
