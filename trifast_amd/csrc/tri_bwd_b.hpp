@@ -213,7 +213,9 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   if (wave == 0) {
 #pragma unroll
     for (int u = 0; u < NBUF; ++u) {
-      reinterpret_cast<uint32_t*>(tri_smem + u * STAGE + OFF_LSE + BJ * 4)[lane] = 0u;
+      // (the lse word shares its MFMA with the key mask: in fp32 the slot of lanes 32..63
+      // belongs to the mask and the queries operand holds a one there)
+      reinterpret_cast<uint32_t*>(tri_smem + u * STAGE + OFF_LSE + BJ * 4)[lane] = sizeof(T) == 4 ? OffsetMask<T>::ones_dword() : 0u;
       reinterpret_cast<uint32_t*>(tri_smem + u * STAGE + OFF_DELTA + BJ * 4)[lane] = 0u;
     }
   }
@@ -233,9 +235,19 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     asm volatile("" : "+v"(scalar_off_hi));
   }
   const frag ones = resident_ones<T>();
-  Rank1<T> lrank[WJ], drank[WJ];
+  // -lse per query and the key mask share one MFMA (see OffsetMask), -delta has its own
+  typename OffsetMask<T>::Queries lrank[WJ];
+  Rank1<T> drank[WJ];
 #pragma unroll
-  for (int tj = 0; tj < WJ; ++tj) { lrank[tj].init(); drank[tj].init(); }
+  for (int tj = 0; tj < WJ; ++tj) { lrank[tj].init(0u, g); drank[tj].init(); }
+  typename OffsetMask<T>::Keys kop;
+  kop.init(perm32(jl), g);
+  frag kop_plain = kop.plain();
+  if constexpr (sizeof(T) == 2) {
+    typename OffsetMask<T>::u32x4 t = __builtin_bit_cast(typename OffsetMask<T>::u32x4, kop_plain);
+    asm volatile("" : "+v"(t));  // kept in registers, not rebuilt from constants per use
+    kop_plain = __builtin_bit_cast(frag, t);
+  }
 
   const float c = a.c;
   const bool wave_live = j_wave < N && k_wave < N;
@@ -260,7 +272,8 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
         qf[tj][s] = oq.natural_at(sl + OFF_Q + tj * 32 * ROWB, s);
         dof[tj][s] = oq.natural_at(sl + OFF_DO + tj * 32 * ROWB, s);
       }
-      lf[tj] = lrank[tj].set(*reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_LSE + tj * 128 + soff)));
+      lrank[tj].set_raw(*reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_LSE + tj * 128 + soff)));
+      lf[tj] = lrank[tj].get();
       df[tj] = drank[tj].set(*reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_DELTA + tj * 128 + soff)));
     }
 #pragma unroll
@@ -278,23 +291,17 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
 #pragma unroll
       for (int tj = 0; tj < WJ; ++tj) {
         f32x16 s;
-        if (!flagged && keepw == 0xffffffffu) {
-          s = E::mfma(ones, lf[tj], biasr[tj][tk]);
+        // Each case ends in the MFMA that defines s from the bias tile in place (a
+        // select between accumulator inits would copy 16 registers).
+        if (!flagged) {
+          if (keepw == 0xffffffffu) s = E::mfma(kop_plain, lf[tj], biasr[tj][tk]);
+          else s = E::mfma(kop.masked(keepw), lf[tj], biasr[tj][tk]);  // masked keys: large negative score
 #pragma unroll
           for (int sd = 0; sd < DS; ++sd) s = E::mfma(kf[tk][sd], qf[tj][sd], s);
         } else {
-          // rare: a fully masked row ignores q.k and the bias; masked keys get a
-          // large negative score.  (Kept a real branch: a select between the two
-          // accumulator inits would copy 16 registers in the common case.)
+          // rare: a fully masked row ignores q.k and the bias
           asm volatile("" ::);
-          if (flagged) s = zero16();
-          else s = biasr[tj][tk];
-          if (keepw != 0xffffffffu) s = E::mfma(mask_operand<T>(keepw, perm32(jl)), ones, s);
-          s = E::mfma(ones, lf[tj], s);
-          if (!flagged) {
-#pragma unroll
-            for (int sd = 0; sd < DS; ++sd) s = E::mfma(kf[tk][sd], qf[tj][sd], s);
-          }
+          s = E::mfma(kop.masked(keepw), lf[tj], zero16());
         }
         f32x16 dp = E::mfma(ones, df[tj], zero16());
 #pragma unroll

@@ -14,10 +14,10 @@
 // (fp32, times log2(e), converted once per stage and shared by the R rows) is
 // the accumulator init of the score MFMA, the resident K operand is scaled by
 // log2(e)/sqrt(d) once, and the per-query terms -lse*log2(e) and -delta enter
-// through one extra MFMA each (see rank1_operand), so that P = exp2(acc) needs no
-// arithmetic before the exponential and dS = P * dP' is one multiply.  Masked keys get a
-// large negative score through one more MFMA (see mask_operand), which makes
-// their P and dS zero.
+// through one extra MFMA each (see rank1_operand, OffsetMask), so that P = exp2(acc)
+// needs no arithmetic before the exponential and dS = P * dP' is one multiply.  Masked
+// keys get a large negative score from the MFMA that adds -lse, which makes their P
+// and dS zero.
 //
 // Replaces _bwd_kv of reference src/trifast/triton.py:143-263.
 #pragma once
@@ -75,8 +75,9 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
   // per-row state: K and V tiles as B operands (lane owns key k_wave + kl).  A
   // fully masked row drops the q.k and bias terms from its scores: its K operand
   // is zero here (K itself is not needed for dk, dv) and it skips the bias.
-  bool flagged[R], tile_live[R], tile_mixed[R];
-  frag kf[R][DS], vf[R][DS], maskf[R];
+  bool flagged[R], tile_live[R];
+  frag kf[R][DS], vf[R][DS];
+  frag keyop[R];  // ones | mask element of this lane's key: B operand of the offset-and-mask MFMA
   f32x16 dkacc[R][DM], dvacc[R][DM];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -87,8 +88,11 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
     const int w = k_wave >> 5;
     const uint32_t word = __builtin_amdgcn_readfirstlane((wave_active && w < a.nwords) ? a.keep[((int64_t)b * N + i) * a.nwords + w] : 0u);
     tile_live[r] = word != 0;
-    tile_mixed[r] = word != 0xffffffffu;
-    maskf[r] = mask_operand<T>(word, kl);
+    {
+      typename OffsetMask<T>::Keys ko;
+      ko.init(kl, g);
+      keyop[r] = ko.masked(word);
+    }
 #pragma unroll
     for (int s = 0; s < DS; ++s) {
       const int dofs = 2 * KP * s + KP * g;
@@ -170,6 +174,8 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
   };
   // the per-query operand word (lse or delta term) of the query this lane's A
   // operand row stands for, in tile (r, u)
+  typename OffsetMask<T>::Queries lseop;  // the query's -lse word | ones: A operand of that MFMA
+  lseop.init(0u, g);
   auto query_word = [&](const unsigned char* st, int off, int r, int u) -> uint32_t {
     return reinterpret_cast<const uint32_t*>(st + off)[r * BJ + 32 * u + perm32(kl)];
   };
@@ -198,17 +204,16 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void 
         if (jt0 + 32 * u + perm32(kl) >= N) lw = split_word<T>(E::kMaskElem);
       }
       const frag ones = E::splat(1.0f);
-      if (!flagged[r] && !tile_mixed[r]) {
-        sc = E::mfma(rank1_operand<T>(lw, g), ones, biasv[u]);
+      // -lse per query and the key mask through one MFMA (see OffsetMask; the roles of
+      // the two operands are swapped here: rows are queries, columns are keys)
+      lseop.set(lw, g);
+      if (!flagged[r]) {
+        sc = E::mfma(lseop.get(), keyop[r], biasv[u]);
       } else {
         // rare: kept a real branch so that the common case starts from the bias
         // tile in place (a select between the two inits would copy 16 registers)
         asm volatile("" ::);
-        f32x16 init;
-        if (flagged[r]) init = zero16();
-        else init = biasv[u];
-        if (tile_mixed[r]) init = E::mfma(ones, maskf[r], init);
-        sc = E::mfma(rank1_operand<T>(lw, g), ones, init);
+        sc = E::mfma(lseop.get(), keyop[r], zero16());
       }
       dp = E::mfma(rank1_operand<T>(query_word(st, OFF_DELTA, r, u), g), ones, zero16());
 #pragma unroll

@@ -19,7 +19,7 @@ struct BwdQFamily {
   }
   template <typename T, int D, int NW, int R, int BK>
   static hipError_t run(const BwdArgs& a, int bh, hipStream_t st, bool dry) {
-    constexpr int lds = 2 * (2 * R * BK * D + NW * (BK / 32) * 1024) * (int)sizeof(T);
+    constexpr int lds = 2 * ((2 * R * BK * D + NW * (BK / 32) * 1024) * (int)sizeof(T) + 256);
     // Q, dO operands and the dq accumulator of the R rows stay in registers
     constexpr int acc_regs = R * (((D + 31) / 32) * 16 + 2 * (D / 2) * (int)sizeof(T) / 4);
     if constexpr (lds <= kMaxLds && (acc_regs <= 160 || R == 1)) {

@@ -276,8 +276,8 @@ int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype)
   // falls back to tile 0 and then to the first tile that supports it.
   int pick = 0;
   switch (kernel) {
-    case TRIFAST_KERNEL_FWD: pick = n <= 64 ? 0 : 3; break;     // 4 pair rows share a bias tile
-    case TRIFAST_KERNEL_BWD_Q: pick = n <= 64 ? 0 : 1; break;   // 2 pair rows, 64 keys per stage
+    case TRIFAST_KERNEL_FWD: pick = n <= 64 ? 0 : 4; break;     // 2 pair rows share a bias tile, 3 waves per SIMD
+    case TRIFAST_KERNEL_BWD_Q: pick = n <= 64 ? 0 : 2; break;   // 2 pair rows, 32 keys per stage
     case TRIFAST_KERNEL_BWD_KV: pick = n <= 64 ? 0 : 1; break;  // 2 pair rows, 32 queries per stage
     case TRIFAST_KERNEL_BWD_B: pick = n <= 128 ? 2 : 4; break;  // 128 x 128 block of 16 waves; 64 x 64 at small n
 

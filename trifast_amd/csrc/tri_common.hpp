@@ -219,6 +219,84 @@ TRI_DEV uint32_t split_word(float x) {
     return (uint32_t)__builtin_bit_cast(uint16_t, hi) | ((uint32_t)__builtin_bit_cast(uint16_t, lo) << 16);
   }
 }
+// the value a split word stands for (what the MFMA adds for it)
+template <typename T>
+TRI_DEV float unsplit_word(uint32_t w) {
+  if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(float, w);
+  } else {
+    const T hi = __builtin_bit_cast(T, (uint16_t)(w & 0xffffu));
+    const T lo = __builtin_bit_cast(T, (uint16_t)(w >> 16));
+    return (float)hi + (float)lo;
+  }
+}
+
+// Per-query offset and key mask through ONE extra MFMA of a transposed score tile
+// (rows = keys, columns = queries): the contraction slots are shared between the two
+// rank-1 terms.
+//   slots of dword 0 of lane group 0: keys operand 1,      queries operand: split word
+//   slots of dword 1 of every lane:   keys operand: mask element of the key (or 0),
+//                                     queries operand 1
+// (fp32 has one slot per lane group: group 0 carries the offset, group 1 the mask.)
+// Both operands are kept in place: per tile only the mask dword of the keys operand
+// changes, and the word of the queries operand changes when the offset does.
+template <typename T>
+struct OffsetMask {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef typename Elem<T>::frag frag;
+  static TRI_DEV uint32_t ones_dword() {
+    if constexpr (sizeof(T) == 4) return __builtin_bit_cast(uint32_t, 1.0f);
+    else return (uint32_t)__builtin_bit_cast(uint16_t, (T)1.0f) * 0x10001u;
+  }
+  static TRI_DEV uint32_t mask_dword() {
+    if constexpr (sizeof(T) == 4) return __builtin_bit_cast(uint32_t, Elem<T>::kMaskElem);
+    else return (uint32_t)__builtin_bit_cast(uint16_t, (T)Elem<T>::kMaskElem) * 0x10001u;
+  }
+  static TRI_DEV frag as_frag(u32x4 v) {
+    if constexpr (sizeof(T) == 4) return __builtin_bit_cast(float, v[0]);
+    else return __builtin_bit_cast(frag, v);
+  }
+  // keys operand of the lane whose operand row stands for key `key_in_tile`
+  struct Keys {
+    u32x4 v;
+    uint32_t bit;
+    int g;
+    TRI_DEV void init(int key_in_tile, int g_) {
+      g = g_;
+      bit = 1u << key_in_tile;
+      v = u32x4{g ? 0u : ones_dword(), 0u, 0u, 0u};
+    }
+    // no key of the tile is masked
+    TRI_DEV frag plain() const { return as_frag(v); }
+    // bit k of keepw set = key k of the tile is attended
+    TRI_DEV frag masked(uint32_t keepw) {
+      const uint32_t m = (keepw & bit) ? 0u : mask_dword();
+      if constexpr (sizeof(T) == 4) {
+        u32x4 t = v;
+        if (g) t[0] = m;
+        return as_frag(t);
+      } else {
+        v[1] = m;
+        return as_frag(v);
+      }
+    }
+  };
+  // queries operand of the lane that owns a query
+  struct Queries {
+    u32x4 v;
+    TRI_DEV void init(uint32_t word, int g) {
+      if constexpr (sizeof(T) == 4) v = u32x4{g ? ones_dword() : word, 0u, 0u, 0u};
+      else v = u32x4{g ? 0u : word, ones_dword(), 0u, 0u};
+    }
+    TRI_DEV void set(uint32_t word, int g) {
+      if (!g) v[0] = word;
+    }
+    // `word` already holds what lanes 32..63 need (zero; fp32: one)
+    TRI_DEV void set_raw(uint32_t word) { v[0] = word; }
+    TRI_DEV frag get() const { return as_frag(v); }
+  };
+};
+
 // The operand is kept in one variable whose first dword is replaced per use
 // (rank1_set), so that the zero slots are written once and not per tile.
 template <typename T>

@@ -23,7 +23,7 @@ struct FwdFamily {
   template <typename T, int D, int NW, int R, int BK>
   static hipError_t run(const FwdArgs& a, int bh, hipStream_t st, bool dry) {
     // two stages of: K and V rows of the R pair rows + one packed bias tile per wave and key tile
-    constexpr int lds = 2 * (2 * R * BK * D + NW * (BK / 32) * 1024) * (int)sizeof(T);
+    constexpr int lds = 2 * ((2 * R * BK * D + NW * (BK / 32) * 1024) * (int)sizeof(T) + 256);
     // R rows of accumulators and Q operands per wave must stay in registers
     constexpr int acc_regs = R * (((D + 31) / 32) * 16 + D / 2 * (int)sizeof(T) / 4);
     if constexpr (lds <= kMaxLds && (acc_regs <= 160 || R == 1)) {
