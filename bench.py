@@ -36,10 +36,10 @@ PEAK_HBM_GBS = 8000.0
 # profiles/bench_M_hbm_traffic.txt (readings scaled by a plain 256 MiB copy).  Reported
 # as roofline.traffic when the benchmark runs that workload with that tile.
 MEASURED_TRAFFIC_MIB = {
-    ("M", "_fwd", (128, 32, 4)): 1517.5,
-    ("M", "_bwd_q", (128, 32, 4)): 2307.8,
-    ("M", "_bwd_kv", (32, 128, 4)): 2101.3,
-    ("M", "_bwd_b", (128, 128, 16)): 1648.9,
+    ("M", "_fwd", (128, 32, 4)): 1476.0,
+    ("M", "_bwd_q", (128, 32, 4)): 2301.6,
+    ("M", "_bwd_kv", (32, 128, 4)): 2089.6,
+    ("M", "_bwd_b", (128, 128, 16)): 1701.9,
 }
 
 # name -> (dtype, b, n, h, d, description)

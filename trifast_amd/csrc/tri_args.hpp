@@ -38,8 +38,7 @@ struct FwdArgs {
   float* lse;
   Str5 sq, sk, sv;
   int H, N, NP, nwords;
-  float c;                   // log2(e) / sqrt(d): raw score -> log2 domain
-  float sqrt_d;              // bias multiplier into the raw-score domain
+  float c;                   // log2(e) / sqrt(d): multiplier of the resident Q operand (base-2 scores)
   float neg_inf;             // finfo(dtype).min, reported in lse of fully masked rows
 };
 
@@ -65,7 +64,7 @@ struct BwdArgs {
   int BH;                    // b * h
   int nchunks, rows_per_chunk;  // db kernel: split of the pair rows over workgroups
   float c;                   // log2(e) / sqrt(d)
-  float sqrt_d;
+  float sqrt_d;              // raw-score domain of the db kernel: bias and lse multiplier
   float scale;               // 1 / sqrt(d)
 };
 

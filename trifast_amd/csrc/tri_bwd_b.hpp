@@ -14,9 +14,9 @@
 // (column) and 16 keys of each tile.  The additive terms ride on the matrix pipe:
 // the bias tiles (register-resident, fp32, raw-score domain) are the accumulator
 // init of every row's score MFMA, and the per-query terms -lse*sqrt(d) and -delta
-// enter through one extra MFMA each (see rank1_operand), which leaves one
-// multiply, one exp2 and one fma per element to the vector ALU.  Masked keys get a
-// large negative score through one more MFMA (see mask_operand).
+// enter through one extra MFMA each (see rank1_operand, OffsetMask), which leaves
+// one multiply, one exp2 and one fma per element to the vector ALU.  Masked keys get
+// a large negative score from the MFMA that adds -lse.
 //
 // All workgroups of one (batch*head, chunk) read the same rows at about the same
 // time; the block index is remapped so that they run on one XCD and share its L2.

@@ -339,7 +339,6 @@ int trifast_fwd(void* o, float* lse, const void* q, const void* k, const void* v
   a.sq = str5(q_strides); a.sk = str5(k_strides); a.sv = str5(v_strides);
   a.H = (int)h; a.N = (int)n; a.NP = w.np; a.nwords = w.nwords;
   a.c = (float)(1.4426950408889634 / std::sqrt((double)d));
-  a.sqrt_d = (float)std::sqrt((double)d);
   a.neg_inf = dtype_min(dtype);
   hipError_t e = tri::fwd_launch(a, (int)(b * h), (int)d, dtype, tile, st);
   if (e != hipSuccess) return hip_fail(e, "forward launch");

@@ -35,9 +35,6 @@ namespace tri {
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
-// Finite stand-in for "minus infinity" on raw scores: large enough that
-// exp2((NEG - max) * c) is exactly 0, finite so that NEG - NEG is never NaN.
-constexpr float kNeg = -1.0e30f;
 
 TRI_DEV int perm32(int m) {  // swap bits 2 and 3
   return (m & 0x13) | ((m & 4) << 1) | ((m & 8) >> 1);

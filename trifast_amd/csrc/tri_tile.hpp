@@ -297,17 +297,6 @@ TRI_DEV f32x16 bias_tile(const T* pack_bh, int NP, int jt, int kt, int lane, flo
   return s;
 }
 
-// Additive key mask through the matrix pipe.  One extra MFMA adds, to every score
-// of a masked key, the sum over all contraction slots of kMaskElem * 1: the
-// operand returned here holds kMaskElem in every slot when key `key_in_tile` of
-// the tile is masked (bit clear in keepw) and zeros otherwise; the other operand
-// is Elem<T>::splat(1).  The lane passes the key its operand row / column stands
-// for.
-template <typename T>
-TRI_DEV typename Elem<T>::frag mask_operand(uint32_t keepw, int key_in_tile) {
-  return ((keepw >> key_in_tile) & 1u) ? Elem<T>::zero() : Elem<T>::splat(Elem<T>::kMaskElem);
-}
-
 // Which 32-key tiles matter to the R pair rows of a workgroup, as bitmaps over
 // the key tiles, one 64-bit word per 64 tiles, built once into LDS:
 //   live  = some row attends to some key of the tile (other tiles are skipped:
@@ -390,19 +379,9 @@ struct KeyTileMasks {
 };
 
 // Compile-time versions of a stage loop, chosen per workgroup: every row attends to
-// every key (no mask work, no per-tile branch); some keys are masked but no row is
-// fully masked (one mask MFMA per tile, dead tiles skipped); anything.
+// every key (constant keys operand, no per-tile branch); some keys are masked but no
+// row is fully masked (dead tiles skipped); anything.
 constexpr int kPlain = 0, kMasked = 1, kGeneral = 2;
-
-// Additive key mask of one 32-key tile in the transposed-score layout: value v
-// of lane group g is 0 when key cidx(v, g) is attended to and kNeg otherwise.
-TRI_DEV f32x16 mask_tile(uint32_t keepw, int g) {
-  const uint32_t myw = keepw >> (8 * g);
-  f32x16 m;
-#pragma unroll
-  for (int v = 0; v < 16; ++v) m[v] = ((myw >> (16 * (v / 8) + (v % 8))) & 1u) ? 0.f : kNeg;
-  return m;
-}
 
 // Store a 32-row tile of an [n x D] output held transposed in registers
 // (lane owns row `row`, values are columns 32*mt + 8*a4 + 4*g + 0..3), scaled.
