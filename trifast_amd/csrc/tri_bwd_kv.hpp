@@ -30,7 +30,7 @@
 namespace tri {
 
 template <typename T, int D, int NW, int R, int BJ, int NBUF>
-__global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512) ? 2 : 1) void tri_bwd_kv_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512 || (D * (int)sizeof(T) == 128 && R == 1)) ? 2 : 1) void tri_bwd_kv_kernel(const BwdArgs a) {
   using E = Elem<T>;
   using frag = typename E::frag;
   using Tile = LdsTile<T, D>;

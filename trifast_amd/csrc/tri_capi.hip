@@ -272,14 +272,25 @@ int trifast_supports(int kernel, int tile, int64_t n, int64_t h, int64_t d, int 
 
 int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype) {
   (void)h;
-  // Picks measured on MI355X at d = 32; anything that does not fit the shape
-  // falls back to tile 0 and then to the first tile that supports it.
+  // Picks measured on MI355X (bf16/fp16 at d = 16, 32, 64 and fp32 at d = 32, 64), by
+  // the bytes of one q/k/v row: the wider the row, the fewer pair rows and tiles per
+  // wave fit in registers.  Anything that does not fit the shape falls back to tile 0
+  // and then to the first tile that supports it.
+  const int64_t row_bytes = d * elem_size(dtype);
   int pick = 0;
   switch (kernel) {
-    case TRIFAST_KERNEL_FWD: pick = n <= 64 ? 0 : 4; break;     // 2 pair rows share a bias tile, 3 waves per SIMD
-    case TRIFAST_KERNEL_BWD_Q: pick = n <= 64 ? 0 : 2; break;   // 2 pair rows, 32 keys per stage
-    case TRIFAST_KERNEL_BWD_KV: pick = n <= 64 ? 0 : 1; break;  // 2 pair rows, 32 queries per stage
-    case TRIFAST_KERNEL_BWD_B: pick = n <= 128 ? 2 : 4; break;  // 128 x 128 block of 16 waves; 64 x 64 at small n
+    case TRIFAST_KERNEL_FWD:  // 2 pair rows share a bias tile, 3 waves per SIMD; one row for wide rows
+      pick = (n <= 64 || row_bytes >= 256) ? 0 : 4;
+      break;
+    case TRIFAST_KERNEL_BWD_Q:  // 2 pair rows, 32 keys per stage; one row from 128-byte rows on
+      pick = (n <= 64 || row_bytes >= 128) ? 0 : 2;
+      break;
+    case TRIFAST_KERNEL_BWD_KV:  // 2 pair rows, 32 queries per stage; one row, 64 queries for wide 16-bit rows
+      pick = (n <= 64 || row_bytes >= 256 || (row_bytes == 128 && dtype != TRIFAST_F32)) ? 0 : 1;
+      break;
+    case TRIFAST_KERNEL_BWD_B:  // 128 x 128 block of 16 waves; 8 waves, then 64 x 64 of 4 waves, as rows widen or n shrinks
+      pick = (n <= 128 || row_bytes >= 256) ? 2 : (row_bytes == 128 ? 3 : 4);
+      break;
 
     default: return fail(TRIFAST_EINVAL, "unknown kernel id %d", kernel);
   }
