@@ -1,0 +1,77 @@
+"""Pair tensors with more than 2^31 elements: n = 4096, h = 6, d = 32 in bf16.
+
+Offsets into q/k/v/o and the gradients no longer fit 32 bits there, which the smaller
+parity shapes never exercise.  The n^3 logits of the whole problem are out of reach for
+a dense check (1 TiB in fp32), but triangle attention is local to a pair row: o[i], dq[i],
+dk[i], dv[i] depend on row i of q, k, v, do only, and the bias gradient is the sum of
+per-row terms.  With do zero outside a few chosen rows, db is the sum over those rows, so
+everything is checked exactly against the row-wise restatement of
+reference src/trifast/equiv.py:42-69 below, in float32, with the reference's tolerance rule
+(tests/utils.py:31-36) against the same computation in bf16.
+"""
+
+import math
+
+import pytest
+import torch
+
+import trifast_amd
+from oracle import triangle_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+N, H, D = 4096, 6, 32
+ROWS = (0, 1, 1777, 4095)  # first, second, one in the middle, last
+
+
+def row_attention(q_i, k_i, v_i, bias, mask_i):
+    """One pair row: q_i, k_i, v_i [h, n, d], bias [h, n, n], mask_i [n] (True = masked)."""
+    s = torch.einsum("hjd,hkd->hjk", q_i, k_i) / math.sqrt(q_i.shape[-1]) + bias
+    s = s + mask_i.to(s.dtype)[None, None, :] * torch.finfo(s.dtype).min
+    return torch.einsum("hjk,hkd->hjd", torch.softmax(s, dim=-1), v_i)
+
+
+def rows_reference(q, k, v, bias, mask, do, dtype):
+    """o, dq, dk, dv of the chosen rows and db summed over them, computed in `dtype`."""
+    out = {}
+    db = torch.zeros_like(bias[0], dtype=torch.float32)
+    for i in ROWS:
+        q_i, k_i, v_i = (t[0, :, i].to(dtype).detach().requires_grad_(True) for t in (q, k, v))
+        b = bias[0].to(dtype).detach().requires_grad_(True)
+        o_i = row_attention(q_i, k_i, v_i, b, mask[0, i])
+        o_i.backward(do[0, :, i].to(dtype))
+        out[i] = tuple(t.detach().float() for t in (o_i, q_i.grad, k_i.grad, v_i.grad))
+        db += b.grad.float()
+    return out, db
+
+
+def test_offsets_beyond_32_bits():
+    assert H * N * N * D > 2**31
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(4096)
+    dtype = torch.bfloat16
+    q, k, v = (torch.randn(1, H, N, N, D, device=dev, dtype=dtype, generator=g) for _ in range(3))
+    bias = torch.randn(1, H, N, N, device=dev, dtype=dtype, generator=g)
+    mask = torch.rand(1, N, N, device=dev, generator=g) < 0.3
+    mask[0, 1777, :] = True  # a fully masked row among the checked ones
+    do = torch.zeros_like(q)
+    for i in ROWS:
+        do[0, :, i] = torch.randn(H, N, D, device=dev, dtype=dtype, generator=g)
+
+    q, k, v, bias = (t.requires_grad_(True) for t in (q, k, v, bias))
+    o = trifast_amd.triangle_attention(q, k, v, bias, mask)
+    o.backward(do)
+    torch.cuda.synchronize()
+
+    ref, db_ref = rows_reference(q, k, v, bias, mask, do, torch.float32)
+    pt, db_pt = rows_reference(q, k, v, bias, mask, do, dtype)
+    eps = orc.DTYPE_EPS[dtype]
+    for i in ROWS:
+        got = (o[0, :, i], q.grad[0, :, i], k.grad[0, :, i], v.grad[0, :, i])
+        for name, x, p, r in zip(("o", "dq", "dk", "dv"), got, pt[i], ref[i]):
+            assert torch.isfinite(x.float()).all(), f"row {i} {name}: non-finite values"
+            orc.compare_values(x.detach(), p, r, f"n={N} row {i} {name}", eps=eps)
+    orc.compare_values(bias.grad[0], db_pt, db_ref, f"n={N} db", eps=eps)
+    # rows that received no upstream gradient have none to give
+    for i in (2, 4094):
+        assert not q.grad[0, :, i].any() and not k.grad[0, :, i].any() and not v.grad[0, :, i].any()
