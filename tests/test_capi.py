@@ -75,9 +75,9 @@ def test_workspace_sizes_are_quadratic_in_n():
     plane = 4 * 1024 * 1024  # h * n * n elements
     # forward: keep words, row flags and one packed copy of the bias in the input dtype
     assert plane * 2 <= f1 <= plane * 2 + (1 << 20)
-    # backward: two packed bias copies, three 32-bit per-query planes (delta and lse in two
-    # scalings) and at most 8 fp32 db partials
-    assert plane * (2 * 2 + 3 * 4) <= b1 <= plane * (2 * 2 + 3 * 4 + 8 * 4) + (1 << 20)
+    # backward: two packed bias copies, two 32-bit per-query planes (delta and lse) and at
+    # most 8 fp32 db partials
+    assert plane * (2 * 2 + 2 * 4) <= b1 <= plane * (2 * 2 + 2 * 4 + 8 * 4) + (1 << 20)
     # O(n^2): doubling n may not cost more than four times the memory
     assert 1.9 < b2 / b1 < 4.1
     assert lib.trifast_fwd_workspace_bytes(0, 4, 16, 32, _lib.BF16) < 0

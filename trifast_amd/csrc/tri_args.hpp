@@ -38,7 +38,8 @@ struct FwdArgs {
   float* lse;
   Str5 sq, sk, sv;
   int H, N, NP, nwords;
-  float c;                   // log2(e) / sqrt(d): multiplier of the resident Q operand (base-2 scores)
+  float c;                   // log2(e) / sqrt(d): raw score -> log2 domain
+  float sqrt_d;              // bias multiplier into the raw-score domain
   float neg_inf;             // finfo(dtype).min, reported in lse of fully masked rows
 };
 
@@ -51,12 +52,9 @@ struct BwdArgs {
   // [b*h, n, n] 32-bit workspaces indexed [i, j], written by the dq kernel for the
   // other two: the per-query terms of the backward as rank-1 MFMA operand words
   // (see split_word): delta = -rowsum(o * do); lse2 = -lse * sqrt(d), the
-  // log-sum-exp in the raw-score domain (ln n instead of lse for fully masked rows),
-  // for the db kernel; lse2l = -lse * log2(e), the same in the base-2 domain, for
-  // the dk/dv kernel
+  // log-sum-exp in the raw-score domain (ln n instead of lse for fully masked rows)
   uint32_t* delta;
   uint32_t* lse2;
-  uint32_t* lse2l;
   float* dbpart;             // [nchunks, b*h, n, n] fp32 partial db (nchunks > 1 only)
   void *dq, *dk, *dv, *db;
   Str5 sq, sk, sv, sdo;
@@ -64,7 +62,7 @@ struct BwdArgs {
   int BH;                    // b * h
   int nchunks, rows_per_chunk;  // db kernel: split of the pair rows over workgroups
   float c;                   // log2(e) / sqrt(d)
-  float sqrt_d;              // raw-score domain of the db kernel: bias and lse multiplier
+  float sqrt_d;
   float scale;               // 1 / sqrt(d)
 };
 

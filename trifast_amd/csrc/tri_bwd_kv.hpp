@@ -11,13 +11,11 @@
 //   dv^T += dO^T P,   dk^T += Q^T dS,   dk = dk^T / sqrt(d),
 // whose A operands dO^T, Q^T come from the natural tiles through transposing LDS
 // reads.  The per-element additive terms ride on the matrix pipe: the bias tile
-// (fp32, times log2(e), converted once per stage and shared by the R rows) is
-// the accumulator init of the score MFMA, the resident K operand is scaled by
-// log2(e)/sqrt(d) once, and the per-query terms -lse*log2(e) and -delta enter
-// through one extra MFMA each (see rank1_operand, OffsetMask), so that P = exp2(acc)
-// needs no arithmetic before the exponential and dS = P * dP' is one multiply.  Masked
-// keys get a large negative score from the MFMA that adds -lse, which makes their P
-// and dS zero.
+// (fp32, raw-score domain, converted once per stage and shared by the R rows) is
+// the accumulator init of the score MFMA, and the per-query terms -lse*sqrt(d) and
+// -delta enter through one extra MFMA each (see rank1_operand, OffsetMask), so that
+// P = exp2(c * acc) and dS = P * dP' are one multiply each.  Masked keys get a large
+// negative score from the MFMA that adds -lse, which makes their P and dS zero.
 //
 // Replaces _bwd_kv of reference src/trifast/triton.py:143-263.
 #pragma once
@@ -29,8 +27,16 @@
 
 namespace tri {
 
+// Two waves per SIMD (at most 256 registers) wherever the tile fits them or nearly
+// does: a few registers over would otherwise halve the occupancy.
+template <typename T, int D, int R, int BJ>
+constexpr int bwd_kv_min_waves() {
+  constexpr int row_bytes = D * (int)sizeof(T);
+  return (row_bytes >= 512 || (row_bytes == 128 && R == 1) || (row_bytes <= 64 && R * BJ <= 64)) ? 2 : 1;
+}
+
 template <typename T, int D, int NW, int R, int BJ, int NBUF>
-__global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512 || (D * (int)sizeof(T) == 128 && R == 1)) ? 2 : 1) void tri_bwd_kv_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(NW * 64, (bwd_kv_min_waves<T, D, R, BJ>())) void tri_bwd_kv_kernel(const BwdArgs a) {
   using E = Elem<T>;
   using frag = typename E::frag;
   using Tile = LdsTile<T, D>;
@@ -69,7 +75,7 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512 || (D * (int)si
   const T* vbh = reinterpret_cast<const T*>(a.v) + b * a.sv.b + h * a.sv.h;
   const T* dobh = reinterpret_cast<const T*>(a.dout) + b * a.sdo.b + h * a.sdo.h;
   const T* pack_bh = reinterpret_cast<const T*>(a.packk) + (int64_t)bh * a.NP * a.NP * 1024;
-  const float* lse2_bh = reinterpret_cast<const float*>(a.lse2l) + (int64_t)bh * N * N;    // 32-bit words, moved as floats
+  const float* lse2_bh = reinterpret_cast<const float*>(a.lse2) + (int64_t)bh * N * N;    // 32-bit words, moved as floats
   const float* delta_bh = reinterpret_cast<const float*>(a.delta) + (int64_t)bh * N * N;
 
   // per-row state: K and V tiles as B operands (lane owns key k_wave + kl).  A
@@ -97,7 +103,7 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512 || (D * (int)si
     for (int s = 0; s < DS; ++s) {
       const int dofs = 2 * KP * s + KP * g;
       const int kc = min(key, N - 1);
-      kf[r][s] = flagged[r] ? E::zero() : scale_frag<T>(*reinterpret_cast<const frag*>(kbh + i * a.sk.i + (int64_t)kc * a.sk.j + dofs), a.c);
+      kf[r][s] = flagged[r] ? E::zero() : *reinterpret_cast<const frag*>(kbh + i * a.sk.i + (int64_t)kc * a.sk.j + dofs);
       vf[r][s] = *reinterpret_cast<const frag*>(vbh + i * a.sv.i + (int64_t)kc * a.sv.j + dofs);
     }
 #pragma unroll
@@ -162,18 +168,19 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512 || (D * (int)si
       if constexpr (sizeof(T) == 2) {
         const typename E::vec x = *reinterpret_cast<const typename E::vec*>(src + r2 * (BIAS_B / 2) + lane * 16);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) bv[8 * r2 + e] = (float)x[e] * kLog2e;
+        for (int e = 0; e < 8; ++e) bv[8 * r2 + e] = (float)x[e] * a.sqrt_d;
       } else {
         const f32x4 x0 = *reinterpret_cast<const f32x4*>(src + r2 * (BIAS_B / 2) + lane * 16);
         const f32x4 x1 = *reinterpret_cast<const f32x4*>(src + r2 * (BIAS_B / 2) + 1024 + lane * 16);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { bv[8 * r2 + e] = x0[e] * kLog2e; bv[8 * r2 + 4 + e] = x1[e] * kLog2e; }
+        for (int e = 0; e < 4; ++e) { bv[8 * r2 + e] = x0[e] * a.sqrt_d; bv[8 * r2 + 4 + e] = x1[e] * a.sqrt_d; }
       }
     }
     return bv;
   };
   // the per-query operand word (lse or delta term) of the query this lane's A
   // operand row stands for, in tile (r, u)
+  const float c = a.c;
   typename OffsetMask<T>::Queries lseop;  // the query's -lse word | ones: A operand of that MFMA
   lseop.init(0u, g);
   auto query_word = [&](const unsigned char* st, int off, int r, int u) -> uint32_t {
@@ -192,7 +199,7 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512 || (D * (int)si
 #pragma unroll
     for (int u = 0; u < JU; ++u) biasv[u] = bias_from_lds(st, u);
 
-    // base-2 scores: bias tile (accumulator init) - lse*log2(e) (per query, one MFMA) + Q (cK)^T;
+    // scores: bias tile (accumulator init) - lse*sqrt(d) (per query, one MFMA) + Q K^T;
     // dP - delta: -delta (per query, one MFMA) + dO V^T
     auto chains = [&](int t, f32x16& sc, f32x16& dp) {
       const int u = t / R, r = t % R;
@@ -234,7 +241,7 @@ __global__ __launch_bounds__(NW * 64, (D * (int)sizeof(T) >= 512 || (D * (int)si
         float p[16], ds[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          p[v] = fast_exp2(sc[v]);
+          p[v] = fast_exp2(sc[v] * c);
           ds[v] = p[v] * dp[v];
         }
 #pragma unroll

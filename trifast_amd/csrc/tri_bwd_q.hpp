@@ -5,17 +5,15 @@
 // operands, lse, delta and the dq accumulator in registers); K[i] and V[i] are
 // streamed through LDS in tiles of BK keys (direct global->LDS loads,
 // double-buffered, swizzled) together with the packed bias tiles, and the bias
-// tile (fp32, times log2(e)) is shared by the R rows as the accumulator init of the
-// score MFMA.  With transposed scores (a lane owns one query) P is recomputed from
-// the saved log-sum-exp in the base-2 domain (the resident Q operand is scaled by
-// c = log2(e)/sqrt(d) once),
-//   P^T = exp2(K (cQ)^T + bias*log2e - lse*log2e),  dP^T - delta = V dO^T - delta,
-//   dS^T = P^T * (dP^T - delta),  dq^T += K^T dS^T,  dq = dq^T / sqrt(d),
+// tile (fp32, raw-score domain) is shared by the R rows as the accumulator init of
+// the score MFMA.  With transposed scores (a lane owns one query) P is recomputed
+// from the saved log-sum-exp,
+//   P^T = exp2(S^T c - lse*log2e),  dP^T - delta = V dO^T - delta,  dS^T = P^T * (dP^T - delta),
+//   dq^T += K^T dS^T,               dq = dq^T / sqrt(d),
 // with K^T read from the natural K tile through transposing LDS reads.  -delta is
 // the accumulator init of the dP MFMA (16 registers per row that never change),
-// so the subtraction costs nothing.  -lse per query and a large negative score for
-// masked keys (which makes their P and dS zero) enter through one extra MFMA (see
-// OffsetMask), so nothing is computed before the exponential.
+// so the subtraction costs nothing.  Masked keys get a large negative score
+// through one extra MFMA (see OffsetMask), which makes their P and dS zero.
 //
 // This kernel runs first: it writes -delta and -lse*sqrt(d) (ln n for lse in fully
 // masked rows) per query, as rank-1 MFMA operand words, for the dk/dv and db kernels.
@@ -77,7 +75,6 @@ __global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(co
   bool any_flagged = false;
   const uint32_t* keep_row[R];
   frag qf[R][DS], dof[R][DS];
-  typename OffsetMask<T>::Queries qop[R];  // -lse (base 2) as MFMA operand
   float lse2[R];
   f32x16 ndelta[R];  // -delta in all 16 slots: accumulator init of the dP MFMA
   f32x16 dqacc[R][DM];
@@ -93,9 +90,7 @@ __global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(co
 #pragma unroll
     for (int s = 0; s < DS; ++s) {
       const int dofs = 2 * KP * s + KP * g;
-      // Q is scaled by log2(e) / sqrt(d) once (rounded to the input dtype, as the forward
-      // kernel does): the score MFMA then works in the base-2 domain
-      qf[r][s] = (flagged[r] || j >= N) ? E::zero() : scale_frag<T>(*reinterpret_cast<const frag*>(qbh + i * a.sq.i + (int64_t)jc * a.sq.j + dofs), a.c);
+      qf[r][s] = (flagged[r] || j >= N) ? E::zero() : *reinterpret_cast<const frag*>(qbh + i * a.sq.i + (int64_t)jc * a.sq.j + dofs);
       dof[r][s] = (j >= N) ? E::zero() : *reinterpret_cast<const frag*>(dobh + i * a.sdo.i + (int64_t)jc * a.sdo.j + dofs);
       const frag of = *reinterpret_cast<const frag*>(orow + dofs);
       if constexpr (KP == 1) {
@@ -111,22 +106,24 @@ __global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(co
       // the per-query terms of the other two backward kernels, as rank-1 MFMA operand words
       a.delta[((int64_t)bh * N + i) * N + j] = split_word<T>(-dsum);
       a.lse2[((int64_t)bh * N + i) * N + j] = split_word<T>(-lse2[r] * (kLn2 * a.sqrt_d));
-      a.lse2l[((int64_t)bh * N + i) * N + j] = split_word<T>(-lse2[r]);
     }
-    qop[r].init(split_word<T>(-lse2[r]), g);
 #pragma unroll
     for (int v = 0; v < 16; ++v) ndelta[r][v] = -dsum;
 #pragma unroll
     for (int mt = 0; mt < DM; ++mt) dqacc[r][mt] = zero16();
   }
-  typename OffsetMask<T>::Keys kop;  // ones | key mask as MFMA operand
+  const float c = a.c;
+
+  // the key mask enters the scores through one extra MFMA: keys operand with the mask
+  // element of this lane's key (patched in place per tile) against a constant queries
+  // operand (see OffsetMask; its per-query offset is not used here: the word is zero)
+  typename OffsetMask<T>::Keys kop;
   kop.init(perm32(jl), g);
-  frag kop_plain = kop.plain();
-  if constexpr (sizeof(T) == 2) {
-    // (opaque: kept in registers instead of being rebuilt from constants per tile)
-    typename OffsetMask<T>::u32x4 t = __builtin_bit_cast(typename OffsetMask<T>::u32x4, kop_plain);
-    asm volatile("" : "+v"(t));
-    kop_plain = __builtin_bit_cast(frag, t);
+  frag qzero;
+  {
+    typename OffsetMask<T>::Queries qz;
+    qz.init(split_word<T>(0.f), g);
+    qzero = qz.get();
   }
 
   KeyTileMasks masks;
@@ -183,12 +180,12 @@ __global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(co
       if constexpr (sizeof(T) == 2) {
         const typename E::vec x = *reinterpret_cast<const typename E::vec*>(src + r2 * (BIAS_B / 2) + lane * 16);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) bv[8 * r2 + e] = (float)x[e] * kLog2e;
+        for (int e = 0; e < 8; ++e) bv[8 * r2 + e] = (float)x[e] * a.sqrt_d;
       } else {
         const f32x4 x0 = *reinterpret_cast<const f32x4*>(src + r2 * (BIAS_B / 2) + lane * 16);
         const f32x4 x1 = *reinterpret_cast<const f32x4*>(src + r2 * (BIAS_B / 2) + 1024 + lane * 16);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { bv[8 * r2 + e] = x0[e] * kLog2e; bv[8 * r2 + 4 + e] = x1[e] * kLog2e; }
+        for (int e = 0; e < 4; ++e) { bv[8 * r2 + e] = x0[e] * a.sqrt_d; bv[8 * r2 + 4 + e] = x1[e] * a.sqrt_d; }
       }
     }
     return bv;
@@ -221,23 +218,28 @@ __global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(co
       const int u = t / R, r = t % R;
       const unsigned char* kt = st + OFF_K + (r * BK + 32 * u) * ROWB;
       const unsigned char* vt = st + OFF_V + (r * BK + 32 * u) * ROWB;
-      // base-2 scores minus the query's lse: bias tile (accumulator init), then one MFMA
-      // that subtracts lse per query and masks keys (see OffsetMask), then K (cQ)^T
       if constexpr (PLAIN) {
-        sc = E::mfma(kop_plain, qop[r].get(), biasv[u]);
+        sc = E::mfma(ofs.natural(kt, 0), qf[r][0], biasv[u]);
       } else {
         // Each case ends in the MFMA that defines sc, so that the bias tile is used
         // in place as an accumulator init (a select between inits copies 16 registers).
-        if (MODE == kMasked || !flagged[r]) {
-          sc = E::mfma(kop.masked(kw[r][u]), qop[r].get(), biasv[u]);
+        if (MODE == kMasked) {
+          // no fully masked row in the workgroup: the mask MFMA runs for every tile
+          // (its operand is zero where nothing is masked) and nothing branches
+          sc = E::mfma(ofs.natural(kt, 0), qf[r][0], E::mfma(kop.masked(kw[r][u]), qzero, biasv[u]));
+        } else if (!flagged[r]) {
+          if (kw[r][u] != 0xffffffffu)
+            sc = E::mfma(ofs.natural(kt, 0), qf[r][0], E::mfma(kop.masked(kw[r][u]), qzero, biasv[u]));
+          else
+            sc = E::mfma(ofs.natural(kt, 0), qf[r][0], biasv[u]);
         } else {
           // a fully masked row has no bias (and a zero Q), but keys past the end of a
           // ragged last tile stay masked for it too
           asm volatile("" ::);
-          sc = E::mfma(kop.masked(kw[r][u]), qop[r].get(), zero16());
+          sc = E::mfma(kop.masked(kw[r][u]), qzero, zero16());
+          sc = E::mfma(ofs.natural(kt, 0), qf[r][0], sc);
         }
       }
-      sc = E::mfma(ofs.natural(kt, 0), qf[r][0], sc);
       dp = E::mfma(ofs.natural(vt, 0), dof[r][0], ndelta[r]);
 #pragma unroll
       for (int sd = 1; sd < DS; ++sd) {
@@ -259,7 +261,7 @@ __global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(co
         float ds[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const float p = fast_exp2(sc[v]);
+          const float p = fast_exp2(__builtin_fmaf(sc[v], c, -lse2[r]));
           ds[v] = p * dp[v];
         }
 #pragma unroll

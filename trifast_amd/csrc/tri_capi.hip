@@ -129,7 +129,7 @@ float dtype_min(int dtype) {
   }
 }
 
-// workspace layout: keep words | row flags | packq | (backward only) packk | -delta | lse2 | lse2l | db partials
+// workspace layout: keep words | row flags | packq | (backward only) packk | -delta | lse2 | db partials
 struct Workspace {
   uint32_t* keep;
   uint32_t* rowflag;
@@ -137,7 +137,6 @@ struct Workspace {
   void* packk;
   uint32_t* delta;
   uint32_t* lse2;
-  uint32_t* lse2l;
   float* dbpart;
   int nwords, np;
 };
@@ -167,8 +166,6 @@ Workspace carve(void* ws, int64_t b, int64_t h, int64_t n, int dtype) {
   w.delta = reinterpret_cast<uint32_t*>(p);
   p += align256(b * h * n * n * 4);
   w.lse2 = reinterpret_cast<uint32_t*>(p);
-  p += align256(b * h * n * n * 4);
-  w.lse2l = reinterpret_cast<uint32_t*>(p);
   p += align256(b * h * n * n * 4);
   w.dbpart = reinterpret_cast<float*>(p);
   w.nwords = (int)nwords;
@@ -279,11 +276,11 @@ int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype)
   const int64_t row_bytes = d * elem_size(dtype);
   int pick = 0;
   switch (kernel) {
-    case TRIFAST_KERNEL_FWD:  // 2 pair rows share a bias tile, 3 waves per SIMD; one row for wide rows
-      pick = (n <= 64 || row_bytes >= 256) ? 0 : 4;
+    case TRIFAST_KERNEL_FWD:  // 4 pair rows share a bias tile; 2 rows for 128-byte rows, one for wider ones
+      pick = (n <= 64 || row_bytes >= 256) ? 0 : (row_bytes == 128 ? 4 : 3);
       break;
-    case TRIFAST_KERNEL_BWD_Q:  // 2 pair rows, 32 keys per stage; one row from 128-byte rows on
-      pick = (n <= 64 || row_bytes >= 128) ? 0 : 2;
+    case TRIFAST_KERNEL_BWD_Q:  // 2 pair rows, 64 keys per stage; one row from 128-byte rows on
+      pick = (n <= 64 || row_bytes >= 128) ? 0 : 1;
       break;
     case TRIFAST_KERNEL_BWD_KV:  // 2 pair rows, 32 queries per stage; one row, 64 queries for wide 16-bit rows
       pick = (n <= 64 || row_bytes >= 256 || (row_bytes == 128 && dtype != TRIFAST_F32)) ? 0 : 1;
@@ -314,7 +311,7 @@ int64_t trifast_bwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, 
   (void)d;
   if (b < 1 || h < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
   const int64_t chunks = tri::bwd_b_chunks(n, b * h);
-  return ws_mask_bytes(b, n) + 2 * ws_pack_bytes(b, h, n, dtype) + 3 * align256(b * h * n * n * 4) +
+  return ws_mask_bytes(b, n) + 2 * ws_pack_bytes(b, h, n, dtype) + 2 * align256(b * h * n * n * 4) +
          (chunks > 1 ? align256(chunks * b * h * n * n * 4) : 0);
 }
 
@@ -350,6 +347,7 @@ int trifast_fwd(void* o, float* lse, const void* q, const void* k, const void* v
   a.sq = str5(q_strides); a.sk = str5(k_strides); a.sv = str5(v_strides);
   a.H = (int)h; a.N = (int)n; a.NP = w.np; a.nwords = w.nwords;
   a.c = (float)(1.4426950408889634 / std::sqrt((double)d));
+  a.sqrt_d = (float)std::sqrt((double)d);
   a.neg_inf = dtype_min(dtype);
   hipError_t e = tri::fwd_launch(a, (int)(b * h), (int)d, dtype, tile, st);
   if (e != hipSuccess) return hip_fail(e, "forward launch");
@@ -403,7 +401,7 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   a.q = q; a.k = k; a.v = v; a.o = o; a.dout = dout;
   a.packq = w.packq; a.packk = w.packk;
   a.lse = lse;
-  a.keep = w.keep; a.rowflag = w.rowflag; a.delta = w.delta; a.lse2 = w.lse2; a.lse2l = w.lse2l; a.dbpart = w.dbpart;
+  a.keep = w.keep; a.rowflag = w.rowflag; a.delta = w.delta; a.lse2 = w.lse2; a.dbpart = w.dbpart;
   a.BH = (int)(b * h);
   a.nchunks = tri::bwd_b_chunks(n, b * h);
   a.rows_per_chunk = (int)((n + a.nchunks - 1) / a.nchunks);

@@ -35,6 +35,9 @@ namespace tri {
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
+// Finite stand-in for "minus infinity" on raw scores: large enough that
+// exp2((NEG - max) * c) is exactly 0, finite so that NEG - NEG is never NaN.
+constexpr float kNeg = -1.0e30f;
 
 TRI_DEV int perm32(int m) {  // swap bits 2 and 3
   return (m & 0x13) | ((m & 4) << 1) | ((m & 8) >> 1);
@@ -216,18 +219,6 @@ TRI_DEV uint32_t split_word(float x) {
     return (uint32_t)__builtin_bit_cast(uint16_t, hi) | ((uint32_t)__builtin_bit_cast(uint16_t, lo) << 16);
   }
 }
-// the value a split word stands for (what the MFMA adds for it)
-template <typename T>
-TRI_DEV float unsplit_word(uint32_t w) {
-  if constexpr (sizeof(T) == 4) {
-    return __builtin_bit_cast(float, w);
-  } else {
-    const T hi = __builtin_bit_cast(T, (uint16_t)(w & 0xffffu));
-    const T lo = __builtin_bit_cast(T, (uint16_t)(w >> 16));
-    return (float)hi + (float)lo;
-  }
-}
-
 // Per-query offset and key mask through ONE extra MFMA of a transposed score tile
 // (rows = keys, columns = queries): the contraction slots are shared between the two
 // rank-1 terms.
@@ -330,19 +321,6 @@ TRI_DEV typename Elem<T>::frag resident_ones() {
     f = __builtin_bit_cast(typename Elem<T>::frag, v);
   }
   return f;
-}
-
-// every element of an operand fragment times s, rounded back to T
-template <typename T>
-TRI_DEV typename Elem<T>::frag scale_frag(typename Elem<T>::frag f, float s) {
-  if constexpr (sizeof(T) == 4) {
-    return f * s;
-  } else {
-    float x[Elem<T>::KP];
-#pragma unroll
-    for (int e = 0; e < Elem<T>::KP; ++e) x[e] = (float)f[e] * s;
-    return Elem<T>::pack(x);
-  }
 }
 
 TRI_DEV f32x16 zero16() {

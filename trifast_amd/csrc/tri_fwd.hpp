@@ -15,20 +15,19 @@
 // for O^T += V^T P^T, whose A operand V^T comes from the natural V tile through
 // transposing LDS reads.
 //
-// Base-2 domain: acc = log2(e) * bias - ref + (c q).k with c = log2(e) / sqrt(d).  The
-// converted bias tile is the accumulator init and is shared by the R rows; the
-// resident Q operand is scaled by c once; -ref (per query) and the key mask enter
-// through one extra MFMA (see OffsetMask), so that p = exp2(acc) needs no
-// arithmetic before the exponential.  `ref` is the reference of the online softmax:
-// it is set from the row's first tile and raised only when the probabilities of
-// some query of the wave sum to more than 2^kLazy within a tile, so the accumulator
-// rescale is rare and no maximum is searched otherwise; p stays below 2^kLazy,
-// which fp32/bf16/fp16 hold.  References are whole numbers, exact as operand words.
+// Raw-score domain: acc = sqrt(d) * bias + q.k (the converted bias tile is the
+// accumulator init of the score MFMA and is shared by the R rows);
+// p = exp2(acc * c - ref * c) with c = log2(e) / sqrt(d).  `ref` is the running
+// reference of the online softmax: it is raised to the running maximum only when
+// the probabilities of some query of the wave sum to more than 2^kLazy within a
+// tile, so the accumulator rescale is rare and no maximum is searched otherwise;
+// p stays below 2^kLazy, which fp32/bf16/fp16 hold.
 //
 // Masks: a bitmap over the key tiles says which stages are live (others are
 // skipped) and whether all of them are plain (every row attends to every key:
-// the workgroup then runs a loop with a constant keys operand and no per-tile
-// branch).  Otherwise a masked key gets a large negative score from the same MFMA.
+// the workgroup then runs a loop with no mask work and no per-tile branch).
+// Otherwise a masked key gets a large negative score through one extra MFMA
+// (see OffsetMask).
 //
 // Replaces _fwd of reference src/trifast/triton.py:19-132.
 #pragma once
@@ -92,12 +91,7 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
   const uint32_t* keep_row[R];
   frag qf[R][DS];
   f32x16 oacc[R][DM];
-  // softmax state per query: reference mc (base-2 domain), running sum; the row has
-  // not met its first live tile while `fresh`
-  float mc[R], lrun[R];
-  bool fresh[R];
-  typename OffsetMask<T>::Queries qop[R];  // -mc as MFMA operand
-  const float c = a.c;
+  float mref[R], mc[R], lrun[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int i = min(i0 + r, N - 1);  // rows past the end repeat the last one and are not stored
@@ -106,28 +100,29 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
     keep_row[r] = a.keep + ((int64_t)b * N + i) * a.nwords;
 #pragma unroll
     for (int s = 0; s < DS; ++s) {
-      // Q is scaled by log2(e) / sqrt(d) once (rounded to the input dtype, as the
-      // reference rounds its scaled q): the score MFMA then works in the base-2 domain
       if (j < N && !flagged[r])
-        qf[r][s] = scale_frag<T>(*reinterpret_cast<const frag*>(qbh + i * a.sq.i + (int64_t)j * a.sq.j + 2 * KP * s + KP * g), c);
+        qf[r][s] = *reinterpret_cast<const frag*>(qbh + i * a.sq.i + (int64_t)j * a.sq.j + 2 * KP * s + KP * g);
       else
         qf[r][s] = E::zero();
     }
-    mc[r] = 0.f;
+    mref[r] = kNeg;
+    mc[r] = kNeg;
     lrun[r] = 0.f;
-    fresh[r] = true;
-    qop[r].init(split_word<T>(0.f), g);
 #pragma unroll
     for (int mt = 0; mt < DM; ++mt) oacc[r][mt] = zero16();
   }
-  typename OffsetMask<T>::Keys kop;  // ones | key mask as MFMA operand
+  const float c = a.c;
+
+  // the key mask enters the scores through one extra MFMA: keys operand with the mask
+  // element of this lane's key (patched in place per tile) against a constant queries
+  // operand (see OffsetMask; its per-query offset is not used here: the word is zero)
+  typename OffsetMask<T>::Keys kop;
   kop.init(perm32(jl), g);
-  frag kop_plain = kop.plain();
-  if constexpr (sizeof(T) == 2) {
-    // (opaque: kept in registers instead of being rebuilt from constants per tile)
-    typename OffsetMask<T>::u32x4 t = __builtin_bit_cast(typename OffsetMask<T>::u32x4, kop_plain);
-    asm volatile("" : "+v"(t));
-    kop_plain = __builtin_bit_cast(frag, t);
+  frag qzero;
+  {
+    typename OffsetMask<T>::Queries qz;
+    qz.init(split_word<T>(0.f), g);
+    qzero = qz.get();
   }
 
   KeyTileMasks masks;
@@ -181,7 +176,7 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
       }
     }
   };
-  // the 16 bias values of this lane for key tile u of the stage, base-2 domain
+  // the 16 bias values of this lane for key tile u of the stage, raw-score domain
   auto bias_from_lds = [&](int buf, int u) -> f32x16 {
     const unsigned char* src = tri_smem + buf * STAGE + OFF_B + (wave * KU + u) * BIAS_B;
     f32x16 bv;
@@ -190,12 +185,12 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
       if constexpr (sizeof(T) == 2) {
         const typename E::vec x = *reinterpret_cast<const typename E::vec*>(src + r2 * (BIAS_B / 2) + lane * 16);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) bv[8 * r2 + e] = (float)x[e] * kLog2e;
+        for (int e = 0; e < 8; ++e) bv[8 * r2 + e] = (float)x[e] * a.sqrt_d;
       } else {
         const f32x4 x0 = *reinterpret_cast<const f32x4*>(src + r2 * (BIAS_B / 2) + lane * 16);
         const f32x4 x1 = *reinterpret_cast<const f32x4*>(src + r2 * (BIAS_B / 2) + 1024 + lane * 16);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { bv[8 * r2 + e] = x0[e] * kLog2e; bv[8 * r2 + 4 + e] = x1[e] * kLog2e; }
+        for (int e = 0; e < 4; ++e) { bv[8 * r2 + e] = x0[e] * a.sqrt_d; bv[8 * r2 + 4 + e] = x1[e] * a.sqrt_d; }
       }
     }
     return bv;
@@ -208,11 +203,12 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
   // arithmetic of tile t, so the matrix pipe works on t+1 while the vector ALU
   // works on t.  K operands are read from LDS two tiles ahead.
   //
-  // Softmax of a tile: p = exp2(acc) is computed against the current reference
-  // without looking for the maximum first; only for the row's first live tile, and
-  // when the rounded probabilities of some query sum to more than 2^kLazy (which
-  // includes the overflow to +inf of a query that outgrew the reference by a lot),
-  // is the reference moved to the maximum of the tile and the tile redone.
+  // Softmax of a tile: p = exp2(acc * c - ref * c) is computed against the current
+  // reference without looking for the maximum first; only when the rounded
+  // probabilities of some query sum to more than 2^kLazy (which includes the
+  // overflow to +inf of a query that outgrew the reference by a lot, and the very
+  // first tile, whose reference is -1e30) is the reference raised to the running
+  // maximum and the tile recomputed.
   auto compute_stage = [&](auto mode_tag, int kt0, int buf) __attribute__((always_inline)) {
     constexpr int MODE = decltype(mode_tag)::value;
     constexpr bool PLAIN = MODE == kPlain;
@@ -241,27 +237,33 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
     f32x16 biasv[KU];
 #pragma unroll
     for (int u = 0; u < KU; ++u) biasv[u] = bias_from_lds(buf, u);
-    // base-2 scores minus the row's reference: bias tile (accumulator init), then one
-    // MFMA that subtracts the reference per query and masks keys, then K (cQ)^T
     auto scores = [&](int t, const frag* kf) -> f32x16 {
       const int u = t / R, r = t % R;
       f32x16 sc;
       if constexpr (PLAIN) {
-        sc = E::mfma(kop_plain, qop[r].get(), biasv[u]);
+        sc = E::mfma(kf[0], qf[r][0], biasv[u]);
       } else {
         // Each case ends in the MFMA that defines sc, so that the bias tile is used
         // in place as an accumulator init (a select between inits copies 16 registers).
-        if (MODE == kMasked || !flagged[r]) {
-          sc = E::mfma(kop.masked(kw[r][u]), qop[r].get(), biasv[u]);
+        if (MODE == kMasked) {
+          // no fully masked row in the workgroup: the mask MFMA runs for every tile
+          // (its operand is zero where nothing is masked) and nothing branches
+          sc = E::mfma(kf[0], qf[r][0], E::mfma(kop.masked(kw[r][u]), qzero, biasv[u]));
+        } else if (!flagged[r]) {
+          if (kw[r][u] != 0xffffffffu)
+            sc = E::mfma(kf[0], qf[r][0], E::mfma(kop.masked(kw[r][u]), qzero, biasv[u]));
+          else
+            sc = E::mfma(kf[0], qf[r][0], biasv[u]);
         } else {
           // a fully masked row has no bias (and a zero Q: all its scores are equal),
           // but keys past the end of a ragged last tile stay masked for it too
           asm volatile("" ::);
-          sc = E::mfma(kop.masked(kw[r][u]), qop[r].get(), zero16());
+          sc = E::mfma(kop.masked(kw[r][u]), qzero, zero16());
+          sc = E::mfma(kf[0], qf[r][0], sc);
         }
       }
 #pragma unroll
-      for (int sd = 0; sd < DS; ++sd) sc = E::mfma(kf[sd], qf[r][sd], sc);
+      for (int sd = 1; sd < DS; ++sd) sc = E::mfma(kf[sd], qf[r][sd], sc);
       return sc;
     };
 
@@ -294,53 +296,36 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
         for (int s2 = 0; s2 < PS; ++s2) {
           float p[KP];
 #pragma unroll
-          for (int e = 0; e < KP; ++e) p[e] = fast_exp2(sc[KP * s2 + e]);
+          for (int e = 0; e < KP; ++e) p[e] = fast_exp2(__builtin_fmaf(sc[KP * s2 + e], c, -mc[r]));
           pf[s2] = E::pack(p);
           ts = frag_sum(pf[s2], ts);
         }
-        if (__any(!(ts <= kLazyLimit)) || fresh[r]) {
-          // the row's first tile, or some query outgrew the reference: move the
-          // reference to the maximum of this tile, rounded up to a whole number (exact
-          // as an operand word), and redo the tile.  After the first tile the
-          // reference only rises.  (The empty volatile asm keeps the compiler from
-          // executing this rare path speculatively in line with the common one.)
+        if (__any(!(ts <= kLazyLimit))) {
+          // some query outgrew the reference: raise it to the running maximum.
+          // (The empty volatile asm keeps the compiler from executing this rare
+          // path speculatively in line with the common one.)
           asm volatile("" ::);
           float mx = fmaxf(sc[0], sc[1]);
 #pragma unroll
           for (int v = 2; v < 16; ++v) mx = fmaxf(mx, sc[v]);
-          mx = half_max(mx);  // relative to the current reference
-          float dm = __builtin_ceilf(mx);
-          if (!fresh[r]) dm = fmaxf(dm, 0.f);
-          const uint32_t word = split_word<T>(-(mc[r] + dm));
-          const float mnew = -unsplit_word<T>(word);
-          dm = mnew - mc[r];
-          if (!fresh[r]) {
-            const float alpha = fast_exp2(-dm);
-            lrun[r] *= alpha;
+          mx = half_max(mx);
+          const float mnew = fmaxf(mref[r], mx);
+          const float alpha = fast_exp2((mref[r] - mnew) * c);
+          lrun[r] *= alpha;
 #pragma unroll
-            for (int mt = 0; mt < DM; ++mt)
+          for (int mt = 0; mt < DM; ++mt)
 #pragma unroll
-              for (int v = 0; v < 16; ++v) oacc[r][mt][v] *= alpha;
-          }
-          mc[r] = mnew;
-          qop[r].set(word, g);
-          fresh[r] = false;
+            for (int v = 0; v < 16; ++v) oacc[r][mt][v] *= alpha;
+          mref[r] = mnew;
+          mc[r] = mnew * c;
           ts = 0.f;
 #pragma unroll
           for (int s2 = 0; s2 < PS; ++s2) {
             float p[KP];
 #pragma unroll
-            for (int e = 0; e < KP; ++e) p[e] = fast_exp2(sc[KP * s2 + e] - dm);
+            for (int e = 0; e < KP; ++e) p[e] = fast_exp2(__builtin_fmaf(sc[KP * s2 + e], c, -mc[r]));
             pf[s2] = E::pack(p);
             ts = frag_sum(pf[s2], ts);
-          }
-          // with one row per workgroup the next tile's scores, already computed, are
-          // relative to the old reference
-          if constexpr (R == 1) {
-            if (t + 1 < TS) {
-#pragma unroll
-              for (int v = 0; v < 16; ++v) sn[v] -= dm;
-            }
           }
         }
         lrun[r] += ts;
