@@ -34,12 +34,14 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch (fetch + write) of the kernels of workload M with the tiles the
 # tuner picks there, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
 # profiles/bench_M_hbm_traffic.txt (readings scaled by a plain 256 MiB copy).  Reported
-# as roofline.traffic when the benchmark runs that workload with that tile.
+# as roofline.traffic when the benchmark runs that workload with that tile (keyed by the
+# tile's index in the library's table of the kernel).
 MEASURED_TRAFFIC_MIB = {
-    ("M", "_fwd", (128, 32, 4)): 1476.0,
-    ("M", "_bwd_q", (128, 32, 4)): 2301.6,
-    ("M", "_bwd_kv", (32, 128, 4)): 2089.6,
-    ("M", "_bwd_b", (128, 128, 16)): 1701.9,
+    ("M", "_fwd", 3): 1517.5,
+    ("M", "_fwd", 4): 1474.7,
+    ("M", "_bwd_q", 2): 2252.8,
+    ("M", "_bwd_kv", 1): 2098.3,
+    ("M", "_bwd_b", 4): 1682.5,
 }
 
 # name -> (dtype, b, n, h, d, description)
@@ -160,7 +162,7 @@ def kernel_breakdown(q, k, v, bias, mask, do, reps):
         tile = tuner.pick(kernel, n, h, d, q.dtype, launch)
         launch(tile)
         torch.cuda.synchronize()
-        out[_lib.KERNEL_NAMES[kernel]] = {"ms": _event_ms(lambda: launch(tile), reps), "tile": _lib.tile_info(kernel, tile)}
+        out[_lib.KERNEL_NAMES[kernel]] = {"ms": _event_ms(lambda: launch(tile), reps), "tile": dict(_lib.tile_info(kernel, tile), id=tile)}
     return out
 
 
@@ -276,7 +278,7 @@ def main():
         rec["tflops"] = gemms[name] * 2 * b * h * n**3 * d / rec["ms"] / 1e9
     dom = max(kern, key=lambda key: kern[key]["ms"])
     tile = kern[dom]["tile"]
-    mib = MEASURED_TRAFFIC_MIB.get((args.workload, dom, (tile["BLOCK_J"], tile["BLOCK_K"], tile["num_waves"])))
+    mib = MEASURED_TRAFFIC_MIB.get((args.workload, dom, tile["id"]))
     traffic = None if mib is None else mib * 2**20
     roofline = {
         "kernel": dom,

@@ -134,6 +134,24 @@ def test_pick_times_every_supported_tile_on_a_miss(tmp_path, monkeypatch):
     tuner.reset()
 
 
+def test_pick_prefers_the_default_tile_on_a_near_tie(tmp_path, monkeypatch):
+    monkeypatch.setenv("TRIFAST_CONFIG_DIR", str(tmp_path))
+    monkeypatch.setenv("TRIFAST_AUTOTUNE", "1")
+    monkeypatch.delenv("TRIFAST_FORCE_TUNE", raising=False)
+    monkeypatch.setattr(tuner, "_device_tag", lambda device=None: "Test-GPU_9-5")
+    default = _lib.load().trifast_default_tile(_lib.KERNEL_BWD_KV, 1024, 4, 32, _lib.BF16)
+    other = next(t for t in tuner.supported_tiles(_lib.KERNEL_BWD_KV, 1024, 4, 32, torch.bfloat16) if t != default)
+    # 1 % faster is within the scatter of the timings: the default stays
+    monkeypatch.setattr(tuner, "_time_launch", lambda launch, tile, **kw: 0.99 if tile == other else (1.0 if tile == default else 5.0))
+    tuner.reset()
+    assert tuner.pick(_lib.KERNEL_BWD_KV, 1024, 4, 32, torch.bfloat16, lambda t: None) == default
+    # 10 % faster replaces it
+    monkeypatch.setenv("TRIFAST_FORCE_TUNE", "1")
+    monkeypatch.setattr(tuner, "_time_launch", lambda launch, tile, **kw: 0.9 if tile == other else (1.0 if tile == default else 5.0))
+    assert tuner.pick(_lib.KERNEL_BWD_KV, 1024, 4, 32, torch.bfloat16, lambda t: None) == other
+    tuner.reset()
+
+
 def test_tune_cli_flags_and_sweep():
     p = tune.build_parser()
     a = p.parse_args([])

@@ -38,6 +38,9 @@ _TRUE = ("1", "true", "yes", "on")
 FILE_LOCK = threading.Lock()
 
 
+TIE_MARGIN = 1.02  # a tile must beat the default by more than this factor to replace it
+
+
 def force_tune() -> bool:
     return os.getenv("TRIFAST_FORCE_TUNE", "0").lower() in _TRUE
 
@@ -197,6 +200,11 @@ def pick(kernel: int, n: int, h: int, d: int, dtype: torch.dtype, launch: Callab
     else:
         cache.timings = {t: _time_launch(launch, t) for t in tiles}
         best = min(cache.timings, key=cache.timings.get)
+        # near-ties go to the library's default tile: timings of a few launches scatter by
+        # a percent or two, and a stable choice is worth more than that
+        default = lib.trifast_default_tile(kernel, n, h, d, code)
+        if default in cache.timings and cache.timings[default] <= TIE_MARGIN * cache.timings[best]:
+            best = default
     cache.cache[key] = best
     cache.write()
     if print_autotuning():
