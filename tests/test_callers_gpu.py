@@ -1,0 +1,76 @@
+"""Callers either side of the operator: leading batch dims and the ending-node entry.
+
+Both are thin host-side layers over the starting-node operator; they are checked
+against the oracle (leading dims: one call per batch element) and against the
+ending-node formula written out with einsum (AlphaFold 2 supplement, algorithm 14),
+values and gradients, with the reference's tolerance rule (tests/utils.py:31-36).
+"""
+
+import math
+
+import pytest
+import torch
+
+import trifast_amd
+from oracle import triangle_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _inputs(lead, h, n, d, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = (torch.randn(*lead, h, n, n, d, generator=g) for _ in range(3))
+    b = torch.randn(*lead, h, n, n, generator=g)
+    mask = torch.rand(*lead, n, n, generator=g) < 0.25
+    do = torch.randn(*lead, h, n, n, d, generator=g)
+    return [t.to(DEV).to(dtype) for t in (q, k, v, b)] + [mask.to(DEV), do.to(DEV).to(dtype)]
+
+
+def ending_node_reference(q, k, v, b, mask):
+    """a[i,j,k] = softmax_k(q[i,j].k[k,j]/sqrt(d) + b[k,i] + mask[k,j]*min); o[i,j] = sum_k a[i,j,k] v[k,j]."""
+    d = q.shape[-1]
+    s = torch.einsum("bhijd,bhkjd->bhijk", q, k) / math.sqrt(d)
+    s = s + b.permute(0, 1, 3, 2)[:, :, :, None, :]  # [b,h,i,1,k] <- b[k,i]
+    s = s + (mask.to(s.dtype) * torch.finfo(s.dtype).min).permute(0, 2, 1)[:, None, None, :, :]  # [b,1,1,j,k] <- mask[k,j]
+    return torch.einsum("bhijk,bhkjd->bhijd", torch.softmax(s, dim=-1), v)
+
+
+def _grads(fn, q, k, v, b, mask, do):
+    q, k, v, b = (t.detach().clone().requires_grad_(True) for t in (q, k, v, b))
+    o = fn(q, k, v, b, mask)
+    o.backward(do)
+    return o.detach(), q.grad, k.grad, v.grad, b.grad
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_ending_node_entry(dtype):
+    q, k, v, b, mask, do = _inputs((2,), 2, 40, 32, dtype, seed=11)
+    got = _grads(trifast_amd.triangle_attention_ending_node, q, k, v, b, mask, do)
+    f32 = lambda t: t.float()
+    ref = _grads(ending_node_reference, f32(q), f32(k), f32(v), f32(b), mask, f32(do))
+    pt = _grads(ending_node_reference, q, k, v, b, mask, do)
+    for name, x, p, r in zip(("o", "dq", "dk", "dv", "db"), got, pt, ref):
+        assert x.shape == r.shape
+        orc.compare_values(x, p, r, f"ending node {dtype} {name}", eps=orc.DTYPE_EPS[dtype])
+
+
+@pytest.mark.parametrize("lead", [(), (2, 3)], ids=["no_batch", "two_batch_dims"])
+def test_leading_batch_dims(lead):
+    dtype = torch.bfloat16
+    q, k, v, b, mask, do = _inputs(lead, 2, 33, 32, dtype, seed=5)
+    got = _grads(trifast_amd.triangle_attention, q, k, v, b, mask, do)
+    assert got[0].shape == q.shape and got[4].shape == b.shape
+    # the same, one batch element at a time through the 5-D operator
+    fold = lambda t, keep: t.reshape(-1, *t.shape[-keep:])
+    fq, fk, fv, fb, fm, fdo = fold(q, 4), fold(k, 4), fold(v, 4), fold(b, 3), fold(mask, 2), fold(do, 4)
+    for x in range(fq.shape[0]):
+        one = _grads(trifast_amd.triangle_attention, fq[x : x + 1], fk[x : x + 1], fv[x : x + 1], fb[x : x + 1], fm[x : x + 1], fdo[x : x + 1])
+        for name, a, c in zip(("o", "dq", "dk", "dv", "db"), got, one):
+            assert torch.equal(fold(a, c.dim() - 1)[x : x + 1], c), f"batch element {x}: {name} differs"
+
+
+def test_leading_dims_must_agree():
+    q, k, v, b, mask, _ = _inputs((2, 3), 1, 16, 16, torch.float32, seed=1)
+    with pytest.raises(ValueError, match="leading batch dims"):
+        trifast_amd.triangle_attention(q, k, v, b[0], mask)

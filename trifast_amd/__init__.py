@@ -1,10 +1,11 @@
 """trifast_amd: fused triangle self-attention for AMD Instinct MI355X (gfx950).
 
-Same Python surface as the reference package (src/trifast/__init__.py:1-3).
+Same Python surface as the reference package (src/trifast/__init__.py:1-3), plus an
+ending-node entry on untransposed tensors.
 """
 
-from trifast_amd.torch import triangle_attention
+from trifast_amd.torch import triangle_attention, triangle_attention_ending_node
 
 __version__ = "0.1.12"
 
-__all__ = ["triangle_attention"]
+__all__ = ["triangle_attention", "triangle_attention_ending_node"]

@@ -224,6 +224,47 @@ def triangle_attention(
     q, k, v: [b, h, n, n, d]; b (bias): [b, h, n, n]; mask: [b, n, n] bool with
     True = key masked out.  Returns o: [b, h, n, n, d].  Reference
     src/trifast/torch.py:220-228.
+
+    Beyond the reference (its own TODO, src/trifast/torch.py:29,84): any number of
+    leading batch dims, q [*batch, h, n, n, d] with bias [*batch, h, n, n] and mask
+    [*batch, n, n], including none at all; they are folded into one batch dim (views
+    where the layout allows it) and restored on the output.
     """
-    o, _ = _triangle_attention(q, k, v, b, mask)
-    return o
+    if q.dim() == 5:
+        o, _ = _triangle_attention(q, k, v, b, mask)
+        return o
+    if q.dim() < 4:
+        raise ValueError(f"q must be [*batch, h, n, n, d], got shape {tuple(q.shape)}")
+    lead = q.shape[:-4]
+    if b.shape[:-3] != lead or mask.shape[:-2] != lead or k.shape != q.shape or v.shape != q.shape:
+        raise ValueError(
+            f"leading batch dims must agree: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}, "
+            f"bias {tuple(b.shape)}, mask {tuple(mask.shape)}"
+        )
+    fold = lambda t, keep: t.reshape(-1, *t.shape[-keep:])
+    o, _ = _triangle_attention(fold(q, 4), fold(k, 4), fold(v, 4), fold(b, 3), fold(mask, 2))
+    return o.reshape(*lead, *o.shape[1:])
+
+
+def triangle_attention_ending_node(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    b: torch.Tensor,
+    mask: torch.Tensor,
+) -> torch.Tensor:
+    """Triangle self-attention around the ending node, on tensors in the ordinary
+    (untransposed) pair layout:
+
+        a[i, j, k] = softmax_k(q[i, j] . k[k, j] / sqrt(d) + b[k, i] + mask[k, j] * finfo.min)
+        o[i, j]    = sum_k a[i, j, k] v[k, j]
+
+    with q, k, v: [*batch, h, n, n, d] indexed [.., i, j, :], b: [*batch, h, n, n],
+    mask: [*batch, n, n] (True = masked out).  This is the starting-node operator on
+    the pair-transposed problem; the transposes are views (q, k, v are read in place
+    through their strides, bias and mask are re-tiled by the pre-passes anyway), so
+    nothing is copied.  The result is a transposed view of a contiguous tensor.
+    The reference has no such entry: its callers transpose and copy by hand.
+    """
+    t = lambda x: x.transpose(-3, -2)
+    return t(triangle_attention(t(q), t(k), t(v), b.transpose(-1, -2), mask.transpose(-1, -2)))
