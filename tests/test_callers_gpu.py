@@ -74,3 +74,69 @@ def test_leading_dims_must_agree():
     q, k, v, b, mask, _ = _inputs((2, 3), 1, 16, 16, torch.float32, seed=1)
     with pytest.raises(ValueError, match="leading batch dims"):
         trifast_amd.triangle_attention(q, k, v, b[0], mask)
+
+
+class PairAttentionBlock(torch.nn.Module):
+    """Projections of a pair representation x [b, n, n, c] into q, k, v, bias, then the
+    operator: the module of reference tests/unit/test_trifast.py:152-169, with the heads
+    moved in front of the pair dims as the operator expects ([b, h, n, n, d])."""
+
+    def __init__(self, h: int, d: int, attention):
+        super().__init__()
+        self.h, self.attention = h, attention
+        self.q = torch.nn.Linear(d, h * d)
+        self.k = torch.nn.Linear(d, h * d)
+        self.v = torch.nn.Linear(d, h * d)
+        self.b = torch.nn.Linear(d, h)
+
+    def forward(self, x, mask):
+        heads = lambda t: t.unflatten(-1, (self.h, -1)).permute(0, 3, 1, 2, 4)  # views: read in place
+        return self.attention(heads(self.q(x)), heads(self.k(x)), heads(self.v(x)), self.b(x).permute(0, 3, 1, 2), mask)
+
+
+@pytest.mark.parametrize(
+    "n,h,d,do_mask,bs,dtype",
+    [(16, 1, 16, False, 1, torch.float16), (32, 1, 32, False, 1, torch.bfloat16), (64, 1, 64, False, 4, torch.float32), (48, 4, 32, True, 2, torch.bfloat16)],
+)
+def test_weight_updates(n, h, d, do_mask, bs, dtype):
+    """Reference tests/unit/test_trifast.py:172-210: every parameter of a module around the
+    operator moves under Adam."""
+    torch.manual_seed(0)
+    x = torch.randn(bs, n, n, d, device=DEV, dtype=dtype, requires_grad=True)
+    model = PairAttentionBlock(h, d, trifast_amd.triangle_attention).to(DEV, dtype)
+    opt = torch.optim.Adam(model.parameters(), lr=1e-3)
+    mask = torch.randint(0, 2, (bs, n, n), device=DEV, dtype=torch.bool) if do_mask else torch.zeros(bs, n, n, device=DEV, dtype=torch.bool)
+    before = {name: p.detach().clone() for name, p in model.named_parameters()}
+    for step in range(5):
+        out = model(x, mask)
+        label = torch.randn_like(out) * 4
+        opt.zero_grad()
+        torch.nn.functional.mse_loss(out, label).backward()
+        if step == 0:
+            # (later steps are Adam's business: in pure fp16 its epsilon underflows)
+            assert torch.isfinite(out).all()
+            for name, p in model.named_parameters():
+                assert torch.isfinite(p.grad).all() and p.grad.abs().max() > 0, f"gradient of {name}"
+        opt.step()
+    for name, p in model.named_parameters():
+        assert not torch.all(before[name] == p), f"parameter {name} did not update"
+
+
+def test_parameter_gradients_match_the_oracle():
+    """The same module around the oracle gives the same parameter and input gradients (fp32)."""
+    torch.manual_seed(1)
+    n, h, d, bs = 24, 2, 32, 2
+    x = torch.randn(bs, n, n, d, device=DEV)
+    mask = torch.rand(bs, n, n, device=DEV) < 0.2
+    label = torch.randn(bs, h, n, n, d, device=DEV)
+    ours = PairAttentionBlock(h, d, trifast_amd.triangle_attention).to(DEV)
+    theirs = PairAttentionBlock(h, d, orc.attention_reference).to(DEV)
+    theirs.load_state_dict(ours.state_dict())
+    grads = []
+    for model in (ours, theirs):
+        xi = x.clone().requires_grad_(True)
+        torch.nn.functional.mse_loss(model(xi, mask), label).backward()
+        grads.append({"x": xi.grad, **{name: p.grad for name, p in model.named_parameters()}})
+    for name in grads[0]:
+        a, r = grads[0][name], grads[1][name]
+        assert (a - r).abs().max().item() <= 2e-5 * max(r.abs().max().item(), 1e-6) + 1e-7, f"{name}: {(a - r).abs().max().item():.3e}"
