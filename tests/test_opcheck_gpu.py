@@ -56,3 +56,51 @@ def test_compile_fullgraph_matches_eager():
         assert torch.equal(x, y), f"{name} differs between compiled and eager"
     ref = orc.attention_reference(q.float(), k.float(), v.float(), b.float(), m)
     assert (oc.float() - ref).abs().max() < 0.05
+
+
+def test_hip_graph_capture_and_replay():
+    """Forward and backward captured into one HIP graph (what `mode="reduce-overhead"`
+    does underneath, reference scripts/compile.py:5-24): the library launches kernels
+    only — no allocation, no memset, no synchronisation — so capture records it whole.
+    Every replay, with eager work and a synchronisation between replays and new input
+    values each time, must reproduce the eager result bit for bit."""
+    n, h, d = 96, 2, 32
+    dev, dtype = "cuda", torch.bfloat16
+    gen = torch.Generator(device=dev).manual_seed(3)
+    rand = lambda *shape: torch.randn(*shape, device=dev, dtype=dtype, generator=gen)
+    q, k, v = (rand(1, h, n, n, d).requires_grad_(True) for _ in range(3))
+    b = rand(1, h, n, n).requires_grad_(True)
+    mask = torch.rand(1, n, n, device=dev, generator=gen) < 0.2
+    do = rand(1, h, n, n, d)
+
+    def step():
+        o = trifast_amd.triangle_attention(q, k, v, b, mask)
+        o.backward(do)
+        return o
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):  # warm-up outside the capture, as graph capture of autograd needs
+            step()
+            for t in (q, k, v, b):
+                t.grad = None
+    torch.cuda.current_stream().wait_stream(side)
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        o = step()
+    for trial in range(3):
+        with torch.no_grad():
+            for t in (q, k, v, b, do):
+                t.copy_(rand(*t.shape))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [x.detach().clone() for x in (o, q.grad, k.grad, v.grad, b.grad)]
+        # the same step eagerly, on copies
+        eq, ek, ev, eb = (t.detach().clone().requires_grad_(True) for t in (q, k, v, b))
+        eo = trifast_amd.triangle_attention(eq, ek, ev, eb, mask)
+        eo.backward(do)
+        torch.cuda.synchronize()
+        for name, x, e in zip(("o", "dq", "dk", "dv", "db"), got, (eo, eq.grad, ek.grad, ev.grad, eb.grad)):
+            assert torch.equal(x, e.detach()), f"replay {trial}: {name} differs from the eager result"
