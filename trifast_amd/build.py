@@ -32,6 +32,14 @@ HIPCC_FLAGS = [
 ]
 
 
+# per-source additions, measured on MI355X: the db kernel (4 waves per SIMD, short
+# dependent chains per row) runs 3-4 % faster when scheduled for instruction-level
+# parallelism; the other kernels are better off with the default strategy
+PER_SOURCE_FLAGS = {
+    "tri_bwd_b.hip": ["-mllvm", "-amdgpu-sched-strategy=max-ilp"],
+}
+
+
 def _hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -44,7 +52,7 @@ def sources() -> list[Path]:
 
 
 def _compile(src: Path, obj: Path, verbose: bool, extra: tuple[str, ...] = ()) -> None:
-    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *PER_SOURCE_FLAGS.get(src.name, []), *extra, "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src.name}:\n{res.stdout}\n{res.stderr}")
