@@ -190,8 +190,13 @@ __global__ __launch_bounds__(NW * 64, (bwd_kv_min_waves<T, D, R, BJ>())) void tr
   // One stage of compute.  The JU*R tiles run as a software pipeline inside the
   // wave: the two MFMA chains (scores, dP) of tile t+1 are issued before the
   // exponentials of tile t.  EDGE stages hold queries past the end.
-  auto compute_stage = [&](auto edge_tag, int jt0, int buf) __attribute__((always_inline)) {
+  // COMMON stages belong to a wave none of whose rows is fully masked or has a dead key
+  // tile: the stage then has no branch, and the MFMA chains of the next tile are
+  // scheduled into the vector arithmetic of the current one (branches would split them
+  // into blocks of their own).
+  auto compute_stage = [&](auto edge_tag, auto common_tag, int jt0, int buf) __attribute__((always_inline)) {
     constexpr bool EDGE = decltype(edge_tag)::value;
+    constexpr bool COMMON = decltype(common_tag)::value && !EDGE;
     const unsigned char* st = tri_smem + buf * STAGE;
     if (!wave_active) return;
     constexpr int TS = JU * R;
@@ -214,7 +219,7 @@ __global__ __launch_bounds__(NW * 64, (bwd_kv_min_waves<T, D, R, BJ>())) void tr
       // -lse per query and the key mask through one MFMA (see OffsetMask; the roles of
       // the two operands are swapped here: rows are queries, columns are keys)
       lseop.set(lw, g);
-      if (!flagged[r]) {
+      if (COMMON || !flagged[r]) {
         sc = E::mfma(lseop.get(), keyop[r], biasv[u]);
       } else {
         // rare: kept a real branch so that the common case starts from the bias
@@ -237,7 +242,7 @@ __global__ __launch_bounds__(NW * 64, (bwd_kv_min_waves<T, D, R, BJ>())) void tr
       const int u = t / R, r = t % R;
       f32x16 sn, dn;
       if (t + 1 < TS) chains(t + 1, sn, dn);
-      if (tile_live[r] && (!EDGE || jt0 + 32 * u < N)) {
+      if (COMMON || (tile_live[r] && (!EDGE || jt0 + 32 * u < N))) {
         float p[16], ds[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
@@ -267,28 +272,37 @@ __global__ __launch_bounds__(NW * 64, (bwd_kv_min_waves<T, D, R, BJ>())) void tr
     issue_loads(0, 0);
     wait_dma();
     __syncthreads();
-    int s = 0;
-    for (; s + 1 < nfull; s += 2) {
-      issue_loads((s + 1) * BJ, 1);
-      compute_stage(std::false_type{}, s * BJ, 0);
-      wait_dma();
-      __syncthreads();
-      if ((s + 2) * BJ < N) issue_loads((s + 2) * BJ, 0);
-      compute_stage(std::false_type{}, (s + 1) * BJ, 1);
-      wait_dma();
-      __syncthreads();
-    }
+    // (the whole loop exists twice; a wave picks its version once.  Both run the same
+    // stages and barriers.)
+    auto whole_stages = [&](auto common_tag) __attribute__((always_inline)) {
+      int s = 0;
+      for (; s + 1 < nfull; s += 2) {
+        issue_loads((s + 1) * BJ, 1);
+        compute_stage(std::false_type{}, common_tag, s * BJ, 0);
+        wait_dma();
+        __syncthreads();
+        if ((s + 2) * BJ < N) issue_loads((s + 2) * BJ, 0);
+        compute_stage(std::false_type{}, common_tag, (s + 1) * BJ, 1);
+        wait_dma();
+        __syncthreads();
+      }
+      return s;
+    };
+    bool common = wave_active;
+#pragma unroll
+    for (int r = 0; r < R; ++r) common = common && !flagged[r] && tile_live[r];
+    const int s = common ? whole_stages(std::true_type{}) : whole_stages(std::false_type{});
     // buffer 0 now holds stage s: the last whole one, the ragged one, or a spare
     if (s < nfull) {
       if (ragged) issue_loads((s + 1) * BJ, 1);
-      compute_stage(std::false_type{}, s * BJ, 0);
+      compute_stage(std::false_type{}, std::false_type{}, s * BJ, 0);
       if (ragged) {
         wait_dma();
         __syncthreads();
-        compute_stage(std::true_type{}, (s + 1) * BJ, 1);
+        compute_stage(std::true_type{}, std::false_type{}, (s + 1) * BJ, 1);
       }
     } else if (ragged) {
-      compute_stage(std::true_type{}, s * BJ, 0);
+      compute_stage(std::true_type{}, std::false_type{}, s * BJ, 0);
     }
   } else {
     // one stage only (the double buffer does not fit in LDS): load, then compute
@@ -296,14 +310,14 @@ __global__ __launch_bounds__(NW * 64, (bwd_kv_min_waves<T, D, R, BJ>())) void tr
       issue_loads(s * BJ, 0);
       wait_dma();
       __syncthreads();
-      compute_stage(std::false_type{}, s * BJ, 0);
+      compute_stage(std::false_type{}, std::false_type{}, s * BJ, 0);
       __syncthreads();
     }
     if (ragged) {
       issue_loads(nfull * BJ, 0);
       wait_dma();
       __syncthreads();
-      compute_stage(std::true_type{}, nfull * BJ, 0);
+      compute_stage(std::true_type{}, std::false_type{}, nfull * BJ, 0);
     }
   }
 
