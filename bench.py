@@ -126,6 +126,16 @@ def _event_ms(fn, reps):
     return start.elapsed_time(end) / reps
 
 
+def _quantile(sorted_values, q):
+    """Linear-interpolated quantile of an ascending list."""
+    if not sorted_values:
+        return None
+    x = q * (len(sorted_values) - 1)
+    lo = int(x)
+    hi = min(lo + 1, len(sorted_values) - 1)
+    return sorted_values[lo] + (sorted_values[hi] - sorted_values[lo]) * (x - lo)
+
+
 def kernel_breakdown(q, k, v, bias, mask, do, reps):
     """Average launch duration (ms) of the four kernels, each timed with events on the
     stream it is launched on (torch's current stream), through the C ABI."""
@@ -255,16 +265,28 @@ def main():
     torch.cuda.synchronize()
     torch.cuda.reset_peak_memory_stats()
     base_mem = torch.cuda.memory_allocated()
+    # the K timed steps: wall clock around all of them (the headline), and an event pair
+    # per step for the spread (median, 10th and 90th percentile)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    marks[0].record()
+    for i in range(args.steps):
         step()
+        marks[i + 1].record()
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
     peak_extra = torch.cuda.max_memory_allocated() - base_mem
 
     fwd_only()
     torch.cuda.synchronize()
     ms_fwd = _event_ms(fwd_only, args.steps)
+    # matrix peak at the device's maximum shader clock: 4096 dense bf16/fp16 FLOP per clock and CU
+    from trifast_amd import _lib
+
+    clock_mhz = _lib.load().trifast_device_clock_mhz(dev.index or 0)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    peak_at_clock = cus * 4096 * clock_mhz / 1e6 if clock_mhz > 0 else None
 
     f_fwd, f_bwd = flops(b, h, n, d)
     peak = PEAK_F32_TFLOPS if dtype == torch.float32 else PEAK_BF16_TFLOPS
@@ -311,6 +333,10 @@ def main():
         "fwd_tflops": tf_fwd,
         "fwd_frac_of_peak": tf_fwd / peak,
         "peak_extra_mem_mib": peak_extra / 2**20,
+        "step_ms_quantiles": {"p10": _quantile(per_step, 0.1), "median": _quantile(per_step, 0.5), "p90": _quantile(per_step, 0.9)},
+        "peak_tflops_nominal": peak,
+        "max_clock_mhz": clock_mhz,
+        "peak_tflops_at_max_clock": None if dtype == torch.float32 else peak_at_clock,
         "kernels": {name: {"ms": round(rec["ms"], 4), "tflops": round(rec["tflops"], 1), "tile": rec["tile"]} for name, rec in kern.items()},
         "roofline": roofline,
         "autotune": tuner.autotune_enabled(),

@@ -63,6 +63,13 @@ int trifast_abi_version(void);
 const char* trifast_last_error(void);
 
 /*
+ * Maximum shader clock of a device in MHz (negative error code on failure).  No
+ * counterpart in the reference: the benchmark uses it to state the matrix peak at the
+ * device's own clock next to the nominal one.
+ */
+int trifast_device_clock_mhz(int device);
+
+/*
  * Compiled tile instantiations, for the tuner.  Replaces the triton.Config lists
  * of reference src/trifast/autotune_helpers.py:58-211.
  *   trifast_num_tiles(kernel)            number of instantiations of that kernel

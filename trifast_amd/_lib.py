@@ -28,6 +28,7 @@ _INTP = POINTER(c_int)
 SIGNATURES = {
     "trifast_abi_version": (c_int, []),
     "trifast_last_error": (c_char_p, []),
+    "trifast_device_clock_mhz": (c_int, [c_int]),
     "trifast_num_tiles": (c_int, [c_int]),
     "trifast_tile_info": (c_int, [c_int, c_int, _INTP, _INTP, _INTP]),
     "trifast_supports": (c_int, [c_int, c_int, c_int64, c_int64, c_int64, c_int]),

@@ -228,6 +228,17 @@ int trifast_abi_version(void) { return TRIFAST_ABI_VERSION; }
 
 const char* trifast_last_error(void) { return g_err; }
 
+int trifast_device_clock_mhz(int device) {
+  g_err[0] = 0;
+  int khz = 0;
+  const hipError_t e = hipDeviceGetAttribute(&khz, hipDeviceAttributeClockRate, device);
+  if (e != hipSuccess) {
+    hip_fail(e, "hipDeviceGetAttribute(clock rate)");
+    return TRIFAST_EINVAL;
+  }
+  return khz / 1000;
+}
+
 int trifast_num_tiles(int kernel) {
   switch (kernel) {
     case TRIFAST_KERNEL_FWD: return tri::fwd_num_tiles();
