@@ -140,3 +140,14 @@ def test_parameter_gradients_match_the_oracle():
     for name in grads[0]:
         a, r = grads[0][name], grads[1][name]
         assert (a - r).abs().max().item() <= 2e-5 * max(r.abs().max().item(), 1e-6) + 1e-7, f"{name}: {(a - r).abs().max().item():.3e}"
+
+
+def test_device_clock_export():
+    """The benchmark's helper reports a plausible shader clock and rejects a bad device."""
+    from trifast_amd import _lib
+
+    lib = _lib.load()
+    mhz = lib.trifast_device_clock_mhz(0)
+    assert 500 <= mhz <= 5000, mhz
+    assert lib.trifast_device_clock_mhz(10_000) < 0
+    assert "clock" in _lib.last_error()

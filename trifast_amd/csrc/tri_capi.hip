@@ -230,10 +230,13 @@ const char* trifast_last_error(void) { return g_err; }
 
 int trifast_device_clock_mhz(int device) {
   g_err[0] = 0;
-  int khz = 0;
-  const hipError_t e = hipDeviceGetAttribute(&khz, hipDeviceAttributeClockRate, device);
+  int count = 0, khz = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e == hipSuccess && (device < 0 || device >= count)) return fail(TRIFAST_EINVAL, "device clock: no device %d (%d visible)", device, count);
+  if (e == hipSuccess) e = hipDeviceGetAttribute(&khz, hipDeviceAttributeClockRate, device);
   if (e != hipSuccess) {
-    hip_fail(e, "hipDeviceGetAttribute(clock rate)");
+    (void)hipGetLastError();  // the runtime keeps the error for the next caller otherwise
+    hip_fail(e, "device clock");
     return TRIFAST_EINVAL;
   }
   return khz / 1000;
