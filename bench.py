@@ -164,7 +164,7 @@ def kernel_breakdown(q, k, v, bias, mask, do, reps):
     def bwd_one(kernel, tile):
         rc = lib.trifast_bwd_one(kernel, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), db.data_ptr(), dov.data_ptr(), qv.data_ptr(), kv.data_ptr(),
                                  vv.data_ptr(), bv.data_ptr(), mu8.data_ptr(), o.data_ptr(), lse.data_ptr(), b, h, n, d, code,
-                                 S(dov), S(qv), S(kv), S(vv), S(bv), S(mu8), tile, ws.data_ptr(), ws.numel(), stream)
+                                 S(dov), S(qv), S(kv), S(vv), S(bv), S(mu8), None, None, None, None, tile, ws.data_ptr(), ws.numel(), stream)
         _lib.check(rc, "trifast_bwd_one")
 
     for kernel in (_lib.KERNEL_FWD, _lib.KERNEL_BWD_Q, _lib.KERNEL_BWD_KV, _lib.KERNEL_BWD_B):

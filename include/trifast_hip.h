@@ -18,10 +18,14 @@
  *       q, k, v, do : [b, h, n, n, d]  element strides {sb, sh, si, sj, sd}, sd == 1
  *       bias        : [b, h, n, n]     element strides {sb, sh, sj, sk}, any
  *       mask        : [b, n, n] bytes  strides {sb, si, sk}, any; nonzero = key masked OUT
- *       o, dq, dk, dv : contiguous [b, h, n, n, d];  db : contiguous [b, h, n, n]
+ *       o           : contiguous [b, h, n, n, d]
+ *       dq, dk, dv  : [b, h, n, n, d]  element strides like q (sd == 1), or contiguous
+ *       db          : [b, h, n, n]     element strides {sb, sh, sj, sk}, any, or contiguous
  *       lse         : contiguous float32 [b, h, n, n], natural log, indexed [i, j]
- *     Vector loads need 16-byte alignment: base pointers of q, k, v, do, o must be
- *     16-byte aligned and their si/sj/sh/sb strides multiples of 16/sizeof(elem).
+ *     Vector accesses need 16-byte alignment: base pointers of q, k, v, do, o, dq, dk,
+ *     dv, db must be 16-byte aligned and the si/sj/sh/sb strides of the q-like ones
+ *     multiples of 16/sizeof(elem); lse must be 4-byte aligned.  Outputs must not
+ *     overlap themselves or each other (no zero strides over a dim larger than 1).
  *     bias and mask are re-tiled by pre-pass kernels into the workspace, so they
  *     carry no alignment or contiguity requirement.
  */
@@ -35,7 +39,7 @@
 extern "C" {
 #endif
 
-#define TRIFAST_ABI_VERSION 1
+#define TRIFAST_ABI_VERSION 2
 
 /* dtype codes */
 #define TRIFAST_F32 0
@@ -107,6 +111,11 @@ int trifast_fwd(void* o, float* lse,
  * gradient has), but its rows must be 16-byte aligned with last stride 1: the
  * caller materialises a do that is not.  o and lse are the forward's contiguous
  * outputs.  tiles[3] = {bwd_q, bwd_kv, bwd_b} tile ids (<0: default).
+ * dq/dk/dv/db_strides give the layout the gradients are written in (NULL:
+ * contiguous).  The reference's backward allocates its gradients like its saved,
+ * possibly strided inputs (src/trifast/torch.py:85-104); passing the inputs' own
+ * strides lets a caller hand the gradients to leaves that are transposed views
+ * without a re-layout copy.
  */
 int trifast_bwd(void* dq, void* dk, void* dv, void* db,
                 const void* dout, const void* q, const void* k, const void* v,
@@ -114,6 +123,8 @@ int trifast_bwd(void* dq, void* dk, void* dv, void* db,
                 int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
                 const int64_t* do_strides, const int64_t* q_strides, const int64_t* k_strides,
                 const int64_t* v_strides, const int64_t* bias_strides, const int64_t* mask_strides,
+                const int64_t* dq_strides, const int64_t* dk_strides, const int64_t* dv_strides,
+                const int64_t* db_strides,
                 const int* tiles, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
@@ -129,6 +140,8 @@ int trifast_bwd_one(int kernel,
                     int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
                     const int64_t* do_strides, const int64_t* q_strides, const int64_t* k_strides,
                     const int64_t* v_strides, const int64_t* bias_strides, const int64_t* mask_strides,
+                    const int64_t* dq_strides, const int64_t* dk_strides, const int64_t* dv_strides,
+                    const int64_t* db_strides,
                     int tile, void* workspace, int64_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus

@@ -151,3 +151,78 @@ def test_device_clock_export():
     assert 500 <= mhz <= 5000, mhz
     assert lib.trifast_device_clock_mhz(10_000) < 0
     assert "clock" in _lib.last_error()
+
+
+def test_gradients_take_the_layout_of_transposed_leaves():
+    """Leaves that are pair-transposed views (the ending-node call pattern) receive
+    gradients written in their own layout by the kernels: autograd stores them as they
+    are instead of re-laying them out with a copy each (reference backward: gradients
+    follow the saved, possibly strided inputs, src/trifast/torch.py:85-104)."""
+    dtype = torch.float16
+    q, k, v, b, mask, do = _inputs((2,), 2, 72, 64, dtype, seed=21)
+    tq, tk, tv, tdo = (t.transpose(2, 3) for t in (q, k, v, do))
+    tb, tm = b.transpose(-1, -2), mask.transpose(-1, -2)
+    leaves = [t.detach().requires_grad_(True) for t in (tq, tk, tv, tb)]
+    assert not any(t.is_contiguous() for t in leaves)
+    from trifast_amd import torch as tt
+
+    o, lse = tt._triangle_attention(*leaves, tm)
+    raw = tt.triangle_attention_bwd(tdo, *(t.detach() for t in leaves), o.detach(), lse, tm)
+    for g, leaf in zip(raw[:4], leaves):
+        assert g.stride() == leaf.stride() and g.shape == leaf.shape
+    o.backward(tdo)
+    for g, leaf, r in zip((t.grad for t in leaves), leaves, raw[:4]):
+        assert g.stride() == leaf.stride()
+        assert torch.equal(g, r)
+    # values: against the oracle on the same views
+    f32 = lambda t: t.float()
+    ref = orc.forward_backward(f32(tq), f32(tk), f32(tv), f32(tb), tm, f32(tdo))
+    pt = orc.forward_backward(tq, tk, tv, tb, tm, tdo)
+    got = (o.detach(), *(t.grad for t in leaves))
+    for name, x, p, r in zip(("o", "dq", "dk", "dv", "db"), got, pt, ref):
+        orc.compare_values(x, p, r, f"strided gradients {name}", eps=orc.DTYPE_EPS[dtype])
+    # odd n: db rows are not 16-byte multiples, the strided scalar path is used
+    q, k, v, b, mask, do = _inputs((1,), 2, 37, 32, torch.bfloat16, seed=22)
+    tb = b.transpose(-1, -2)
+    got = _grads(trifast_amd.triangle_attention, q, k, v, tb, mask, do)
+    want = _grads(trifast_amd.triangle_attention, q, k, v, tb.contiguous(), mask, do)
+    assert torch.equal(got[4], want[4])
+
+
+def test_broadcast_upstream_gradient_is_not_materialised():
+    """``o.sum().backward()`` hands the backward an all-ones tensor with every stride 0
+    (the reference's own test and tuning protocol, tests/unit/test_trifast.py:51): it is
+    read as one row through zero strides, so no tensor of q's size is allocated for it."""
+    n, h, d = 256, 2, 32
+    dtype = torch.bfloat16
+    q, k, v, b, mask, _ = _inputs((1,), h, n, d, dtype, seed=23)
+    from trifast_amd import torch as tt
+
+    o, lse = tt._triangle_attention(q, k, v, b, mask)
+    ones = torch.ones((), device=DEV, dtype=dtype).expand(q.shape)
+    assert ones.stride() == (0, 0, 0, 0, 0)
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    got = tt.triangle_attention_bwd(ones, q, k, v, b, o, lse, mask)
+    torch.cuda.synchronize()
+    extra = torch.cuda.max_memory_allocated() - base
+    qbytes = q.numel() * q.element_size()
+    ws = _ws_bytes(1, h, n, d)
+    # three gradients of q's size, db, dmask, the workspace -- and not a fourth q-sized tensor
+    assert extra < 3 * qbytes + ws + qbytes // 2, (extra, qbytes, ws)
+    want = tt.triangle_attention_bwd(ones.contiguous(), q, k, v, b, o, lse, mask)
+    for x, y in zip(got[:4], want[:4]):
+        assert torch.equal(x, y)
+    # one [d] row expanded over b, h, i, j is the other all-zero-stride case
+    row = torch.randn(d, device=DEV).to(dtype).expand(q.shape)
+    got = tt.triangle_attention_bwd(row, q, k, v, b, o, lse, mask)
+    want = tt.triangle_attention_bwd(row.contiguous(), q, k, v, b, o, lse, mask)
+    for x, y in zip(got[:4], want[:4]):
+        assert torch.equal(x, y)
+
+
+def _ws_bytes(b, h, n, d):
+    from trifast_amd import _lib
+
+    return _lib.load().trifast_bwd_workspace_bytes(b, h, n, d, _lib.BF16)

@@ -100,8 +100,51 @@ def test_argument_errors_come_back_as_codes_not_crashes():
     bad_stride = _lib.i64_array([0, 0, 0, 32, 2])
     rc = lib.trifast_fwd(0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 1, 1, 8, 32, _lib.BF16, bad_stride, st5, st5, st4, st3, -1, None, 0, None)
     assert rc == -3 and "last stride" in _lib.last_error()
-    rc = lib.trifast_bwd_one(0, *([0x1000] * 12), 1, 1, 8, 32, _lib.BF16, st5, st5, st5, st5, st4, st3, -1, None, 0, None)
+    none4 = (None, None, None, None)
+    rc = lib.trifast_bwd_one(0, *([0x1000] * 12), 1, 1, 8, 32, _lib.BF16, st5, st5, st5, st5, st4, st3, *none4, -1, None, 0, None)
     assert rc == -1 and "backward kernel" in _lib.last_error()
+
+
+def test_output_pointers_and_strides_are_checked():
+    """Gradients and lse are written / read with vector accesses: a misaligned pointer or
+    a stride the kernels cannot write comes back as TRIFAST_EALIGN, not as a fault."""
+    lib = _lib.load()
+    st5 = _lib.i64_array([0, 0, 8 * 32, 32, 1])
+    st4 = _lib.i64_array([0, 0, 8, 1])
+    st3 = _lib.i64_array([0, 8, 1])
+    ws_bytes = lib.trifast_bwd_workspace_bytes(1, 1, 8, 32, _lib.BF16)
+
+    def bwd(dq=0x1000, dk=0x1000, dv=0x1000, db=0x1000, lse=0x1000, out_strides=(None, None, None, None)):
+        # (the workspace check comes after every pointer check, so a null workspace ends a
+        # call whose pointers were accepted with TRIFAST_EWORKSPACE before anything is launched)
+        return lib.trifast_bwd(dq, dk, dv, db, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, lse,
+                               1, 1, 8, 32, _lib.BF16, st5, st5, st5, st5, st4, st3, *out_strides, None, None, ws_bytes, None)
+
+    assert bwd() == -4
+    assert bwd(db=0x1002) == -3 and "db" in _lib.last_error()
+    assert bwd(lse=0x1002) == -3 and "lse" in _lib.last_error()
+    assert bwd(dq=0x1008) == -3 and "dq" in _lib.last_error()
+    assert bwd(dv=0x1004) == -3 and "dv" in _lib.last_error()
+    assert bwd(db=None) == -1 and "db" in _lib.last_error()
+    bad = _lib.i64_array([0, 0, 8 * 32, 32, 2])
+    assert bwd(out_strides=(bad, None, None, None)) == -3 and "dq" in _lib.last_error()
+    odd = _lib.i64_array([0, 0, 8 * 36, 36, 1])  # rows that are not 16-byte aligned
+    assert bwd(out_strides=(None, odd, None, None)) == -3 and "dk" in _lib.last_error()
+    transposed = _lib.i64_array([0, 0, 32, 8 * 32, 1])  # i <-> j transposed layout is fine
+    assert bwd(out_strides=(transposed, transposed, transposed, _lib.i64_array([0, 0, 1, 8]))) == -4
+    # forward: lse
+    rc = lib.trifast_fwd(0x1000, 0x1002, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 1, 1, 8, 32, _lib.BF16, st5, st5, st5, st4, st3, -1, None, 0, None)
+    assert rc == -3 and "lse" in _lib.last_error()
+
+
+def test_db_chunks_do_not_inflate_the_workspace():
+    """One chunk of pair rows stays one chunk whatever b*h is (no partials, no reduce
+    pass): an odd head count costs no more workspace per head than an even one."""
+    lib = _lib.load()
+    per_head = lambda h, n: lib.trifast_bwd_workspace_bytes(1, h, n, 32, _lib.BF16) / h
+    assert per_head(5, 2048) <= 1.01 * per_head(8, 2048)
+    assert per_head(5, 4096) <= 1.01 * per_head(8, 4096)
+    assert per_head(1, 4096) <= 1.01 * per_head(8, 4096)
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

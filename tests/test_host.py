@@ -162,3 +162,17 @@ def test_tune_cli_flags_and_sweep():
     assert len(tune.valid_dtypes("all")) == 3
     with pytest.raises(SystemExit):
         p.parse_args(["--dtype", "int8"])
+
+
+def test_equiv_module_matches_the_oracle():
+    """``trifast.equiv`` (the reference's public pure-PyTorch functions) gives the
+    oracle's numbers, fully masked rows included."""
+    from trifast.equiv import attention_reference, triangle_attention_simple
+    from oracle import triangle_oracle as orc
+
+    g = torch.Generator().manual_seed(3)
+    q, k, v, b, m = orc.gen_tensors(9, 8, 2, True, "cpu", torch.float32, 2, 1.0, generator=g)
+    m[:, 4, :] = True
+    q, k, v, b = (t.detach() for t in (q, k, v, b))
+    torch.testing.assert_close(attention_reference(q, k, v, b, m), orc.attention_reference(q, k, v, b, m), rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(triangle_attention_simple(q, k, v, b, m), orc.triangle_attention_simple(q, k, v, b, m), rtol=1e-6, atol=1e-6)

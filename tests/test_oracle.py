@@ -143,3 +143,66 @@ def test_golden_fixtures(name):
         torch.testing.assert_close(got, t[key], rtol=1e-5, atol=1e-6, msg=key)
         if f"{key}_f64" in t:
             torch.testing.assert_close(got.double(), t[f"{key}_f64"], rtol=1e-4, atol=2e-5, msg=key + "_f64")
+
+
+# ------------------------------------------------- checker helpers, hand-computed
+def test_cosine_similarity_hand_values():
+    # (1,2,2).(2,1,2) = 8, both norms 3: cos = 8/9; orthogonal and opposite vectors
+    a, b = torch.tensor([1.0, 2.0, 2.0]), torch.tensor([2.0, 1.0, 2.0])
+    assert abs(orc.cosine_similarity(a, b) - 8.0 / 9.0) < 1e-6
+    assert abs(orc.cosine_similarity(torch.tensor([1.0, 0.0, 0.0]), torch.tensor([0.0, 3.0, 0.0]))) < 1e-7
+    assert abs(orc.cosine_similarity(a, -2 * a) + 1.0) < 1e-6
+    # inputs of any shape and dtype are flattened and compared in float32
+    assert abs(orc.cosine_similarity(a.reshape(1, 3).bfloat16(), b.reshape(3, 1).half()) - 8.0 / 9.0) < 1e-6
+    # a zero vector gives 0, not NaN (the eps in the denominator)
+    assert orc.cosine_similarity(torch.zeros(3), b) == 0.0
+
+
+def test_direction_checks_hand_values():
+    ref = torch.tensor([1.0, 0.0, 0.0])
+    good = torch.tensor([1.0, 0.1, 0.0])      # cos = 1/sqrt(1.01) = 0.99504
+    worse = torch.tensor([1.0, 0.15, 0.0])    # cos = 1/sqrt(1.0225) = 0.98894
+    bad = torch.tensor([1.0, 1.0, 0.0])       # cos = 0.7071
+    orc.compare_directions(good, good, ref)
+    with pytest.raises(AssertionError, match="kernel->ref"):
+        orc.compare_directions(worse, good, ref)  # 0.98894 < 0.99
+    with pytest.raises(AssertionError, match="pt->ref"):
+        orc.compare_directions(good, worse, ref)
+    # relative rule: cos(kernel) >= 0.99 * cos(pt); 0.98894 >= 0.99 * 0.99504 = 0.98509
+    orc.compare_relative_direction(worse, good, ref)
+    orc.compare_relative_direction(bad, bad, ref)  # equal cosines always pass
+    with pytest.raises(AssertionError, match="relative direction"):
+        orc.compare_relative_direction(bad, good, ref)  # 0.7071 < 0.98509
+
+
+def test_compare_dot_hand_values():
+    # scores are dot(x, ref) / dot(ref, ref): ref.ref = 9; kernel 8/9, pt 9/9
+    ref = torch.tensor([1.0, 2.0, 2.0])
+    kern = torch.tensor([2.0, 1.0, 2.0])
+    with pytest.raises(AssertionError, match="dot product"):
+        orc.compare_dot(kern, ref, ref)  # 8/9 - 1 = -0.111 < -0.01
+    orc.compare_dot(kern, ref, ref, threshold=0.12)
+    orc.compare_dot(ref, kern, ref)       # a kernel better than pt is fine (+0.111)
+    orc.compare_dot(0.995 * ref, ref, ref)  # -0.005 >= -0.01
+    with pytest.raises(AssertionError):
+        orc.compare_dot(0.98 * ref, ref, ref)  # -0.02
+
+
+def test_gen_tensors_shapes_draw_order_and_mask():
+    n, d, h, bs = 24, 8, 3, 2
+    g = torch.Generator().manual_seed(5)
+    q, k, v, b, m = orc.gen_tensors(n, d, h, True, "cpu", torch.float32, bs, 2.0, generator=g)
+    assert q.shape == k.shape == v.shape == (bs, h, n, n, d) and b.shape == (bs, h, n, n) and m.shape == (bs, n, n)
+    assert all(t.requires_grad and t.dtype == torch.float32 for t in (q, k, v, b)) and m.dtype == torch.bool
+    # draw order q, k, v, bias, mask from one generator: replay the same draws by hand
+    g2 = torch.Generator().manual_seed(5)
+    for got in (q, k, v):
+        assert torch.equal(got.detach(), torch.normal(0, 2.0, (bs, h, n, n, d), generator=g2))
+    assert torch.equal(b.detach(), torch.normal(0, 2.0, (bs, h, n, n), generator=g2))
+    assert torch.equal(m, torch.randint(0, 2, (bs, n, n), generator=g2).bool())
+    # std is honoured; the mask is a fair coin (1152 draws: 3 sigma = 4.4 %)
+    assert abs(q.detach().std().item() - 2.0) < 0.05
+    assert abs(m.float().mean().item() - 0.5) < 0.06
+    # without a mask: all False (nothing masked out)
+    *_, m0 = orc.gen_tensors(n, d, h, False, "cpu", torch.float32, bs, 1.0, generator=g)
+    assert m0.dtype == torch.bool and not m0.any()

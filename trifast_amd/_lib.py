@@ -10,12 +10,9 @@ import ctypes
 from ctypes import POINTER, c_char_p, c_int, c_int64, c_void_p
 from pathlib import Path
 
-import os
+LIB_PATH = Path(__file__).resolve().parent / "libtrifast_hip.so"
 
-# TRIFAST_LIB points at another build of the same library (kernel experiments)
-LIB_PATH = Path(os.environ.get("TRIFAST_LIB") or Path(__file__).resolve().parent / "libtrifast_hip.so")
-
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 F32, BF16, F16 = 0, 1, 2
 KERNEL_FWD, KERNEL_BWD_Q, KERNEL_BWD_KV, KERNEL_BWD_B = 0, 1, 2, 3
@@ -48,6 +45,7 @@ SIGNATURES = {
          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
          c_int64, c_int64, c_int64, c_int64, c_int,
          _I64P, _I64P, _I64P, _I64P, _I64P, _I64P,
+         _I64P, _I64P, _I64P, _I64P,
          _INTP, c_void_p, c_int64, c_void_p],
     ),
     "trifast_bwd_one": (
@@ -56,6 +54,7 @@ SIGNATURES = {
          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
          c_int64, c_int64, c_int64, c_int64, c_int,
          _I64P, _I64P, _I64P, _I64P, _I64P, _I64P,
+         _I64P, _I64P, _I64P, _I64P,
          c_int, c_void_p, c_int64, c_void_p],
     ),
 }

@@ -67,8 +67,8 @@ def _compile(src: Path, obj: Path, verbose: bool, extra: tuple[str, ...] = ()) -
 def build(verbose: bool = False, jobs: int | None = None, out: Path | None = None, extra: tuple[str, ...] = ()) -> Path:
     """Compile every translation unit and link the shared library.  Always rebuilds.
 
-    ``out`` / ``extra`` build a variant (other output path, extra hipcc flags such as
-    ``-DNAME``) without touching the in-tree library; used for kernel experiments."""
+    ``out`` writes the library elsewhere and ``extra`` appends hipcc flags (e.g. ``-DNAME``);
+    the in-tree library is then left alone."""
     out = Path(out) if out else LIB_PATH
     build_dir = PKG_DIR / "build" / (out.stem if out != LIB_PATH else "main")
     build_dir.mkdir(parents=True, exist_ok=True)
@@ -91,11 +91,4 @@ def build(verbose: bool = False, jobs: int | None = None, out: Path | None = Non
 
 
 if __name__ == "__main__":
-    import argparse
-
-    ap = argparse.ArgumentParser(description=__doc__)
-    ap.add_argument("--out", default=None, help="write the library here instead of in-tree")
-    ap.add_argument("extra", nargs="*", help="extra hipcc flags, e.g. -DNAME (after --)")
-    ns = ap.parse_args()
-    path = build(verbose=True, out=ns.out, extra=tuple(ns.extra))
-    print(f"built {path}")
+    print(f"built {build(verbose=True)}")

@@ -58,6 +58,8 @@ struct BwdArgs {
   float* dbpart;             // [nchunks, b*h, n, n] fp32 partial db (nchunks > 1 only)
   void *dq, *dk, *dv, *db;
   Str5 sq, sk, sv, sdo;
+  Str5 sdq, sdk, sdv;        // element strides of the gradients (d stride 1)
+  int64_t sdb_b, sdb_h, sdb_j, sdb_k;  // element strides of db [b, h, j, k]
   int H, N, NP, nwords;
   int BH;                    // b * h
   int nchunks, rows_per_chunk;  // db kernel: split of the pair rows over workgroups

@@ -37,8 +37,7 @@ struct BwdBFamily {
       hipError_t e = launch_dyn(tri_bwd_b_kernel<T, D, GJ, GK, WJ, WK, nbuf>, grid, dim3(GJ * GK * 64), lds, st, a);
       if (e != hipSuccess || a.nchunks == 1) return e;
       const int64_t count = (int64_t)bh * a.N * a.N;
-      hipLaunchKernelGGL(tri_bwd_b_reduce_kernel<T>, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st,
-                         a.dbpart, reinterpret_cast<T*>(a.db), count, a.nchunks);
+      hipLaunchKernelGGL(tri_bwd_b_reduce_kernel<T>, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st, a, count);
       return hipGetLastError();
     } else {
       return hipErrorInvalidConfiguration;
@@ -71,12 +70,17 @@ int bwd_b_chunks(int64_t n, int64_t bh) {
   if (chunks > max_chunks) chunks = max_chunks;
   if (chunks > 8) chunks = 8;
   if (chunks < 1) chunks = 1;
-  // The kernel runs each (batch*head, chunk) group on one XCD: make the number of
-  // groups a multiple of the 8 XCDs when the row count allows it.
-  int64_t g = bh % 8 == 0 ? 8 : (bh % 4 == 0 ? 4 : (bh % 2 == 0 ? 2 : 1));
-  const int64_t m = 8 / g;  // chunks must be a multiple of m
-  const int64_t rounded = (chunks + m - 1) / m * m;
-  if (rounded <= max_chunks && rounded <= 8) chunks = rounded;
+  // The kernel runs each (batch*head, chunk) group on one XCD: when the rows are split
+  // anyway, make the number of groups a multiple of the 8 XCDs if the row count allows
+  // it.  (One chunk stays one chunk: it needs no partials and no reduce pass.)
+  if (chunks > 1) {
+    int64_t g = bh % 8 == 0 ? 8 : (bh % 4 == 0 ? 4 : (bh % 2 == 0 ? 2 : 1));
+    const int64_t m = 8 / g;  // chunks must be a multiple of m
+    const int64_t rounded = (chunks + m - 1) / m * m;
+    if (rounded <= max_chunks && rounded <= 8) chunks = rounded;
+  }
+  // the groups are the grid's z extent (padded to a multiple of 8), at most 65535
+  while (chunks > 1 && (bh * chunks + 7) / 8 * 8 > 65535) --chunks;
   return (int)chunks;
 }
 

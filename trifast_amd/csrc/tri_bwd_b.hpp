@@ -349,9 +349,11 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   // a single chunk writes db itself; several chunks write fp32 partials.  The lane
   // owns query j; its 16 values are two runs of 8 consecutive keys.
   const bool direct = a.nchunks == 1;
-  T* db_bh = reinterpret_cast<T*>(a.db) + (int64_t)bh * N * N;
+  T* db_bh = reinterpret_cast<T*>(a.db) + b * a.sdb_b + h * a.sdb_h;
   float* part = a.dbpart + ((int64_t)chunk * a.BH + bh) * N * N;
   const bool vec_store = (N % 8) == 0;
+  // 16-byte stores of 8 keys need db contiguous along k with rows that stay aligned
+  const bool db_vec = a.sdb_k == 1 && ((a.sdb_j | a.sdb_h | a.sdb_b) % 8) == 0;
 #pragma unroll
   for (int tj = 0; tj < WJ; ++tj) {
     const int j = j_wave + 32 * tj + jl;
@@ -378,8 +380,8 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
           }
           continue;
         }
-        T* dst = db_bh + (int64_t)j * N + key0;
-        if (vec_store && key0 + 8 <= N) {
+        T* dst = db_bh + j * a.sdb_j + key0 * a.sdb_k;
+        if (db_vec && key0 + 8 <= N) {
           if constexpr (sizeof(T) == 2) {
             typename E::vec ov;
 #pragma unroll
@@ -397,7 +399,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (key0 + e < N) dst[e] = (T)dbacc[tj][tk][8 * r + e];
+            if (key0 + e < N) dst[e * a.sdb_k] = (T)dbacc[tj][tk][8 * r + e];
         }
       }
     }
@@ -406,12 +408,13 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
 
 // db = sum over chunks of the fp32 partials, in chunk order
 template <typename T>
-__global__ __launch_bounds__(256) void tri_bwd_b_reduce_kernel(const float* part, T* db, int64_t count, int nchunks) {
-  const int64_t x = (int64_t)blockIdx.x * 256 + threadIdx.x;
+__global__ __launch_bounds__(256) void tri_bwd_b_reduce_kernel(const BwdArgs a, int64_t count) {
+  const int64_t x = (int64_t)blockIdx.x * 256 + threadIdx.x;  // ((bh * N) + j) * N + k
   if (x >= count) return;
-  float acc = part[x];
-  for (int ch = 1; ch < nchunks; ++ch) acc += part[(int64_t)ch * count + x];
-  db[x] = (T)acc;
+  float acc = a.dbpart[x];
+  for (int ch = 1; ch < a.nchunks; ++ch) acc += a.dbpart[(int64_t)ch * count + x];
+  const int k = (int)(x % a.N), j = (int)((x / a.N) % a.N), bh = (int)(x / ((int64_t)a.N * a.N));
+  reinterpret_cast<T*>(a.db)[(bh / a.H) * a.sdb_b + (bh % a.H) * a.sdb_h + j * a.sdb_j + k * a.sdb_k] = (T)acc;
 }
 
 }  // namespace tri

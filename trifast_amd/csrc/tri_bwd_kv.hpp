@@ -326,8 +326,8 @@ __global__ __launch_bounds__(NW * 64, (bwd_kv_min_waves<T, D, R, BJ>())) void tr
   for (int r = 0; r < R; ++r) {
     const int i = i0 + r;
     if (i >= N) continue;
-    T* dkrow = reinterpret_cast<T*>(a.dk) + (((int64_t)bh * N + i) * N + key) * D;
-    T* dvrow = reinterpret_cast<T*>(a.dv) + (((int64_t)bh * N + i) * N + key) * D;
+    T* dkrow = reinterpret_cast<T*>(a.dk) + b * a.sdk.b + h * a.sdk.h + i * a.sdk.i + key * a.sdk.j;
+    T* dvrow = reinterpret_cast<T*>(a.dv) + b * a.sdv.b + h * a.sdv.h + i * a.sdv.i + key * a.sdv.j;
     store_rows<T, D, DM>(dkrow, dkacc[r], a.scale, g);
     store_rows<T, D, DM>(dvrow, dvacc[r], 1.0f, g);
   }

@@ -312,7 +312,7 @@ __global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(co
   for (int r = 0; r < R; ++r) {
     const int i = i0 + r;
     if (i >= N) continue;
-    T* dqrow = reinterpret_cast<T*>(a.dq) + (((int64_t)bh * N + i) * N + j) * D;
+    T* dqrow = reinterpret_cast<T*>(a.dq) + b * a.sdq.b + h * a.sdq.h + i * a.sdq.i + j * a.sdq.j;
     store_rows<T, D, DM>(dqrow, dqacc[r], a.scale, g);
   }
 }

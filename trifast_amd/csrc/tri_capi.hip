@@ -177,7 +177,8 @@ int check_common(int64_t b, int64_t h, int64_t n, int64_t d, int dtype) {
   if (b < 1 || h < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive (b=%lld h=%lld n=%lld)", (long long)b, (long long)h, (long long)n);
   if (dtype != TRIFAST_F32 && dtype != TRIFAST_BF16 && dtype != TRIFAST_F16) return fail(TRIFAST_EINVAL, "unknown dtype code %d", dtype);
   if (!tri::head_dim_ok((int)d)) return fail(TRIFAST_EUNSUPPORTED, "head dim %lld is not one of the compiled ones (16, 32, 64, 128)", (long long)d);
-  if (n > 65535 || b * h > 65535) return fail(TRIFAST_EINVAL, "n and b*h must be at most 65535");
+  // (b*h, padded to a multiple of 8, is a grid extent)
+  if (n > 65535 || b * h > 65528) return fail(TRIFAST_EINVAL, "n must be at most 65535 and b*h at most 65528");
   return 0;
 }
 
@@ -193,6 +194,14 @@ int check_qlike(const char* name, const void* p, const int64_t* s, int dtype) {
 }
 
 tri::Str5 str5(const int64_t* s) { return tri::Str5{s[0], s[1], s[2], s[3]}; }
+
+// contiguous [b, h, n, n, d] / [b, h, n, n] element strides, for outputs whose strides are not given
+void contiguous5(int64_t* s, int64_t h, int64_t n, int64_t d) {
+  s[4] = 1; s[3] = d; s[2] = n * d; s[1] = n * n * d; s[0] = h * n * n * d;
+}
+void contiguous4(int64_t* s, int64_t h, int64_t n) {
+  s[3] = 1; s[2] = n; s[1] = n * n; s[0] = h * n * n;
+}
 
 int run_bias_prep(const void* bias, const int64_t* bs, const Workspace& w, bool want_k, int64_t b, int64_t h,
                   int64_t n, int dtype, hipStream_t st) {
@@ -342,6 +351,7 @@ int trifast_fwd(void* o, float* lse, const void* q, const void* k, const void* v
   if ((rc = check_qlike("k", k, k_strides, dtype))) return rc;
   if ((rc = check_qlike("v", v, v_strides, dtype))) return rc;
   if ((reinterpret_cast<uintptr_t>(o) & 15) != 0) return fail(TRIFAST_EALIGN, "o: base pointer is not 16-byte aligned");
+  if ((reinterpret_cast<uintptr_t>(lse) & 3) != 0) return fail(TRIFAST_EALIGN, "lse: base pointer is not 4-byte aligned");
   if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
       workspace_bytes < trifast_fwd_workspace_bytes(b, h, n, d, dtype))
     return fail(TRIFAST_EWORKSPACE, "workspace missing, misaligned or smaller than trifast_fwd_workspace_bytes");
@@ -373,6 +383,8 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
                     const float* lse, int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
                     const int64_t* do_strides, const int64_t* q_strides, const int64_t* k_strides,
                     const int64_t* v_strides, const int64_t* bias_strides, const int64_t* mask_strides,
+                    const int64_t* dq_strides, const int64_t* dk_strides, const int64_t* dv_strides,
+                    const int64_t* db_strides,
                     const int* tiles, void* workspace, int64_t workspace_bytes, void* stream) {
   g_err[0] = 0;
   int rc = check_common(b, h, n, d, dtype);
@@ -383,17 +395,30 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   if ((rc = check_qlike("k", k, k_strides, dtype))) return rc;
   if ((rc = check_qlike("v", v, v_strides, dtype))) return rc;
   if ((reinterpret_cast<uintptr_t>(o) & 15) != 0) return fail(TRIFAST_EALIGN, "o: base pointer is not 16-byte aligned");
-  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
-      workspace_bytes < trifast_bwd_workspace_bytes(b, h, n, d, dtype))
-    return fail(TRIFAST_EWORKSPACE, "workspace missing, misaligned or smaller than trifast_bwd_workspace_bytes");
+  if ((reinterpret_cast<uintptr_t>(lse) & 3) != 0) return fail(TRIFAST_EALIGN, "lse: base pointer is not 4-byte aligned");
   const bool all = which < 0;
   const bool do_q = all || which == TRIFAST_KERNEL_BWD_Q;
   const bool do_kv = all || which == TRIFAST_KERNEL_BWD_KV;
   const bool do_b = all || which == TRIFAST_KERNEL_BWD_B;
   if (!do_q && !do_kv && !do_b) return fail(TRIFAST_EINVAL, "kernel id %d is not a backward kernel", which);
-  if (do_q && (!dq || (reinterpret_cast<uintptr_t>(dq) & 15))) return fail(TRIFAST_EINVAL, "dq: null or misaligned");
-  if (do_kv && (!dk || !dv || (reinterpret_cast<uintptr_t>(dk) & 15) || (reinterpret_cast<uintptr_t>(dv) & 15))) return fail(TRIFAST_EINVAL, "dk/dv: null or misaligned");
-  if (do_b && !db) return fail(TRIFAST_EINVAL, "db: null");
+  // gradients: the caller's strides, or contiguous when none are given
+  int64_t c5[5], c4[4];
+  contiguous5(c5, h, n, d);
+  contiguous4(c4, h, n);
+  if (!dq_strides) dq_strides = c5;
+  if (!dk_strides) dk_strides = c5;
+  if (!dv_strides) dv_strides = c5;
+  if (!db_strides) db_strides = c4;
+  if (do_q && (rc = check_qlike("dq", dq, dq_strides, dtype))) return rc;
+  if (do_kv && (rc = check_qlike("dk", dk, dk_strides, dtype))) return rc;
+  if (do_kv && (rc = check_qlike("dv", dv, dv_strides, dtype))) return rc;
+  if (do_b && !db) return fail(TRIFAST_EINVAL, "db: null pointer");
+  // (db is written with 16-byte stores where its strides allow it)
+  if (do_b && (reinterpret_cast<uintptr_t>(db) & 15) != 0) return fail(TRIFAST_EALIGN, "db: base pointer is not 16-byte aligned");
+
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
+      workspace_bytes < trifast_bwd_workspace_bytes(b, h, n, d, dtype))
+    return fail(TRIFAST_EWORKSPACE, "workspace missing, misaligned or smaller than trifast_bwd_workspace_bytes");
 
   int tq = tiles ? tiles[0] : -1, tkv = tiles ? tiles[1] : -1, tb = tiles ? tiles[2] : -1;
   if (tq < 0) tq = trifast_default_tile(TRIFAST_KERNEL_BWD_Q, n, h, d, dtype);
@@ -421,6 +446,8 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   a.rows_per_chunk = (int)((n + a.nchunks - 1) / a.nchunks);
   a.dq = dq; a.dk = dk; a.dv = dv; a.db = db;
   a.sq = str5(q_strides); a.sk = str5(k_strides); a.sv = str5(v_strides); a.sdo = str5(do_strides);
+  a.sdq = str5(dq_strides); a.sdk = str5(dk_strides); a.sdv = str5(dv_strides);
+  a.sdb_b = db_strides[0]; a.sdb_h = db_strides[1]; a.sdb_j = db_strides[2]; a.sdb_k = db_strides[3];
   a.H = (int)h; a.N = (int)n; a.NP = w.np; a.nwords = w.nwords;
   a.c = (float)(1.4426950408889634 / std::sqrt((double)d));
   a.sqrt_d = (float)std::sqrt((double)d);
@@ -446,11 +473,13 @@ int trifast_bwd(void* dq, void* dk, void* dv, void* db, const void* dout, const 
                 const void* v, const void* bias, const uint8_t* mask, const void* o, const float* lse,
                 int64_t b, int64_t h, int64_t n, int64_t d, int dtype, const int64_t* do_strides,
                 const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
-                const int64_t* bias_strides, const int64_t* mask_strides, const int* tiles,
+                const int64_t* bias_strides, const int64_t* mask_strides,
+                const int64_t* dq_strides, const int64_t* dk_strides, const int64_t* dv_strides,
+                const int64_t* db_strides, const int* tiles,
                 void* workspace, int64_t workspace_bytes, void* stream) {
   return bwd_impl(-1, dq, dk, dv, db, dout, q, k, v, bias, mask, o, lse, b, h, n, d, dtype, do_strides,
-                  q_strides, k_strides, v_strides, bias_strides, mask_strides, tiles, workspace,
-                  workspace_bytes, stream);
+                  q_strides, k_strides, v_strides, bias_strides, mask_strides, dq_strides, dk_strides,
+                  dv_strides, db_strides, tiles, workspace, workspace_bytes, stream);
 }
 
 int trifast_bwd_one(int kernel, void* dq, void* dk, void* dv, void* db, const void* dout, const void* q,
@@ -458,14 +487,16 @@ int trifast_bwd_one(int kernel, void* dq, void* dk, void* dv, void* db, const vo
                     const float* lse, int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
                     const int64_t* do_strides, const int64_t* q_strides, const int64_t* k_strides,
                     const int64_t* v_strides, const int64_t* bias_strides, const int64_t* mask_strides,
+                    const int64_t* dq_strides, const int64_t* dk_strides, const int64_t* dv_strides,
+                    const int64_t* db_strides,
                     int tile, void* workspace, int64_t workspace_bytes, void* stream) {
   if (kernel != TRIFAST_KERNEL_BWD_Q && kernel != TRIFAST_KERNEL_BWD_KV && kernel != TRIFAST_KERNEL_BWD_B)
     return fail(TRIFAST_EINVAL, "kernel id %d is not a backward kernel", kernel);
   int tiles[3] = {-1, -1, -1};
   tiles[kernel - TRIFAST_KERNEL_BWD_Q] = tile;
   return bwd_impl(kernel, dq, dk, dv, db, dout, q, k, v, bias, mask, o, lse, b, h, n, d, dtype, do_strides,
-                  q_strides, k_strides, v_strides, bias_strides, mask_strides, tiles, workspace,
-                  workspace_bytes, stream);
+                  q_strides, k_strides, v_strides, bias_strides, mask_strides, dq_strides, dk_strides,
+                  dv_strides, db_strides, tiles, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -181,16 +181,25 @@ def pick(kernel: int, n: int, h: int, d: int, dtype: torch.dtype, launch: Callab
     from trifast_amd.torch import _DTYPE_CODE
 
     code = _DTYPE_CODE[dtype]
-    if not autotune_enabled() and not force_tune():
+
+    def default() -> int:
         tile = lib.trifast_default_tile(kernel, n, h, d, code)
         _lib.check(min(tile, 0), "trifast_default_tile")
         return tile
+
+    if not autotune_enabled() and not force_tune():
+        return default()
     cache = _cache_for(kernel)
     key = make_key(n, h, d, dtype)
     if key in cache.cache and not force_tune():
         tile = cache.cache[key]
         if lib.trifast_supports(kernel, tile, n, h, d, code):
             return tile
+    # timing synchronises with the device, which a stream capture (HIP graph,
+    # torch.compile's reduce-overhead mode) does not survive: a miss under capture
+    # takes the heuristic pick and leaves the cache alone
+    if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+        return default()
     tiles = supported_tiles(kernel, n, h, d, dtype)
     if not tiles:
         raise ValueError(f"no compiled tile of {cache.name} supports n={n} h={h} d={d} dtype={dtype}")
