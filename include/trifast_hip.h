@@ -104,6 +104,28 @@ int trifast_fwd(void* o, float* lse,
                 int tile, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * Forward without a workspace argument and without any allocation.  No counterpart
+ * in the reference: it is for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * Same arguments and results as trifast_fwd; the keep words, row flags and packed
+ * bias tiles live in a static device array of TRIFAST_STATIC_SCRATCH_BYTES inside
+ * the library (one copy per GPU, held until the process ends).  A shape whose
+ * trifast_fwd_workspace_bytes exceeds that is rejected with TRIFAST_EWORKSPACE
+ * (bf16/fp16: b*h*ceil(n/32)^2 <= 6100 or so, e.g. b=1 h=4 n=1024).  The pre-passes
+ * rewrite every byte the kernel reads, so nothing has to be cleared between calls.
+ * All calls on one GPU share the array: calls that overlap on one GPU (different
+ * streams or threads) race; serialise them on one stream.
+ */
+#define TRIFAST_STATIC_SCRATCH_BYTES (12 * 1024 * 1024)
+int trifast_fwd_static(void* o, float* lse,
+                       const void* q, const void* k, const void* v,
+                       const void* bias, const uint8_t* mask,
+                       int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
+                       const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                       const int64_t* bias_strides, const int64_t* mask_strides,
+                       int tile, void* stream);
+
+/*
  * Backward: dq, dk, dv, db from do and the saved q, k, v, bias, mask, o, lse.
  * Replaces the _bwd_q, _bwd_kv and _bwd_b launches of reference
  * src/trifast/torch.py:111-174 (one call, fixed launch order, deterministic).

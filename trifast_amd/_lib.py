@@ -39,6 +39,13 @@ SIGNATURES = {
          _I64P, _I64P, _I64P, _I64P, _I64P,
          c_int, c_void_p, c_int64, c_void_p],
     ),
+    "trifast_fwd_static": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int64, c_int64, c_int64, c_int64, c_int,
+         _I64P, _I64P, _I64P, _I64P, _I64P,
+         c_int, c_void_p],
+    ),
     "trifast_bwd": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p,

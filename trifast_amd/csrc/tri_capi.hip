@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstring>
 #include <limits>
+#include <mutex>
 
 #include "../../include/trifast_hip.h"
 #include "tri_common.hpp"
@@ -101,6 +102,12 @@ hipError_t bias_prep_launch(const BiasPrepArgs& a, int bh, int dtype, hipStream_
 
 }  // namespace tri
 
+// Scratch of trifast_fwd_static: device memory that lives in the library's code
+// object, one copy per GPU, from load until the process ends.  The array's name is
+// a host-side handle only; kernels and pre-passes get the device address that
+// hipGetSymbolAddress returns for the current device (static_scratch below).
+static __device__ __align__(256) unsigned char scratch[TRIFAST_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -116,6 +123,27 @@ int fail(int code, const char* fmt, ...) {
 int hip_fail(hipError_t e, const char* what) {
   snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(e));
   return (int)e > 0 ? (int)e : 1;
+}
+
+// Device address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices) return fail(TRIFAST_EINVAL, "device %d is beyond the %d devices the static scratch table holds", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
 }
 
 int64_t align256(int64_t x) { return (x + 255) & ~int64_t(255); }
@@ -338,11 +366,13 @@ int64_t trifast_bwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, 
          (chunks > 1 ? align256(chunks * b * h * n * n * 4) : 0);
 }
 
-int trifast_fwd(void* o, float* lse, const void* q, const void* k, const void* v, const void* bias,
-                const uint8_t* mask, int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
-                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
-                const int64_t* bias_strides, const int64_t* mask_strides, int tile, void* workspace,
-                int64_t workspace_bytes, void* stream) {
+// Forward with the workspace either given by the caller or (use_static) taken from the
+// library's own static scratch array.
+static int fwd_impl(bool use_static, void* o, float* lse, const void* q, const void* k, const void* v, const void* bias,
+                    const uint8_t* mask, int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
+                    const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                    const int64_t* bias_strides, const int64_t* mask_strides, int tile, void* workspace,
+                    int64_t workspace_bytes, void* stream) {
   g_err[0] = 0;
   int rc = check_common(b, h, n, d, dtype);
   if (rc) return rc;
@@ -352,6 +382,14 @@ int trifast_fwd(void* o, float* lse, const void* q, const void* k, const void* v
   if ((rc = check_qlike("v", v, v_strides, dtype))) return rc;
   if ((reinterpret_cast<uintptr_t>(o) & 15) != 0) return fail(TRIFAST_EALIGN, "o: base pointer is not 16-byte aligned");
   if ((reinterpret_cast<uintptr_t>(lse) & 3) != 0) return fail(TRIFAST_EALIGN, "lse: base pointer is not 4-byte aligned");
+  if (use_static) {
+    const int64_t need = trifast_fwd_workspace_bytes(b, h, n, d, dtype);
+    if (need > (int64_t)TRIFAST_STATIC_SCRATCH_BYTES)
+      return fail(TRIFAST_EWORKSPACE, "trifast_fwd_static: this shape needs %lld bytes of scratch, the static array holds %lld "
+                  "(use trifast_fwd with a caller-provided workspace)", (long long)need, (long long)TRIFAST_STATIC_SCRATCH_BYTES);
+    if ((rc = static_scratch(&workspace))) return rc;
+    workspace_bytes = TRIFAST_STATIC_SCRATCH_BYTES;
+  }
   if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
       workspace_bytes < trifast_fwd_workspace_bytes(b, h, n, d, dtype))
     return fail(TRIFAST_EWORKSPACE, "workspace missing, misaligned or smaller than trifast_fwd_workspace_bytes");
@@ -376,6 +414,23 @@ int trifast_fwd(void* o, float* lse, const void* q, const void* k, const void* v
   hipError_t e = tri::fwd_launch(a, (int)(b * h), (int)d, dtype, tile, st);
   if (e != hipSuccess) return hip_fail(e, "forward launch");
   return 0;
+}
+
+int trifast_fwd(void* o, float* lse, const void* q, const void* k, const void* v, const void* bias,
+                const uint8_t* mask, int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
+                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                const int64_t* bias_strides, const int64_t* mask_strides, int tile, void* workspace,
+                int64_t workspace_bytes, void* stream) {
+  return fwd_impl(false, o, lse, q, k, v, bias, mask, b, h, n, d, dtype, q_strides, k_strides, v_strides,
+                  bias_strides, mask_strides, tile, workspace, workspace_bytes, stream);
+}
+
+int trifast_fwd_static(void* o, float* lse, const void* q, const void* k, const void* v, const void* bias,
+                       const uint8_t* mask, int64_t b, int64_t h, int64_t n, int64_t d, int dtype,
+                       const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                       const int64_t* bias_strides, const int64_t* mask_strides, int tile, void* stream) {
+  return fwd_impl(true, o, lse, q, k, v, bias, mask, b, h, n, d, dtype, q_strides, k_strides, v_strides,
+                  bias_strides, mask_strides, tile, nullptr, 0, stream);
 }
 
 static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const void* dout, const void* q,
