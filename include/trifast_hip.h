@@ -86,6 +86,15 @@ int trifast_tile_info(int kernel, int tile, int* block_j, int* block_k, int* num
 int trifast_supports(int kernel, int tile, int64_t n, int64_t h, int64_t d, int dtype);
 int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype);
 
+/*
+ * 1 for the tiles of TRIFAST_KERNEL_BWD_KV that keep a whole pair row in one
+ * workgroup and produce dq, dk and dv from one computation of the scores (the
+ * reference runs _bwd_q and _bwd_kv for this, src/trifast/torch.py:111-149): with such
+ * a tile trifast_bwd does not launch the dq kernel, and trifast_bwd_one(BWD_KV) writes
+ * dq as well.  0 for every other tile.
+ */
+int trifast_bwd_kv_tile_writes_dq(int tile);
+
 /* Bytes of caller-provided workspace (256-byte aligned) each call needs. */
 int64_t trifast_fwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype);
 int64_t trifast_bwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype);
@@ -154,6 +163,8 @@ int trifast_bwd(void* dq, void* dk, void* dv, void* db,
  * writes only its own outputs), so a tuner can time them separately.  Order
  * matters exactly as in the reference (src/trifast/torch.py:110): BWD_Q first --
  * it also fills the workspace's delta = rowsum(o * do) that the other two read.
+ * A BWD_KV tile for which trifast_bwd_kv_tile_writes_dq is 1 needs no BWD_Q before
+ * it: it writes dq and fills the workspace itself.
  */
 int trifast_bwd_one(int kernel,
                     void* dq, void* dk, void* dv, void* db,

@@ -108,7 +108,7 @@ def test_every_tile(n, h, d, dtype, monkeypatch):
         tiles = {kern: tile if lib.trifast_supports(kern, tile, n, h, d, code) else None for kern in range(4)}
         if all(t is None for t in tiles.values()):
             continue
-        monkeypatch.setattr(tuner, "pick", lambda kern, n_, h_, d_, dt, launch, tiles=tiles: tiles[kern] if tiles[kern] is not None else lib.trifast_default_tile(kern, n_, h_, d_, code))
+        monkeypatch.setattr(tuner, "pick", lambda kern, n_, h_, d_, dt, launch, extra_cost=None, tiles=tiles: tiles[kern] if tiles[kern] is not None else lib.trifast_default_tile(kern, n_, h_, d_, code))
         kern_out = kernel_fwd_bwd(*low, m, do.to(dtype))
         check_all(kern_out, pt, ref, dtype, f"tile {tile} n={n} d={d} {dtype}", directions=False)
         ran += 1

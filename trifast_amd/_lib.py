@@ -30,6 +30,7 @@ SIGNATURES = {
     "trifast_tile_info": (c_int, [c_int, c_int, _INTP, _INTP, _INTP]),
     "trifast_supports": (c_int, [c_int, c_int, c_int64, c_int64, c_int64, c_int]),
     "trifast_default_tile": (c_int, [c_int, c_int64, c_int64, c_int64, c_int]),
+    "trifast_bwd_kv_tile_writes_dq": (c_int, [c_int]),
     "trifast_fwd_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int64, c_int]),
     "trifast_bwd_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int64, c_int]),
     "trifast_fwd": (

@@ -34,22 +34,39 @@ struct BwdKVFamily {
   }
 };
 
+// tile ids: the streaming tiles above, then the row-resident ones (tri_bwd_row.hpp)
+constexpr int kRowKeyTiles[kBwdRowTiles] = {1, 2, 4, 8};
+
+hipError_t row_launch(const BwdArgs& a, int bh, int d, int dtype, int tile, hipStream_t st, bool dry) {
+  switch (dtype) {
+    case kBF16: return bwd_row_launch_bf16(a, bh, d, tile, st, dry);
+    case kF16: return bwd_row_launch_f16(a, bh, d, tile, st, dry);
+  }
+  return hipErrorInvalidConfiguration;  // fp32 rows do not fit
+}
+
 }  // namespace
 
-int bwd_kv_num_tiles() { return BwdKVFamily::kNumTiles; }
+int bwd_kv_num_tiles() { return BwdKVFamily::kNumTiles + kBwdRowTiles; }
+
+bool bwd_kv_tile_writes_dq(int tile) { return tile >= BwdKVFamily::kNumTiles && tile < bwd_kv_num_tiles(); }
 
 TileInfo bwd_kv_tile_info(int tile) {
   // block_j = queries per LDS stage, block_k = keys per workgroup
+  if (bwd_kv_tile_writes_dq(tile)) return TileInfo{32, 128 * kRowKeyTiles[tile - BwdKVFamily::kNumTiles], 4};
   return TileInfo{BwdKVFamily::P(tile, 2), BwdKVFamily::P(tile, 0) * 32, BwdKVFamily::P(tile, 0)};
 }
 
 bool bwd_kv_supports(int tile, int64_t n, int d, int dtype) {
-  if (tile < 0 || tile >= BwdKVFamily::kNumTiles || !head_dim_ok(d) || n < 1) return false;
+  if (tile < 0 || tile >= bwd_kv_num_tiles() || !head_dim_ok(d) || n < 1) return false;
   BwdArgs a{};
+  a.N = (int)n;
+  if (bwd_kv_tile_writes_dq(tile)) return row_launch(a, 1, d, dtype, tile - BwdKVFamily::kNumTiles, nullptr, true) == hipSuccess;
   return dispatch<BwdKVFamily>(a, 1, d, dtype, tile, nullptr, true) == hipSuccess;
 }
 
 hipError_t bwd_kv_launch(const BwdArgs& a, int bh, int d, int dtype, int tile, hipStream_t st) {
+  if (bwd_kv_tile_writes_dq(tile)) return row_launch(a, bh, d, dtype, tile - BwdKVFamily::kNumTiles, st, false);
   return dispatch<BwdKVFamily>(a, bh, d, dtype, tile, st, false);
 }
 

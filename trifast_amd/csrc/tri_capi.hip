@@ -352,6 +352,8 @@ int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype)
   return pick;
 }
 
+int trifast_bwd_kv_tile_writes_dq(int tile) { return tri::bwd_kv_tile_writes_dq(tile) ? 1 : 0; }
+
 int64_t trifast_fwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype) {
   (void)d;
   if (b < 1 || h < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
@@ -452,10 +454,20 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   if ((reinterpret_cast<uintptr_t>(o) & 15) != 0) return fail(TRIFAST_EALIGN, "o: base pointer is not 16-byte aligned");
   if ((reinterpret_cast<uintptr_t>(lse) & 3) != 0) return fail(TRIFAST_EALIGN, "lse: base pointer is not 4-byte aligned");
   const bool all = which < 0;
-  const bool do_q = all || which == TRIFAST_KERNEL_BWD_Q;
+  bool do_q = all || which == TRIFAST_KERNEL_BWD_Q;
   const bool do_kv = all || which == TRIFAST_KERNEL_BWD_KV;
   const bool do_b = all || which == TRIFAST_KERNEL_BWD_B;
   if (!do_q && !do_kv && !do_b) return fail(TRIFAST_EINVAL, "kernel id %d is not a backward kernel", which);
+  int tq = tiles ? tiles[0] : -1, tkv = tiles ? tiles[1] : -1, tb = tiles ? tiles[2] : -1;
+  if (tq < 0) tq = trifast_default_tile(TRIFAST_KERNEL_BWD_Q, n, h, d, dtype);
+  if (tkv < 0) tkv = trifast_default_tile(TRIFAST_KERNEL_BWD_KV, n, h, d, dtype);
+  if (tb < 0) tb = trifast_default_tile(TRIFAST_KERNEL_BWD_B, n, h, d, dtype);
+  if (tq < 0 || tkv < 0 || tb < 0) return TRIFAST_EUNSUPPORTED;
+  // a row-resident dk/dv tile produces dq (and the per-query planes) as well: the dq
+  // kernel is not launched with it, and dq must be given whenever it runs
+  const bool kv_writes_dq = do_kv && tri::bwd_kv_tile_writes_dq(tkv);
+  const bool need_dq = do_q || kv_writes_dq;
+  if (all && kv_writes_dq) do_q = false;
   // gradients: the caller's strides, or contiguous when none are given
   int64_t c5[5], c4[4];
   contiguous5(c5, h, n, d);
@@ -464,7 +476,7 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   if (!dk_strides) dk_strides = c5;
   if (!dv_strides) dv_strides = c5;
   if (!db_strides) db_strides = c4;
-  if (do_q && (rc = check_qlike("dq", dq, dq_strides, dtype))) return rc;
+  if (need_dq && (rc = check_qlike("dq", dq, dq_strides, dtype))) return rc;
   if (do_kv && (rc = check_qlike("dk", dk, dk_strides, dtype))) return rc;
   if (do_kv && (rc = check_qlike("dv", dv, dv_strides, dtype))) return rc;
   if (do_b && !db) return fail(TRIFAST_EINVAL, "db: null pointer");
@@ -475,11 +487,6 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
       workspace_bytes < trifast_bwd_workspace_bytes(b, h, n, d, dtype))
     return fail(TRIFAST_EWORKSPACE, "workspace missing, misaligned or smaller than trifast_bwd_workspace_bytes");
 
-  int tq = tiles ? tiles[0] : -1, tkv = tiles ? tiles[1] : -1, tb = tiles ? tiles[2] : -1;
-  if (tq < 0) tq = trifast_default_tile(TRIFAST_KERNEL_BWD_Q, n, h, d, dtype);
-  if (tkv < 0) tkv = trifast_default_tile(TRIFAST_KERNEL_BWD_KV, n, h, d, dtype);
-  if (tb < 0) tb = trifast_default_tile(TRIFAST_KERNEL_BWD_B, n, h, d, dtype);
-  if (tq < 0 || tkv < 0 || tb < 0) return TRIFAST_EUNSUPPORTED;
   if (do_q && !tri::bwd_q_supports(tq, n, (int)d, dtype)) return fail(TRIFAST_EUNSUPPORTED, "bwd_q tile %d unsupported for this shape", tq);
   if (do_kv && !tri::bwd_kv_supports(tkv, n, (int)d, dtype)) return fail(TRIFAST_EUNSUPPORTED, "bwd_kv tile %d unsupported for this shape", tkv);
   if (do_b && !tri::bwd_b_supports(tb, n, (int)d, dtype)) return fail(TRIFAST_EUNSUPPORTED, "bwd_b tile %d unsupported for this shape", tb);

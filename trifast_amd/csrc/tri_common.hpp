@@ -62,6 +62,22 @@ struct Elem<__bf16> {
   static TRI_DEV f32x16 mfma(frag a, frag b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  // the same with the accumulator held in the accumulation registers (AGPRs): for
+  // long-lived accumulators of kernels that run one wave per SIMD, whose other values
+  // fill the ordinary registers.  Nothing but MFMAs touches `c` between its
+  // initialisation and its final read.  The compiler does not know that the statement
+  // is an MFMA, so the wait states an MFMA needs after a vector-ALU write of one of its
+  // operands (two) are spent inside the statement.
+  static TRI_DEV void mfma_acc(frag a, frag b, f32x16& c) {
+asm("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  // Such an accumulator is zeroed by an MFMA too (0 * 0 + 0): a vector-ALU write to it
+  // right before the first accumulating MFMA is not ordered against that MFMA's read by
+  // anything the compiler knows about an asm statement.
+  static TRI_DEV void mfma_acc_zero(f32x16& c) {
+    const frag z = zero();
+asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %1, 0" : "=a"(c) : "v"(z));  // volatile: one MFMA per accumulator, no copies
+  }
   static TRI_DEV frag splat(float x) {
     frag f;
 #pragma unroll
@@ -88,6 +104,13 @@ struct Elem<_Float16> {
   static constexpr float kMaskElem = -60000.0f;
   static TRI_DEV f32x16 mfma(frag a, frag b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static TRI_DEV void mfma_acc(frag a, frag b, f32x16& c) {
+    asm("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  static TRI_DEV void mfma_acc_zero(f32x16& c) {
+    const frag z = zero();
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %1, 0" : "=a"(c) : "v"(z));
   }
   static TRI_DEV frag splat(float x) {
     frag f;

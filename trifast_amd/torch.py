@@ -209,7 +209,20 @@ def triangle_attention_bwd(
                 primed = True
                 launch_one(kern, t)
 
-            tiles.append(tuner.pick(kernel, n, h, d, q.dtype, timed))
+            # a dk/dv tile that also produces dq saves the dq kernel's launch: the other
+            # dk/dv tiles are charged with it
+            extra = None
+            if kernel == _lib.KERNEL_BWD_KV:
+                dq_ms: list[float] = []
+
+                def extra(t):
+                    if lib.trifast_bwd_kv_tile_writes_dq(t):
+                        return 0.0
+                    if not dq_ms:
+                        dq_ms.append(tuner._time_launch(lambda tile: launch_one(_lib.KERNEL_BWD_Q, tile), tiles[0]))
+                    return dq_ms[0]
+
+            tiles.append(tuner.pick(kernel, n, h, d, q.dtype, timed, extra))
         rc = lib.trifast_bwd(
             _ptr(dq), _ptr(dk), _ptr(dv), _ptr(db),
             _ptr(do), _ptr(q), _ptr(k), _ptr(v), _ptr(b), _ptr(mask_u8), _ptr(o), _ptr(l),

@@ -174,9 +174,12 @@ def _time_launch(launch: Callable[[int], None], tile: int, warmup: int = 1, rep:
     return times[len(times) // 2]
 
 
-def pick(kernel: int, n: int, h: int, d: int, dtype: torch.dtype, launch: Callable[[int], None]) -> int:
+def pick(kernel: int, n: int, h: int, d: int, dtype: torch.dtype, launch: Callable[[int], None],
+         extra_cost: Callable[[int], float] | None = None) -> int:
     """Tile id to run ``kernel`` with.  ``launch(tile)`` runs the kernel once on the
-    caller's real arguments (outputs are overwritten by the caller's final launch)."""
+    caller's real arguments (outputs are overwritten by the caller's final launch).
+    ``extra_cost(tile)`` is added to a tile's measured milliseconds: what the choice of
+    that tile leaves for other kernels to do."""
     lib = _lib.load()
     from trifast_amd.torch import _DTYPE_CODE
 
@@ -207,7 +210,7 @@ def pick(kernel: int, n: int, h: int, d: int, dtype: torch.dtype, launch: Callab
         best = tiles[0]
         cache.timings = {}
     else:
-        cache.timings = {t: _time_launch(launch, t) for t in tiles}
+        cache.timings = {t: _time_launch(launch, t) + (extra_cost(t) if extra_cost else 0.0) for t in tiles}
         best = min(cache.timings, key=cache.timings.get)
         # near-ties go to the library's default tile: timings of a few launches scatter by
         # a percent or two, and a stable choice is worth more than that
