@@ -7,7 +7,7 @@
 namespace tri {
 
 // tile index -> key tiles per wave; a workgroup holds rows of up to 128 * KT keys
-constexpr int kRowKT[kBwdRowTiles] = {1, 2, 4, 8};
+constexpr int kRowKT[kBwdRowTiles] = {2, 4, 6, 8};
 
 template <typename T, int D, int KT>
 hipError_t bwd_row_run(const BwdArgs& a, int bh, hipStream_t st, bool dry) {
