@@ -14,7 +14,7 @@ n=1024, all keys attended.  Prints ONE JSON line:
                attention, forward + autograd backward, on the host cores, on a
                bounded sample of rows of the same workload
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload M|C2|C3|C4a|C4b|C5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload M|C2|C3|C4a|C4b|C5|F32]
 """
 
 from __future__ import annotations
@@ -53,6 +53,8 @@ WORKLOADS = {
     "C4b": (torch.float16, 2, 384, 8, 64, "fp16 b2 n384 h8 d64, transposed views"),
     "C5": (torch.bfloat16, 1, 2048, 4, 32, "bf16 b1 n2048 h4 d32, bias outliers, 5% random mask"),
     "M": (torch.bfloat16, 1, 1024, 4, 32, "bf16 b1 n1024 h4 d32, no mask"),
+    # not one of the reference's configurations: the fp32-MFMA path at a size that fills the GPU
+    "F32": (torch.float32, 1, 512, 4, 32, "fp32 b1 n512 h4 d32, no mask"),
 }
 
 
@@ -167,53 +169,104 @@ def kernel_breakdown(q, k, v, bias, mask, do, reps):
                                  S(dov), S(qv), S(kv), S(vv), S(bv), S(mu8), None, None, None, None, tile, ws.data_ptr(), ws.numel(), stream)
         _lib.check(rc, "trifast_bwd_one")
 
+    # (the tiles the operator itself runs with: its cache is warm after the timed steps)
     for kernel in (_lib.KERNEL_FWD, _lib.KERNEL_BWD_Q, _lib.KERNEL_BWD_KV, _lib.KERNEL_BWD_B):
         launch = fwd if kernel == _lib.KERNEL_FWD else (lambda t, kern=kernel: bwd_one(kern, t))
         tile = tuner.pick(kernel, n, h, d, q.dtype, launch)
         launch(tile)
         torch.cuda.synchronize()
         out[_lib.KERNEL_NAMES[kernel]] = {"ms": _event_ms(lambda: launch(tile), reps), "tile": dict(_lib.tile_info(kernel, tile), id=tile)}
+    # a dk/dv tile that also produces dq replaces the dq kernel: the step does not launch it
+    fused = bool(lib.trifast_bwd_kv_tile_writes_dq(out["_bwd_kv"]["tile"]["id"]))
+    out["_bwd_kv"]["writes_dq"] = fused
+    out["_bwd_q"]["in_step"] = not fused
+    # every timed launch includes the two pre-passes (mask bits, bias re-tiling), which the entry
+    # points do not launch alone: their cost stays inside each figure (about 0.02 ms at n = 1024)
     return out
 
 
-def cpu_baseline(name: str, budget_s: float = 20.0):
-    """Forward + autograd backward of the oracle restatement on the host cores, on the
-    first rows of the same workload (rows are independent; the b*h*n^3 logits of the
-    full job would not fit).  Returns the JSON object for the bench line."""
+def _cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(name: str, tensors, budget_s: float = 20.0):
+    """The oracle restatement on the host cores, on the first pair rows of the workload's own
+    seeded tensors (rows are independent; the b*h*n^3 logits of the full job would not fit in
+    host memory at once, so rows go through in chunks of 8).  Two legs, fp32 and the workload's
+    dtype, each one warm-up plus the median of three repetitions, forward + autograd backward
+    and forward alone.  Returns the JSON object for the bench line."""
     from oracle import triangle_oracle as orc
 
     dtype, b, n, h, d, _ = WORKLOADS[name]
     # the host share of a one-GPU box is 16 cores, whatever the machine reports
     cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or min(os.cpu_count() or 1, 16)
     torch.set_num_threads(cores)
-    g = torch.Generator().manual_seed(1337)
-    rows = min(n, 8)
-    # time a few rows, then size the sample for the budget
-    def run(rows):
-        q, k, v, do = (torch.randn(b, h, rows, n, d, generator=g) * d**-0.5 for _ in range(4))
-        bias = torch.randn(b, h, n, n, generator=g)
-        mask = torch.zeros(b, rows, n, dtype=torch.bool)
+    q, k, v, bias, mask, do = tensors
+    chunk = 8
+
+    def host(rows, dt):
+        qs, ks, vs, dos = (t[:, :, :rows].detach().to("cpu", dt).contiguous() for t in (q, k, v, do))
+        return qs, ks, vs, bias.detach().to("cpu", dt).contiguous(), mask[:, :rows].cpu().contiguous(), dos
+
+    def run(ten, backward):
+        qs, ks, vs, bs, ms, dos = ten
+        rows = qs.shape[2]
         t0 = time.perf_counter()
-        for i0 in range(0, rows, 8):
-            sl = slice(i0, min(rows, i0 + 8))
-            qc, kc, vc = (t[:, :, sl].clone().requires_grad_(True) for t in (q, k, v))
-            bc = bias.clone().requires_grad_(True)
-            orc.attention_reference(qc, kc, vc, bc, mask[:, sl]).backward(do[:, :, sl])
+        for i0 in range(0, rows, chunk):
+            sl = slice(i0, min(rows, i0 + chunk))
+            if backward:
+                qc, kc, vc = (t[:, :, sl].clone().requires_grad_(True) for t in (qs, ks, vs))
+                bc = bs.clone().requires_grad_(True)
+                orc.attention_reference(qc, kc, vc, bc, ms[:, sl]).backward(dos[:, :, sl])
+            else:
+                with torch.no_grad():
+                    orc.attention_reference(qs[:, :, sl], ks[:, :, sl], vs[:, :, sl], bs, ms[:, sl])
         return time.perf_counter() - t0
 
-    run(rows)  # warm-up
-    t_probe = run(rows)
-    sample = int(max(rows, min(n, rows * budget_s / max(t_probe, 1e-6)) // 8 * 8))
-    t = run(sample)
-    fl = sum(flops(b, h, n, d)) * sample / n
-    return {
-        "value": fl / t / 1e12,
+    def leg(dt, budget):
+        probe = host(min(n, chunk), dt)
+        run(probe, True)  # warm-up of the probe
+        t_probe = run(probe, True)
+        # five timed-or-warm passes of fwd+bwd and of fwd (about a third of that) per leg
+        rows = int(max(chunk, min(n, chunk * budget / (5.5 * max(t_probe, 1e-6))) // chunk * chunk))
+        rows = min(rows, n)
+        ten = host(rows, dt)
+        out = {"rows": rows}
+        for key, backward, fl in (("fwd_bwd", True, sum(flops(b, h, n, d))), ("fwd", False, flops(b, h, n, d)[0])):
+            run(ten, backward)  # warm-up
+            t = sorted(run(ten, backward) for _ in range(3))[1]
+            out[key] = {"s": t, "tflops": fl * rows / n / t / 1e12, "full_job_s": t * n / rows}
+        return out
+
+    f32 = leg(torch.float32, budget_s * 0.6)
+    res = {
+        "value": f32["fwd_bwd"]["tflops"],
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"{sample} of {n} pair rows of the same workload, fp32, fwd + autograd bwd in {t:.1f} s "
-                  f"(full job extrapolates to {t * n / sample:.0f} s)",
+        "sample": f"first {f32['rows']} of {n} pair rows of the workload's own seeded tensors in chunks of {chunk}, fp32, "
+                  f"fwd + autograd bwd, 1 warm-up + median of 3: {f32['fwd_bwd']['s']:.2f} s "
+                  f"(full job extrapolates to {f32['fwd_bwd']['full_job_s']:.1f} s)",
+        "fwd_value": f32["fwd"]["tflops"],
+        "fwd_full_job_s": f32["fwd"]["full_job_s"],
+        "cpu_model": _cpu_model(),
+        "os_cpu_count": os.cpu_count(),
     }
+    if dtype != torch.float32:
+        low = leg(dtype, budget_s * 0.4)
+        res["workload_dtype"] = {
+            "dtype": str(dtype).split(".")[-1], "rows": low["rows"],
+            "value": low["fwd_bwd"]["tflops"], "fwd_value": low["fwd"]["tflops"],
+            "full_job_s": low["fwd_bwd"]["full_job_s"],
+        }
+    return res
 
 
 def main():
@@ -288,17 +341,21 @@ def main():
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     peak_at_clock = cus * 4096 * clock_mhz / 1e6 if clock_mhz > 0 else None
 
+    dname = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype]
     f_fwd, f_bwd = flops(b, h, n, d)
     peak = PEAK_F32_TFLOPS if dtype == torch.float32 else PEAK_BF16_TFLOPS
     tf_step = (f_fwd + f_bwd) / ms_step / 1e9
     tf_fwd = f_fwd / ms_fwd / 1e9
 
     kern = kernel_breakdown(q.detach(), k.detach(), v.detach(), bias.detach(), mask, do, max(3, args.steps // 2))
-    # GEMMs each kernel needs for its own outputs (S and dP are recomputed per kernel)
-    gemms = {"_fwd": 2, "_bwd_q": 3, "_bwd_kv": 4, "_bwd_b": 2}
+    # GEMMs each kernel needs for its own outputs (S and dP are recomputed per kernel; the
+    # row-resident dk/dv tile computes them once for dq, dk and dv)
+    gemms = {"_fwd": 2, "_bwd_q": 3, "_bwd_kv": 5 if kern["_bwd_kv"]["writes_dq"] else 4, "_bwd_b": 2}
     for name, rec in kern.items():
         rec["tflops"] = gemms[name] * 2 * b * h * n**3 * d / rec["ms"] / 1e9
-    dom = max(kern, key=lambda key: kern[key]["ms"])
+    in_step = [name for name in kern if kern[name].get("in_step", True)]
+    bwd_ms = sum(kern[name]["ms"] for name in in_step if name != "_fwd")
+    dom = max(in_step, key=lambda key: kern[key]["ms"])
     tile = kern[dom]["tile"]
     mib = MEASURED_TRAFFIC_MIB.get((args.workload, dom, tile["id"]))
     traffic = None if mib is None else mib * 2**20
@@ -315,7 +372,7 @@ def main():
     }
 
     line = {
-        "metric": "fwd+bwd TFLOP/s & % bf16 MFMA peak, bf16 h=4 d=32 n=1024, 1xMI355X",
+        "metric": f"fwd+bwd TFLOP/s & % {dname} MFMA peak, {dname} h={h} d={d} n={n}, 1xMI355X",
         "value": tf_step,
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -325,7 +382,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype],
+        "dtype": dname,
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: {desc}", "b": b, "h": h, "n": n, "d": d},
         "frac_of_peak": tf_step / peak,
@@ -337,12 +394,17 @@ def main():
         "peak_tflops_nominal": peak,
         "max_clock_mhz": clock_mhz,
         "peak_tflops_at_max_clock": None if dtype == torch.float32 else peak_at_clock,
-        "kernels": {name: {"ms": round(rec["ms"], 4), "tflops": round(rec["tflops"], 1), "tile": rec["tile"]} for name, rec in kern.items()},
+        "kernels": {name: {"ms": round(rec["ms"], 4), "tflops": round(rec["tflops"], 1), "tile": rec["tile"],
+                           "in_step": rec.get("in_step", True)} for name, rec in kern.items()},
+        # the backward as a whole, counted as the five GEMMs it needs (10 b h n^3 d) whatever the
+        # kernels recompute, over the launch durations of its kernels
+        "bwd_credited": {"ms": bwd_ms, "tflops": f_bwd / bwd_ms / 1e9, "frac_of_peak": f_bwd / bwd_ms / 1e9 / peak},
+        "kernel_ms_include": "mask and bias pre-passes (and the db partial reduce), about 0.02 ms at n=1024",
         "roofline": roofline,
         "autotune": tuner.autotune_enabled(),
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(args.workload, args.cpu_budget)
+        line["cpu_baseline"] = cpu_baseline(args.workload, (q, k, v, bias, mask, do), args.cpu_budget)
     print(json.dumps(line))
 
 

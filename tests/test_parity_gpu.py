@@ -117,6 +117,41 @@ def test_every_tile(n, h, d, dtype, monkeypatch):
 
 
 # ---------------------------------------------------------------------------
+# the row-resident backward (dq, dk, dv in one pass) at every size class it has:
+# 2, 4, 6 and 8 key tiles per wave, ragged sizes, masked keys, fully masked rows
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("n,h,d", [(131, 2, 32), (300, 1, 32), (520, 1, 32), (700, 1, 32), (1000, 1, 32), (450, 1, 64), (190, 1, 16)])
+def test_row_resident_backward_size_classes(n, h, d, dtype, monkeypatch):
+    lib = _lib.load()
+    code = tt._DTYPE_CODE[dtype]
+    row_tiles = [t for t in range(lib.trifast_num_tiles(_lib.KERNEL_BWD_KV))
+                 if lib.trifast_bwd_kv_tile_writes_dq(t) and lib.trifast_supports(_lib.KERNEL_BWD_KV, t, n, h, d, code)]
+    assert row_tiles, "no row-resident tile supports this shape"
+    tile = row_tiles[0]  # the smallest one that holds the row
+    g = torch.Generator().manual_seed(n + d)
+    q, k, v, b, m = orc.gen_tensors(n, d, h, True, "cpu", torch.float32, 1, 1.0, generator=g)
+    m[:, 3, :] = True          # a fully masked row
+    m[:, 5, : n - 7] = True    # a row that attends to its last keys only (dead key tiles)
+    m[:, 7, :] = False         # a row with no masked key
+    do = torch.randn(q.shape, generator=g)
+    q, k, v, b, m, do = (t.detach().to(DEV) for t in (q, k, v, b, m, do))
+    low = [t.to(dtype) for t in (q, k, v, b)]
+    chunk = 64 if n > 400 else None
+    ref = oracle_fwd_bwd(*(t.float() for t in low), m, do.to(dtype).float(), chunk)
+    pt = oracle_fwd_bwd(*low, m, do.to(dtype), chunk)
+    real_pick = tuner.pick
+    monkeypatch.setattr(tuner, "pick", lambda kern, *a, **kw: tile if kern == _lib.KERNEL_BWD_KV else real_pick(kern, *a, **kw))
+    kern_out = kernel_fwd_bwd(*low, m, do.to(dtype))
+    check_all(kern_out, pt, ref, dtype, f"row-resident tile {tile} n={n} d={d} {dtype}", directions=False)
+    again = kernel_fwd_bwd(*low, m, do.to(dtype))
+    for name, x, y in zip(NAMES, kern_out, again):
+        assert torch.equal(x, y), f"{name} differs between two runs"
+    # masked keys of partially masked rows get exactly zero dk, dv
+    assert kern_out[2][:, :, 5, : n - 7].abs().max() == 0 and kern_out[3][:, :, 5, : n - 7].abs().max() == 0
+
+
+# ---------------------------------------------------------------------------
 # golden fixtures (inputs and answers fixed on disk)
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("name", ["tiny_n6_h2_d16", "plumb_n16_h4_d32", "ragged_n19_h2_d32"])
