@@ -10,18 +10,22 @@
 // queries of the row are streamed through LDS in tiles of 32 (Q, dO rows, direct
 // global->LDS loads, double-buffered).  Per (query tile, key tile), with the
 // scores un-transposed (a lane owns one key and 16 queries):
-//   S  = Q K^T + sqrt(d) (bias - lse)      bias tile -> fp32 once, as accumulator init
+//   S  = Q K^T + sqrt(d) (bias - lse)      every term through the matrix pipe (below)
 //   P  = exp2(c S)
-//   dP = dO V^T - delta                    -delta as accumulator init
+//   dP = dO V^T - delta
 //   dS = P * dP
 //   dv^T += dO^T P,  dk^T += Q^T dS        P, dS are B operands as they are
 //   dq^T += K^T dS^T                       dS goes through a 2 KiB LDS tile of the wave
 //                                          and comes back transposed (ds_read_tr)
-// The per-query terms (-lse sqrt(d), -delta) are the same for every key tile of a
-// query tile: the 16 values a lane needs are loaded once per query tile and enter
-// as accumulator inits, so no rank-1 MFMA and no add is spent on them.  dq of a
-// query tile is the sum of the four waves' partial tiles: they meet in LDS once
-// per query tile and are added in wave order (deterministic, no atomics).
+// A wave alone on its SIMD issues one instruction every four cycles or so, whatever the
+// instruction is, and the matrix pipe has time to spare: so everything that can be said
+// as a matrix product is one.  The packed bias words of a tile are A operands as they
+// are (a lane owns a query and eight keys) against a constant B operand that holds
+// sqrt(d) where the contraction slot is the column's key; -lse sqrt(d) and -delta (per
+// query) and the key mask (per key) are rank-1 products of operand words.  That leaves
+// the vector ALU one multiply and one exp2 per score, one multiply per dS and the two
+// conversions.  dq of a query tile is the sum of the four waves' partial tiles: they
+// meet in LDS once per query tile and are added in wave order (deterministic, no atomics).
 //
 // The prologue also computes delta = rowsum(o * do) of the row and leaves it, with
 // the row's log-sum-exp, in the per-query planes the db kernel reads.
@@ -31,6 +35,7 @@
 // src/trifast/triton.py:274-383 and :143-263 in one pass.
 #pragma once
 #include <type_traits>
+#include <utility>
 
 #include "tri_args.hpp"
 #include "tri_common.hpp"
@@ -40,20 +45,105 @@ namespace tri {
 
 constexpr int kRowWaves = 4;
 
+// ---- the MFMA order of one step of the kernel below ------------------------------------
+enum RowOp { R_SOFF, R_SB, R_SQK, R_DOFF, R_DP, R_ACC, R_DQ };
+struct RowSched {
+  int n;             // MFMAs of the step
+  int kind[48], idx[48];
+  int dq_reads_at;   // the LDS reads for dq follow this MFMA
+  int last_sqk;      // the last MFMA that reads the K rows of the next tile
+  int v_reads_at;    // V operands kept in LDS are read after this MFMA
+  int last_sb;       // the last MFMA that reads bias words (0 without any)
+};
+// Two dependent chains start a tile (scores: per-query offset and key mask, bias parts,
+// q.k; dP: -delta, dO.v) and three finish the one before (dv/dk, dq).  Dependent MFMAs are
+// kept apart: first the head of the score chain alternates with the dv/dk MFMAs, then dq,
+// the q.k part and the dP chain take turns.
+constexpr RowSched make_row_sched(bool has_prev, bool has_next, bool flagged, int nsb, int ds, int nacc, int ndq) {
+  RowSched s{};
+  s.dq_reads_at = -1;
+  s.last_sqk = -1;
+  s.v_reads_at = -1;
+  s.last_sb = 0;
+  int lk[16] = {}, li[16] = {}, ns = 0;
+  if (has_next) {
+    lk[ns] = R_SOFF;
+    li[ns++] = 0;
+    if (!flagged)
+      for (int i = 0; i < nsb; ++i) {
+        lk[ns] = R_SB;
+        li[ns++] = i;
+      }
+  }
+  const int na = has_prev ? nacc : 0;
+  int is = 0, ia = 0;
+  if (is < ns) {
+    if (lk[is] == R_SB) s.last_sb = s.n;
+    s.kind[s.n] = lk[is];
+    s.idx[s.n++] = li[is++];
+  }
+  while (is < ns || ia < na) {
+    if (is < ns) {
+      if (lk[is] == R_SB) s.last_sb = s.n;
+      s.kind[s.n] = lk[is];
+      s.idx[s.n++] = li[is++];
+    }
+    if (ia < na) {
+      s.kind[s.n] = R_ACC;
+      s.idx[s.n++] = ia++;
+    }
+  }
+  const int nq = has_prev ? ndq : 0, nk = (has_next && !flagged) ? ds : 0, np = has_next ? 1 + ds : 0;
+  int iq = 0, ik = 0, ip = 0, first_dq = -1;
+  while (iq < nq || ik < nk || ip < np) {
+    if (iq < nq) {
+      if (first_dq < 0) first_dq = s.n;
+      s.kind[s.n] = R_DQ;
+      s.idx[s.n++] = iq++;
+    }
+    if (ik < nk) {
+      s.last_sqk = s.n;
+      s.kind[s.n] = R_SQK;
+      s.idx[s.n++] = ik++;
+    }
+    if (ip < np) {
+      if (ip == 1) s.v_reads_at = s.n >= 4 ? s.n - 4 : 0;
+      s.kind[s.n] = ip == 0 ? R_DOFF : R_DP;
+      s.idx[s.n++] = ip == 0 ? 0 : ip - 1;
+      ++ip;
+    }
+  }
+  if (first_dq >= 0) s.dq_reads_at = first_dq >= 3 ? first_dq - 3 : 0;
+  return s;
+}
+template <bool HAS_PREV, bool HAS_NEXT, bool FLAGGED, int NSB, int DS, int NACC, int NDQ>
+struct RowSchedOf {
+  static constexpr RowSched value = make_row_sched(HAS_PREV, HAS_NEXT, FLAGGED, NSB, DS, NACC, NDQ);
+};
+
+template <typename F, int... I>
+TRI_DEV void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in order
+template <int N, typename F>
+TRI_DEV void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// Key tiles per wave whose V operands live in LDS instead of registers: the longest rows
+// leave the vector registers no room for all of them (the accumulators fill the other file).
+constexpr int bwd_row_v_lds_tiles(int D, int KT) { return KT * (D / 16) < 16 ? 0 : D <= 32 ? KT - 2 : 1; }
+// dq partial buffers: two (one barrier per query tile) unless the longest rows need the room
+constexpr int bwd_row_red_buffers(int D, int KT) { return D <= 32 && KT * (D / 16) < 16 ? 2 : 1; }
 // LDS bytes of the kernel below
 constexpr int bwd_row_base_lds_bytes(int D, int es, int KT) {
   const int rowb = D * es, dm = (D + 31) / 32, keys = kRowWaves * KT * 32;
-  const int nred = dm == 1 ? 2 : 1;
-  return keys * rowb + 2 * (2 * 32 * rowb) + kRowWaves * 2 * 2048 + nred * kRowWaves * dm * 4096 + 2 * keys * 4;
+  const int nred = bwd_row_red_buffers(D, KT);
+  return keys * rowb + 3 * (2 * 32 * rowb) + kRowWaves * 2048 + nred * kRowWaves * dm * 4096 + 2 * keys * 4 +
+         kRowWaves * bwd_row_v_lds_tiles(D, KT) * (D / 16) * 1024;
 }
-// query tiles per half of the dq staging buffer: what is left of the 160 KiB, at most 8
-constexpr int bwd_row_dq_half(int D, int es, int KT) {
-  const int left = (160 * 1024 - bwd_row_base_lds_bytes(D, es, KT)) / (2 * 32 * D * es);
-  return left > 8 ? 8 : left;
-}
-constexpr int bwd_row_lds_bytes(int D, int es, int KT) {
-  return bwd_row_base_lds_bytes(D, es, KT) + 2 * bwd_row_dq_half(D, es, KT) * 32 * D * es;
-}
+constexpr int bwd_row_lds_bytes(int D, int es, int KT) { return bwd_row_base_lds_bytes(D, es, KT); }
 
 template <typename T, int D, int KT>
 __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const BwdArgs a) {
@@ -69,21 +159,20 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   constexpr int PS = 2;
   constexpr int ROWB = Tile::ROWB;
   constexpr int KEYS = NWV * KT * 32;         // keys (and queries) the workgroup can hold
-  constexpr int NRED = DM == 1 ? 2 : 1;       // dq partial buffers (two: one barrier per query tile)
+  constexpr int NRED = bwd_row_red_buffers(D, KT);  // dq partial buffers
   constexpr int STAGE = 2 * 32 * ROWB;        // Q tile | dO tile
   constexpr int OFF_K = 0;
   constexpr int OFF_ST = KEYS * ROWB;
-  constexpr int OFF_DS = OFF_ST + 2 * STAGE;
-  constexpr int OFF_RED = OFF_DS + NWV * 2 * 2048;
+  constexpr int OFF_DS = OFF_ST + 3 * STAGE;  // three stages: in use, ready, in flight
+  constexpr int OFF_RED = OFF_DS + NWV * 2048;
   constexpr int OFF_NL = OFF_RED + NRED * NWV * DM * 4096;
   constexpr int OFF_ND = OFF_NL + KEYS * 4;
-  // finished dq rows wait here in two halves of DQH query tiles each and leave in bursts of
-  // whole rows: stores inside the tile loop would make every wait for a load a wait for
-  // all memory traffic in flight (loads and stores retire out of order with each other)
-  constexpr int DQH = bwd_row_dq_half(D, (int)sizeof(T), KT);
-  static_assert(DQH >= 1, "no room for the dq staging buffer");
-  constexpr int OFF_DQ = OFF_ND + KEYS * 4;
-  static_assert(OFF_DQ + 2 * DQH * 32 * ROWB == bwd_row_lds_bytes(D, (int)sizeof(T), KT), "the launcher sizes LDS with bwd_row_lds_bytes");
+  constexpr int G2W = (2 * 32 * (ROWB / 16) / 64 + NWV - 1) / NWV;  // global->LDS loads per wave and stage
+  constexpr int VL = bwd_row_v_lds_tiles(D, KT);  // this wave's last VL key tiles keep V in LDS
+  constexpr int VR = KT - VL;
+  constexpr int OFF_V = OFF_ND + KEYS * 4;
+  static_assert(OFF_V + NWV * VL * DS * 1024 == bwd_row_lds_bytes(D, (int)sizeof(T), KT), "the launcher sizes LDS with bwd_row_lds_bytes");
+  static_assert(bwd_row_lds_bytes(D, (int)sizeof(T), KT) <= 160 * 1024, "LDS of one compute unit");
   static_assert((KT - 1) * NWV * 32 * ROWB + 32 * ROWB <= 65536, "key tile offsets are LDS immediates");
   extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
 
@@ -109,11 +198,11 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   const T* krow = reinterpret_cast<const T*>(a.k) + b * a.sk.b + h * a.sk.h + i * a.sk.i;
   const T* vrow = reinterpret_cast<const T*>(a.v) + b * a.sv.b + h * a.sv.h + i * a.sv.i;
   const T* dorow = reinterpret_cast<const T*>(a.dout) + b * a.sdo.b + h * a.sdo.h + i * a.sdo.i;
-  const T* pack_bh = reinterpret_cast<const T*>(a.packk) + (int64_t)bh * a.NP * a.NP * 1024;
+  const T* pack_bh = reinterpret_cast<const T*>(a.packq) + (int64_t)bh * a.NP * a.NP * 1024;
 
   unsigned char* const lds_k = tri_smem + OFF_K;
-  float* const nl = reinterpret_cast<float*>(tri_smem + OFF_NL);
-  float* const nd = reinterpret_cast<float*>(tri_smem + OFF_ND);
+  uint32_t* const nl = reinterpret_cast<uint32_t*>(tri_smem + OFF_NL);  // operand words, see split_word
+  uint32_t* const nd = reinterpret_cast<uint32_t*>(tri_smem + OFF_ND);
 
   // ---- prologue -----------------------------------------------------------------
   // K row -> LDS (rows past the end repeat the last key; their keep bits are clear)
@@ -121,23 +210,40 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   // query tiles 0 (and 1) -> the two stage buffers
   // (per-lane source pointers for query tile 0, computed once; a tile inside the row adds
   // one uniform offset, the ragged last one clamps the query index)
+  // The loads are written as asm: the compiler makes every LDS read that follows a
+  // global->LDS load it knows of wait for that load (the read might be of the bytes in
+  // flight), which would turn the prefetch of the next query tile into a stall at the next
+  // operand read.  Here the stage in flight is not read before the wait and barrier that end
+  // the query tile.  The compiler's own waits stay correct: loads return in issue order, and
+  // a load it does not know of only makes the counter it waits on larger.  (The source
+  // addresses are rebuilt from the lane id every time: kept in registers from one query tile
+  // to the next they would be spilled, and a reload from scratch waits for every load in flight.)
   auto issue_stage = [&](int jt, int buf) {
     unsigned char* st = tri_smem + OFF_ST + buf * STAGE;
-    if (32 * jt + 32 <= N) {
-      // (the source addresses are rebuilt from the lane id every time: kept in registers
-      // from one query tile to the next they would be spilled, and a reload from scratch
-      // waits for every load in flight)
-      int lane_now = lane;
-      asm volatile("" : "+v"(lane_now));  // (opaque: nothing derived from it is hoisted out of the loop)
-      Tile::template fill<32, NWV>(st, [&](int r) { return qrow + (int64_t)(32 * jt + r) * a.sq.j; }, wave, lane_now);
-      Tile::template fill<32, NWV>(st + 32 * ROWB, [&](int r) { return dorow + (int64_t)(32 * jt + r) * a.sdo.j; }, wave, lane_now);
-    } else {
-      asm volatile("" ::);  // keeps this rare path a real branch
-      Tile::template fill<32, NWV>(st, [&](int r) { return qrow + (int64_t)min(32 * jt + r, N - 1) * a.sq.j; }, wave, lane);
-      Tile::template fill<32, NWV>(st + 32 * ROWB, [&](int r) { return dorow + (int64_t)min(32 * jt + r, N - 1) * a.sdo.j; }, wave, lane);
+    int lane_now = lane;
+    asm volatile("" : "+v"(lane_now));  // (opaque: nothing derived from it is hoisted out of the loop)
+    // the stage is one 64-row tile (Q rows, then dO rows) of G2 wave loads of 1 KiB; every
+    // wave issues the same number of them (with fewer loads than waves some are issued twice)
+    constexpr int G2 = 2 * 32 * Tile::CPR / 64;
+    const int jrow = 32 * jt;
+#pragma unroll
+    for (int x = 0; x < (G2 + NWV - 1) / NWV; ++x) {
+      const int gi = (x * NWV + wave) % G2;
+      const bool is_q = gi < G2 / 2;  // wave-uniform
+      const T* rows = is_q ? qrow : dorow;
+      const int64_t stride = is_q ? a.sq.j : a.sdo.j;
+      const int p = gi * 64 + lane_now;
+      const int r = p / Tile::CPR, cc = (p % Tile::CPR) ^ Tile::swz(r);
+      // a 64-bit base per tile (scalar registers) and a 32-bit byte offset per lane; rows past
+      // the end of the pair row (last tile only) read the last row again
+      const T* base = rows + (int64_t)jrow * stride;
+      const uint32_t voff = (uint32_t)(min(r & 31, N - 1 - jrow) * (int)stride + cc * Tile::VEC) * (uint32_t)sizeof(T);
+      const uint32_t dst = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(TRI_L3 unsigned char*)(st + gi * 1024));
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(voff), "s"(base) : "memory", "m0");
     }
   };
   issue_stage(0, 0);
+  issue_stage(min(1, NJ - 1), 1);
 
   // a fully masked row drops q.k and the bias from its scores (all logits equal)
   const bool flagged = __builtin_amdgcn_readfirstlane(a.rowflag[(int64_t)b * N + i]) != 0;
@@ -150,17 +256,23 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   }
   const uint32_t lanebit = 1u << kl;
 
-  // V rows of this lane's keys as B operands
-  frag vf[KT][DS];
+  // V rows of this lane's keys as B operands: in registers for the wave's first VR key
+  // tiles, in a private piece of LDS (operand by operand, 16 bytes per lane) for the rest
+  frag vf[VR > 0 ? VR : 1][DS];
+  frag* const v_lds = reinterpret_cast<frag*>(tri_smem + OFF_V + wave * VL * DS * 1024) + lane;
 #pragma unroll
   for (int t = 0; t < KT; ++t) {
     const int key = min(32 * (NWV * t + wave) + kl, N - 1);
 #pragma unroll
-    for (int s = 0; s < DS; ++s) vf[t][s] = *reinterpret_cast<const frag*>(vrow + (int64_t)key * a.sv.j + 2 * KP * s + KP * g);
+    for (int s = 0; s < DS; ++s) {
+      const frag x = *reinterpret_cast<const frag*>(vrow + (int64_t)key * a.sv.j + 2 * KP * s + KP * g);
+      if (t < VR) vf[t][s] = x;
+      else v_lds[((t - VR) * DS + s) * 64] = x;
+    }
   }
 
   // per-query terms of the row: -delta and -lse*sqrt(d) (ln n for lse in a fully masked
-  // row), kept in LDS for this kernel and written as MFMA operand words for the db kernel
+  // row) as MFMA operand words, kept in LDS for this kernel and written for the db kernel
   {
     const T* orow = reinterpret_cast<const T*>(a.o) + ((int64_t)bh * N + i) * N * D;
     const float* lserow = a.lse + ((int64_t)bh * N + i) * N;
@@ -168,7 +280,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
     uint32_t* lplane = a.lse2 + ((int64_t)bh * N + i) * N;
     const float flat = -__builtin_amdgcn_logf((float)N) * (kLn2 * a.sqrt_d);
     for (int j = tid; j < KEYS; j += NWV * 64) {
-      float nlv = kNeg, ndv = 0.f;  // queries past the end: P = dS = 0
+      float nlv = E::kMaskElem, ndv = 0.f;  // queries past the end: P = dS = 0
       if (j < N) {
         float dsum = 0.f;
 #pragma unroll
@@ -180,11 +292,14 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
         }
         ndv = -dsum;
         nlv = flagged ? flat : -lserow[j] * a.sqrt_d;
-        dplane[j] = split_word<T>(ndv);
-        lplane[j] = split_word<T>(nlv);
       }
-      nl[j] = nlv;
-      nd[j] = ndv;
+      const uint32_t lw = split_word<T>(nlv), dw = split_word<T>(ndv);
+      if (j < N) {
+        dplane[j] = dw;
+        lplane[j] = lw;
+      }
+      nl[j] = lw;
+      nd[j] = dw;
     }
   }
 
@@ -197,61 +312,97 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   ofk.shift(wave * 32 * ROWB);  // key tile t of this wave starts (4 t + wave) * 32 rows into K
   OperandOffsets<T, 32> ofd;
   ofd.init(0, lane);
-  unsigned char* const ds_tile = tri_smem + OFF_DS + wave * 2 * 2048;  // two tiles, used in turn
+  // (one tile: the wave reads dS of a key tile back before it writes the next one)
+  unsigned char* const ds_tile = tri_smem + OFF_DS + wave * 2048;
   const int ds_w0 = DsTile::off(kl, 16 * g), ds_w1 = DsTile::off(kl, 32 + 16 * g);
 
 
   // packed bias tiles of this lane: tile (jt, kt) is 2 x 16 bytes per lane
   typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
-  const T* bias_lane = pack_bh + lane * 8;
+  // (as A operand: operand row m stands for query perm32(m), like the Q and dO operands)
+  const T* bias_lane = pack_bh + (perm32(kl) + 32 * g) * 8;
   auto bias_load = [&](int jt, int t, u32x4v* dst) {
     const int kt = min(NWV * t + wave, a.NP - 1);
+#ifdef TRI_ABL_BIAS0
+    const T* p = bias_lane + (int64_t)(kt & 1) * 1024 + 0 * jt;
+#else
     const T* p = bias_lane + ((int64_t)min(jt, a.NP - 1) * a.NP + kt) * 1024;
+#endif
     dst[0] = *reinterpret_cast<const u32x4v*>(p);
     dst[1] = *reinterpret_cast<const u32x4v*>(p + 512);
   };
   const float c = a.c;
-  const float a_sqrt_d = a.sqrt_d;
+
+  // sqrt(d) * bias through the matrix pipe.  Half r of a packed bias tile gives a lane
+  // (query, g) the keys 16 r + 8 g + 0..7 as its contraction slots; the constant B operand
+  // of half r holds sqrt(d) in the slot that stands for the lane's own key (column) and
+  // zero elsewhere.  sqrt(32) is not a 16-bit number: it goes in as hi + lo, one MFMA each.
+#ifdef TRI_ABL_HIONLY
+  constexpr int NPART = 1;
+#else
+  constexpr int NPART = D == 32 ? 2 : 1;
+#endif
+  constexpr int NSB = 2 * NPART;
+  frag bsel[2][NPART];
+  {
+    const T hi = (T)a.sqrt_d;
+    const T part[2] = {hi, (T)(a.sqrt_d - (float)hi)};
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+      for (int pp = 0; pp < NPART; ++pp) {
+        const int e = kl - 16 * r - 8 * g;
+        const uint32_t bits = (uint32_t)__builtin_bit_cast(uint16_t, part[pp]) << (16 * (e & 1));
+        u32x4v w;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) w[x] = (e >= 0 && e < 8 && (e >> 1) == x) ? bits : 0u;
+        asm volatile("" : "+v"(w));  // resident: not rebuilt from the lane id at every use
+        bsel[r][pp] = __builtin_bit_cast(frag, w);
+      }
+  }
+  // rank-1 operands: per-query words (A side) and the ones / key-mask operand (B side)
+  typename OffsetMask<T>::Queries s_off;
+  s_off.init(0u, g);
+  Rank1<T> d_off;
+  d_off.init();
+  typename OffsetMask<T>::Keys keys_op;
+  keys_op.init(kl, g);
 
   // dq partial tiles of the four waves: [buffer][wave][mt][quarter][lane] x 16 bytes
-  auto red_slot = [&](int buf, int w, int mt, int q) -> f32x4* {
-    return reinterpret_cast<f32x4*>(tri_smem + OFF_RED + (((buf * NWV + w) * DM + mt) * 4 + q) * 1024) + lane;
+  auto red_slot = [&](int buf, int w, int mt, int q, int ln) -> f32x4* {
+    return reinterpret_cast<f32x4*>(tri_smem + OFF_RED + (((buf * NWV + w) * DM + mt) * 4 + q) * 1024) + ln;
   };
-  // sum the partials of query tile jt in wave order; this wave owns quarter `wave` of
-  // every lane's values: head-dim elements 32 mt + 8 wave + 4 g + 0..3 of query 32 jt + kl
-  // (the finished elements go to the dq staging buffer: row-major rows of D elements, query
-  // tile jt in slot jt % (2 DQH))
+  // sum the partials of query tile jt in wave order and store the finished elements; this
+  // wave owns quarter `wave` of every lane's values: head-dim elements 32 mt + 8 wave + 4 g
+  // + 0..3 of query 32 jt + kl, 8 bytes per lane (the four waves' stores complete the rows).
+  // The store is written as asm: a store the compiler knows of makes its waits for loads
+  // waits for everything in flight (stores and loads retire out of order with each other).
+  // Addresses are rebuilt from the lane id at every use: kept in registers across the
+  // key-tile steps they would be spilled, and a reload from scratch waits for every load
+  // in flight.
   T* dqrow = reinterpret_cast<T*>(a.dq) + b * a.sdq.b + h * a.sdq.h + i * a.sdq.i;
   auto reduce_dq = [&](int jt, int buf) {
-    T* slot = reinterpret_cast<T*>(tri_smem + OFF_DQ) + ((jt % (2 * DQH)) * 32 + kl) * D;
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const int j = 32 * jt + (ln & 31);
 #pragma unroll
     for (int mt = 0; mt < DM; ++mt) {
-      const int d0 = 32 * mt + 8 * wave + 4 * g;
-      f32x4 acc = *red_slot(buf, 0, mt, wave);
+      const int d0 = 32 * mt + 8 * wave + 4 * (ln >> 5);
+      f32x4 acc = *red_slot(buf, 0, mt, wave, ln);
 #pragma unroll
-      for (int w = 1; w < NWV; ++w) acc += *red_slot(buf, w, mt, wave);
-      if (d0 < D) {
-        typename E::vec4 ov;
+      for (int w = 1; w < NWV; ++w) acc += *red_slot(buf, w, mt, wave, ln);
+      typename E::vec4 ov;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) ov[e] = (T)(acc[e] * a.scale);
-        *reinterpret_cast<typename E::vec4*>(slot + d0) = ov;
+      for (int e = 0; e < 4; ++e) ov[e] = (T)(acc[e] * a.scale);
+      if (d0 < D && j < N) {
+        typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
+        T* dst = dqrow + (int64_t)j * a.sdq.j + d0;
+        asm volatile("global_store_dwordx2 %0, %1, off" : : "v"(dst), "v"(__builtin_bit_cast(u32x2v, ov)) : "memory");
       }
     }
   };
-  // write query tiles [jt0, jt1) of the staging buffer to dq: whole rows, 16 bytes per lane
-  auto flush_dq = [&](int jt0, int jt1) {
-    constexpr int CPR = Tile::CPR;
-    const int chunks = (jt1 - jt0) * 32 * CPR;
-    for (int cidx_ = tid; cidx_ < chunks; cidx_ += NWV * 64) {
-      const int row = cidx_ / CPR, col = cidx_ % CPR;
-      const int j = 32 * jt0 + row;
-      if (j >= N) break;
-      const T* src = reinterpret_cast<const T*>(tri_smem + OFF_DQ) + ((j % (2 * DQH * 32)) * D + col * Tile::VEC);
-      *reinterpret_cast<typename E::vec*>(dqrow + (int64_t)j * a.sdq.j + col * Tile::VEC) = *reinterpret_cast<const typename E::vec*>(src);
-    }
-  };
 
-  wait_dma();
+  wait_dma_known();
   __syncthreads();
 
   // ---- query tiles ------------------------------------------------------------------
@@ -284,9 +435,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
     // fetched two steps before its use (global memory, through L2)
     u32x4v bias_ring[2][2] = {};
     auto fetch_bias = [&](int jt, int t) {
-#ifndef TRI_ABL_NOBIAS
-      bias_load(jt + t / KT, t % KT, bias_ring[t % 2]);
-#endif
+      if constexpr (!FLAGGED) bias_load(jt + t / KT, t % KT, bias_ring[t % 2]);
     };
     fetch_bias(0, 0);
     fetch_bias(0, 1);
@@ -298,44 +447,31 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
 #else
 #define TRI_TS(k)
 #endif
+    int buf = 0;  // jt % 3: the stage of this query tile
     for (int jt = 0; jt < NJ; ++jt) {
-      const int buf = jt & 1;
-      if (jt + 1 < NJ) issue_stage(jt + 1, buf ^ 1);
-      // the half of the staging buffer whose last query tile was reduced one iteration
-      // ago (and published by the barrier since) leaves now
-      if (jt >= DQH + 1 && (jt - 1) % DQH == 0) {
-        asm volatile("" ::);  // a real branch: taken once in DQH iterations
-        flush_dq(jt - 1 - DQH, jt - 1);
-      }
+      const int buf_fill = buf == 0 ? 2 : buf - 1;  // (jt + 2) % 3: the stage to refill
       if (jt > 0) {
         if constexpr (NRED == 2) reduce_dq(jt - 1, (jt - 1) & 1);
       }
       const unsigned char* qt = tri_smem + OFF_ST + buf * STAGE;
       const unsigned char* dot = qt + 32 * ROWB;
 
-      // the 16 queries of this lane's values: 8 g + 0..7 and 16 + 8 g + 0..7 of the tile
-      f32x16 nlse, ndelta;
-#pragma unroll
-      for (int r = 0; r < 2; ++r)
-#pragma unroll
-        for (int q4 = 0; q4 < 2; ++q4) {
-          const f32x4 x = *reinterpret_cast<const f32x4*>(nl + 32 * jt + 16 * r + 8 * g + 4 * q4);
-          const f32x4 y = *reinterpret_cast<const f32x4*>(nd + 32 * jt + 16 * r + 8 * g + 4 * q4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            nlse[8 * r + 4 * q4 + e] = x[e];
-            ndelta[8 * r + 4 * q4 + e] = y[e];
-          }
-        }
+      // operand words of this lane's query (lanes 32..63 carry zeros)
+      {
+        const uint32_t lw = nl[32 * jt + perm32(kl)], dw = nd[32 * jt + perm32(kl)];
+        s_off.set_raw(g ? 0u : lw);
+        d_off.v[0] = g ? 0u : dw;
+      }
       frag qn[DS], don[DS];
 #pragma unroll
       for (int s = 0; s < DS; ++s) {
         if constexpr (!FLAGGED) qn[s] = ofq.natural(qt, s);
         don[s] = ofq.natural(dot, s);
       }
-      // Q^T, dO^T (A operands of dk, dv) are read again for every key tile, right before
-      // the step that uses them: held for the whole query tile they would be 8 DM registers
-      // too many at the point where most values are live
+      // Q^T, dO^T (A operands of dk, dv): transposing reads are the slowest LDS reads and the
+      // four waves share one LDS pipe, so they are read once per query tile where registers
+      // allow and again for every key tile where they do not
+      constexpr bool QD_ONCE = D <= 32;
       frag qtr[DM][PS], dotr[DM][PS];
       auto load_qd_tr = [&] {
 #pragma unroll
@@ -349,195 +485,139 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
       f32x16 dqacc[DM];
 #pragma unroll
       for (int mt = 0; mt < DM; ++mt) dqacc[mt] = zero16();
+
+      // ---- the state that moves from step to step --------------------------------------
+      f32x16 s_cur, p_cur;   // scores and dP of the tile whose P, dS the step computes
+      f32x16 s_nxt, p_nxt;   // ... of the tile after it, accumulating
+      float p[16], ds[16];
+      frag kn[DS];           // K rows of the next tile as B operand
+      frag pf[PS], dsf[PS];  // P and dS of the last finished tile as B operands
+      frag dst_prev[PS], ktr_prev[DM][PS];
+      frag vn[DS];           // V operands of the next tile when they live in LDS
+      auto load_kn = [&](int t) {
+        if constexpr (!FLAGGED) {
+          const unsigned char* ktile = lds_k + NWV * t * 32 * ROWB;
+#pragma unroll
+          for (int s = 0; s < DS; ++s) kn[s] = ofk.natural(ktile, s);
+        }
+      };
+      load_kn(0);
+      if constexpr (QD_ONCE) load_qd_tr();
       TRI_TS(0)
 
-      // ---- the pieces of one key tile's work -------------------------------------------
-      // quarter a of the score accumulator init of a tile: sqrt(d) * bias - lse * sqrt(d)
-      // (a large negative bias for masked keys and keys past the end); 8 vector instructions
-      auto init_quarter = [&](int a, int t, f32x16& sc) {
-        if constexpr (FLAGGED) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) sc[4 * a + e] = nlse[4 * a + e];  // all logits of the row are equal
-        } else {
-          uint32_t w[2] = {bias_ring[t % 2][a / 2][2 * (a % 2)], bias_ring[t % 2][a / 2][2 * (a % 2) + 1]};
-          if constexpr (MASKED) {
-            const bool kept = (kw[t] & lanebit) != 0;
-            constexpr uint32_t kMaskPair = (std::is_same<T, __bf16>::value ? 0xf149u : 0xf0e2u) * 0x10001u;  // two bf16 of -1e30 / fp16 of -10000
-            w[0] = kept ? w[0] : kMaskPair;
-            w[1] = kept ? w[1] : kMaskPair;
-          }
-          typedef T pair_t __attribute__((ext_vector_type(2)));
-#pragma unroll
-          for (int x = 0; x < 2; ++x) {
-            const pair_t pr = __builtin_bit_cast(pair_t, w[x]);
-            sc[4 * a + 2 * x] = __builtin_fmaf((float)pr[0], a_sqrt_d, nlse[4 * a + 2 * x]);
-            sc[4 * a + 2 * x + 1] = __builtin_fmaf((float)pr[1], a_sqrt_d, nlse[4 * a + 2 * x + 1]);
-          }
-        }
-      };
-      float p[16], ds[16];
-      // quarter bq of P = exp2(c * scores); 8 vector instructions
-      auto p_quarter = [&](int bq, int t, const f32x16& sc) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-#ifdef TRI_ABL_NOEXP
-          p[4 * bq + e] = sc[4 * bq + e] * c;
-#else
-          p[4 * bq + e] = fast_exp2(sc[4 * bq + e] * c);
+      // Step t (t = -1 .. KT): the vector work of tile t (P, dS, their conversions) between
+      // the MFMAs of its neighbours: dv, dk and dq of tile t-1, scores and dP of tile t+1,
+      // in the order of RowSched.  Step -1 only starts tile 0, step KT only finishes tile KT-1.
+      auto step = [&](auto tc) __attribute__((always_inline)) {
+        constexpr int t = decltype(tc)::value - 1;
+        constexpr bool has_prev = t >= 1, has_next = t + 1 < KT, valu = t >= 0 && t < KT;
+        constexpr int tn = has_next ? t + 1 : 0, tp = has_prev ? t - 1 : 0;
+        using Sch = RowSchedOf<has_prev, has_next, FLAGGED, NSB, DS, NACC, NDQ>;
+        constexpr int NM = Sch::value.n;
+        constexpr int NU = valu ? 16 : 0;  // vector units of four instructions
+        // Step KT-2 starts the query tile after next on its way to LDS, right after its last
+        // read of bias words: loads return in issue order,
+        // so the next wait for bias words is a wait for these loads too, and from there it is
+        // the furthest away, at the start of the next query tile.
+        constexpr bool refill = t == KT - 2;
+        constexpr int refill_at = FLAGGED ? 0 : Sch::value.last_sb;
+        SB();
+        if constexpr (valu && !refill) fetch_bias(jt, t + 2);
+        frag kb = keys_op.plain();
+        if constexpr (has_next && MASKED) kb = keys_op.masked(kw[tn]);
+        SB();
+        static_for<NM>([&](auto xc) __attribute__((always_inline)) {
+          constexpr int x = decltype(xc)::value;
+          constexpr int kind = Sch::value.kind[x], idx = Sch::value.idx[x];
+          if constexpr (kind == R_SOFF) {
+            s_nxt = E::mfma(s_off.get(), kb, zero16());
+          } else if constexpr (kind == R_SB) {
+#ifndef TRI_ABL_NOSB
+            s_nxt = E::mfma(__builtin_bit_cast(frag, bias_ring[tn % 2][idx / NPART]), bsel[idx / NPART][idx % NPART], s_nxt);
 #endif
-        }
-        if constexpr (FLAGGED) {
-          // keys past the end of the row stay out of a fully masked row too
-          const bool kept = (kw[t] & lanebit) != 0;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) p[4 * bq + e] = kept ? p[4 * bq + e] : 0.f;
-        }
-      };
-      // half cq of dS = P * (dP - delta); 8 vector instructions
-      auto ds_half = [&](int cq, const f32x16& dp) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) ds[8 * cq + e] = p[8 * cq + e] * dp[8 * cq + e];
-      };
-      frag kn[DS];       // K rows of the next tile as B operand
-      frag pf[PS], dsf[PS];  // P and dS of the last finished tile as B operands
-      auto load_kn = [&](int t) {
-        const unsigned char* ktile = lds_k + NWV * t * 32 * ROWB;
-#pragma unroll
-        for (int s = 0; s < DS; ++s) kn[s] = ofk.natural(ktile, s);
-      };
-      // dv, dk MFMA number x of tile t (x = 2 (s2 DM + mt) + {0: dv, 1: dk})
-      auto acc_mfma = [&](int t, int x) {
-        const int s2 = (x / 2) / DM, mt = (x / 2) % DM;
+          } else if constexpr (kind == R_SQK) {
+            s_nxt = E::mfma(qn[idx], kn[idx], s_nxt);
+          } else if constexpr (kind == R_DOFF) {
+            p_nxt = E::mfma(__builtin_bit_cast(frag, d_off.v), kb, zero16());
+          } else if constexpr (kind == R_DP) {
+            if constexpr (tn < VR) p_nxt = E::mfma(don[idx], vf[tn][idx], p_nxt);
+            else p_nxt = E::mfma(don[idx], vn[idx], p_nxt);
+          } else if constexpr (kind == R_ACC) {
+            constexpr int s2 = (idx / 2) / DM, mt = (idx / 2) % DM;
 #ifndef TRI_ABL_NOACC
-        if (x % 2 == 0) E::mfma_acc(dotr[mt][s2], pf[s2], dvacc[t][mt]);
-        else E::mfma_acc(qtr[mt][s2], dsf[s2], dkacc[t][mt]);
+            if constexpr (idx % 2 == 0) E::mfma_acc(dotr[mt][s2], pf[s2], dvacc[tp][mt]);
+            else E::mfma_acc(qtr[mt][s2], dsf[s2], dkacc[tp][mt]);
 #endif
-      };
-
-      // ---- tile 0: scores and dP with nothing to run beside them -------------------------
-      f32x16 s_cur, p_cur;
-      load_kn(0);
-#pragma unroll
-      for (int a4 = 0; a4 < 4; ++a4) init_quarter(a4, 0, s_cur);
-      p_cur = ndelta;
-#pragma unroll
-      for (int s = 0; s < DS; ++s) {
-        if constexpr (!FLAGGED) s_cur = E::mfma(qn[s], kn[s], s_cur);
-        p_cur = E::mfma(don[s], vf[0][s], p_cur);
-      }
-      load_kn(1);
-      TRI_TS(2)
-
-      // ---- step t: P, dS of tile t (vector ALU) beside the MFMAs of its neighbours: dv, dk
-      // of tile t-1, scores and dP of tile t+1, dq of tile t-1 ------------------------------
-#pragma unroll
-      for (int t = 0; t < KT; ++t) {
-        const bool has_next = t + 1 < KT;
-        f32x16 s_nxt, p_nxt;
-        frag dst_prev[PS], ktr_prev[DM][PS];
-        SB();
-        fetch_bias(jt, t + 2);
-        SB();
-        // score init of tile t+1 | dv, dk of tile t-1
-#pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4) {
-          if (t >= 1) {
-#pragma unroll
-            for (int x = a4 * NACC / 4; x < (a4 + 1) * NACC / 4; ++x) acc_mfma(t - 1, x);
-            if (a4 == 2) {
-              // dS of tile t-1 comes back from LDS with the key index in-lane, with the K
-              // rows of that tile transposed beside it (for dq, two slots further down)
-              const unsigned char* ktile = lds_k + NWV * (t - 1) * 32 * ROWB;
-              const unsigned char* src = ds_tile + ((t - 1) & 1) * 2048;
-#pragma unroll
-              for (int s2 = 0; s2 < PS; ++s2) {
-#ifdef TRI_ABL_NODS
-                dst_prev[s2] = qn[s2 % DS];
-#else
-                dst_prev[s2] = ofd.transposed(src, s2, 0);
-#endif
-#pragma unroll
-                for (int mt = 0; mt < DM; ++mt) ktr_prev[mt][s2] = ofk.transposed(ktile, s2, mt);
-              }
-            }
-          }
-          SB();
-          if (has_next) init_quarter(a4, t + 1, s_nxt);
-          SB();
-        }
-        // P of tile t | scores of tile t+1, then dq of tile t-1
-#pragma unroll
-        for (int bq = 0; bq < 4; ++bq) {
-          if (bq < 2) {
-            if constexpr (!FLAGGED) {
-              if (has_next) {
-#pragma unroll
-                for (int s = bq * DS / 2; s < (bq + 1) * DS / 2; ++s) s_nxt = E::mfma(qn[s], kn[s], s_nxt);
-              }
-            }
           } else {
 #ifndef TRI_ABL_NODQ
-            if (t >= 1) {
-#pragma unroll
-              for (int x = (bq - 2) * NDQ / 2; x < (bq - 1) * NDQ / 2; ++x)
-                dqacc[x % DM] = E::mfma(ktr_prev[x % DM][x / DM], dst_prev[x / DM], dqacc[x % DM]);
-            }
+            dqacc[idx % DM] = E::mfma(ktr_prev[idx % DM][idx / DM], dst_prev[idx / DM], dqacc[idx % DM]);
 #endif
           }
           SB();
-          p_quarter(bq, t, s_cur);
-          SB();
-        }
-        if (t + 2 < KT) load_kn(t + 2);
-        // dS of tile t | dP of tile t+1
-#pragma unroll
-        for (int cq = 0; cq < 2; ++cq) {
-          if (has_next) {
-#pragma unroll
-            for (int s = cq * DS / 2; s < (cq + 1) * DS / 2; ++s) p_nxt = E::mfma(don[s], vf[(t + 1) % KT][s], s == 0 ? ndelta : p_nxt);
-          }
-          SB();
-          ds_half(cq, p_cur);
-          SB();
-        }
-        // P, dS -> B operands; dS -> one of the wave's two LDS tiles [key][query]
-#pragma unroll
-        for (int s2 = 0; s2 < PS; ++s2) pf[s2] = E::pack(&p[KP * s2]);
-        SB();
-#pragma unroll
-        for (int s2 = 0; s2 < PS; ++s2) dsf[s2] = E::pack(&ds[KP * s2]);
-        {
-          unsigned char* dst = ds_tile + (t & 1) * 2048;
-          *reinterpret_cast<frag*>(dst + ds_w0) = dsf[0];
-          *reinterpret_cast<frag*>(dst + ds_w1) = dsf[1];
-        }
-        load_qd_tr();  // for the dv, dk MFMAs of this tile, at the start of the next step
-        SB();
-        if (has_next) { s_cur = s_nxt; p_cur = p_nxt; }
-      }
-      TRI_TS(3)
-      // ---- the last tile's dv, dk and dq ---------------------------------------------------
-      {
-        const unsigned char* ktile = lds_k + NWV * (KT - 1) * 32 * ROWB;
-        const unsigned char* src = ds_tile + ((KT - 1) & 1) * 2048;
-        frag dst_prev[PS], ktr_prev[DM][PS];
-#pragma unroll
-        for (int s2 = 0; s2 < PS; ++s2) {
-          dst_prev[s2] = ofd.transposed(src, s2, 0);
-#pragma unroll
-          for (int mt = 0; mt < DM; ++mt) ktr_prev[mt][s2] = ofk.transposed(ktile, s2, mt);
-        }
-#pragma unroll
-        for (int x = 0; x < NACC; ++x) acc_mfma(KT - 1, x);
 #ifndef TRI_ABL_NODQ
+          if constexpr (has_prev && x == Sch::value.dq_reads_at) {
+            // dS of tile t-1 comes back from LDS with the key index in-lane, with the K
+            // rows of that tile transposed beside it
+            const unsigned char* ktile = lds_k + NWV * tp * 32 * ROWB;
 #pragma unroll
-        for (int x = 0; x < NDQ; ++x) dqacc[x % DM] = E::mfma(ktr_prev[x % DM][x / DM], dst_prev[x / DM], dqacc[x % DM]);
+            for (int s2 = 0; s2 < PS; ++s2) {
+              dst_prev[s2] = ofd.transposed(ds_tile, s2, 0);
+#pragma unroll
+              for (int mt = 0; mt < DM; ++mt) ktr_prev[mt][s2] = ofk.transposed(ktile, s2, mt);
+            }
+          }
 #endif
-      }
-      TRI_TS(4)
+          if constexpr (refill && x == refill_at) {
+            // (the last query tiles fetch the last one again, into a stage nobody reads any more)
+            issue_stage(min(jt + 2, NJ - 1), buf_fill);
+            fetch_bias(jt, t + 2);
+          }
+          if constexpr (has_next && x == Sch::value.last_sqk && t + 2 < KT) load_kn(t + 2);
+          if constexpr (has_next && tn >= VR && x == Sch::value.v_reads_at) {
+#pragma unroll
+            for (int s = 0; s < DS; ++s) vn[s] = v_lds[((tn - VR) * DS + s) * 64];
+          }
+#pragma unroll
+          for (int u = x * NU / NM; u < (x + 1) * NU / NM; ++u) {
+            if (u < 8) {
+#pragma unroll
+#ifdef TRI_ABL_NOEXP
+              for (int e = 0; e < 2; ++e) p[2 * u + e] = s_cur[2 * u + e] * c;
+#else
+              for (int e = 0; e < 2; ++e) p[2 * u + e] = fast_exp2(s_cur[2 * u + e] * c);
+#endif
+            } else if (u < 12) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) ds[4 * (u - 8) + e] = p[4 * (u - 8) + e] * p_cur[4 * (u - 8) + e];
+            } else if (u < 14) {
+              pf[u - 12] = E::pack(&p[KP * (u - 12)]);
+            } else {
+              dsf[u - 14] = E::pack(&ds[KP * (u - 14)]);
+            }
+          }
+          SB();
+        });
+        if constexpr (valu) {
+          // dS -> one of the wave's two LDS tiles [key][query]; Q^T, dO^T for the dv, dk
+          // MFMAs of this tile, which the next step starts with
+#ifndef TRI_ABL_NODQ
+          *reinterpret_cast<frag*>(ds_tile + ds_w0) = dsf[0];
+          *reinterpret_cast<frag*>(ds_tile + ds_w1) = dsf[1];
+#endif
+#ifndef TRI_ABL_NOACC
+          if constexpr (!QD_ONCE) load_qd_tr();
+#endif
+          SB();
+        }
+        if constexpr (has_next) { s_cur = s_nxt; p_cur = p_nxt; }
+        TRI_TS(t < 0 ? 1 : t == KT - 2 ? 6 : t < KT ? 2 : 3)
+      };
+      static_for<KT + 2>(step);
 
       // this wave's partial dq tile -> LDS
-      const int rbuf = NRED == 2 ? buf : 0;
+      const int rbuf = NRED == 2 ? (jt & 1) : 0;
+      int ln = lane;
+      asm volatile("" : "+v"(ln));
 #pragma unroll
       for (int mt = 0; mt < DM; ++mt)
 #pragma unroll
@@ -545,23 +625,24 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
           f32x4 x;
 #pragma unroll
           for (int e = 0; e < 4; ++e) x[e] = dqacc[mt][4 * q + e];
-          *red_slot(rbuf, wave, mt, q) = x;
+          *red_slot(rbuf, wave, mt, q, ln) = x;
         }
+      TRI_TS(4)
+      // The stage of the next query tile was requested a whole query tile ago; since then
+      // the wave has issued the loads of the stage after it and (unless the row is fully
+      // masked) of two bias tiles: everything older than those has landed.  A barrier
+      // without a fence: a fence would wait for the loads in flight.
+      ring_sync<G2W + (FLAGGED ? 0 : 4)>();
+      buf = buf == 2 ? 0 : buf + 1;
       TRI_TS(5)
-      wait_dma();
-      __syncthreads();
-      TRI_TS(6)
       if constexpr (NRED == 1) {
         reduce_dq(jt, 0);
-        __syncthreads();
+        ring_sync<G2W + (FLAGGED ? 0 : 4)>();
       }
     }
     if constexpr (NRED == 2) reduce_dq(NJ - 1, (NJ - 1) & 1);
-    // the query tiles still in the staging buffer: everything from the last flushed half on
-    __syncthreads();
-    flush_dq(NJ >= 2 ? (NJ - 2) / DQH * DQH : 0, NJ);
 #ifdef TRI_ROW_PROF
-    // phase cycle totals of wave 0 of the first workgroup -> the front of the db partial buffer
+    // phase tick totals of wave 0 of the first workgroup -> the front of the db partial buffer
     if (blockIdx.x == 0 && wave == 0 && a.dbpart) {
       prof[7] = __builtin_amdgcn_s_memtime() - tstart;
 #pragma unroll

@@ -32,6 +32,12 @@ TRI_DEV void xcd_remap(int gx, int& x, int& y) {
 #define TRI_L3 __attribute__((address_space(3)))
 
 TRI_DEV void wait_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// The same wait as an instruction the compiler knows: what it waits for no longer counts as
+// in flight when the compiler places its own waits (vmcnt = 0, the other counters at maximum).
+TRI_DEV void wait_dma_known() {
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  asm volatile("" ::: "memory");
+}
 
 // Stage hand-over for a ring of LDS buffers: wait until at most the newest
 // IN_FLIGHT loads of this wave are outstanding (loads complete in issue order, so
