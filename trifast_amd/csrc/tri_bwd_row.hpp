@@ -323,11 +323,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   const T* bias_lane = pack_bh + (perm32(kl) + 32 * g) * 8;
   auto bias_load = [&](int jt, int t, u32x4v* dst) {
     const int kt = min(NWV * t + wave, a.NP - 1);
-#ifdef TRI_ABL_BIAS0
-    const T* p = bias_lane + (int64_t)(kt & 1) * 1024 + 0 * jt;
-#else
     const T* p = bias_lane + ((int64_t)min(jt, a.NP - 1) * a.NP + kt) * 1024;
-#endif
     dst[0] = *reinterpret_cast<const u32x4v*>(p);
     dst[1] = *reinterpret_cast<const u32x4v*>(p + 512);
   };
@@ -337,11 +333,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   // (query, g) the keys 16 r + 8 g + 0..7 as its contraction slots; the constant B operand
   // of half r holds sqrt(d) in the slot that stands for the lane's own key (column) and
   // zero elsewhere.  sqrt(32) is not a 16-bit number: it goes in as hi + lo, one MFMA each.
-#ifdef TRI_ABL_HIONLY
-  constexpr int NPART = 1;
-#else
   constexpr int NPART = D == 32 ? 2 : 1;
-#endif
   constexpr int NSB = 2 * NPART;
   frag bsel[2][NPART];
   {
@@ -439,14 +431,6 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
     };
     fetch_bias(0, 0);
     fetch_bias(0, 1);
-#ifdef TRI_ROW_PROF
-    uint64_t prof[8] = {};
-    const uint64_t tstart = __builtin_amdgcn_s_memtime();
-    uint64_t tlast = tstart;
-#define TRI_TS(k) { SB(); const uint64_t now = __builtin_amdgcn_s_memtime(); prof[k] += now - tlast; tlast = now; SB(); }
-#else
-#define TRI_TS(k)
-#endif
     int buf = 0;  // jt % 3: the stage of this query tile
     for (int jt = 0; jt < NJ; ++jt) {
       const int buf_fill = buf == 0 ? 2 : buf - 1;  // (jt + 2) % 3: the stage to refill
@@ -503,7 +487,6 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
       };
       load_kn(0);
       if constexpr (QD_ONCE) load_qd_tr();
-      TRI_TS(0)
 
       // Step t (t = -1 .. KT): the vector work of tile t (P, dS, their conversions) between
       // the MFMAs of its neighbours: dv, dk and dq of tile t-1, scores and dP of tile t+1,
@@ -532,9 +515,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
           if constexpr (kind == R_SOFF) {
             s_nxt = E::mfma(s_off.get(), kb, zero16());
           } else if constexpr (kind == R_SB) {
-#ifndef TRI_ABL_NOSB
             s_nxt = E::mfma(__builtin_bit_cast(frag, bias_ring[tn % 2][idx / NPART]), bsel[idx / NPART][idx % NPART], s_nxt);
-#endif
           } else if constexpr (kind == R_SQK) {
             s_nxt = E::mfma(qn[idx], kn[idx], s_nxt);
           } else if constexpr (kind == R_DOFF) {
@@ -544,17 +525,12 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
             else p_nxt = E::mfma(don[idx], vn[idx], p_nxt);
           } else if constexpr (kind == R_ACC) {
             constexpr int s2 = (idx / 2) / DM, mt = (idx / 2) % DM;
-#ifndef TRI_ABL_NOACC
             if constexpr (idx % 2 == 0) E::mfma_acc(dotr[mt][s2], pf[s2], dvacc[tp][mt]);
             else E::mfma_acc(qtr[mt][s2], dsf[s2], dkacc[tp][mt]);
-#endif
           } else {
-#ifndef TRI_ABL_NODQ
             dqacc[idx % DM] = E::mfma(ktr_prev[idx % DM][idx / DM], dst_prev[idx / DM], dqacc[idx % DM]);
-#endif
           }
           SB();
-#ifndef TRI_ABL_NODQ
           if constexpr (has_prev && x == Sch::value.dq_reads_at) {
             // dS of tile t-1 comes back from LDS with the key index in-lane, with the K
             // rows of that tile transposed beside it
@@ -566,7 +542,6 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
               for (int mt = 0; mt < DM; ++mt) ktr_prev[mt][s2] = ofk.transposed(ktile, s2, mt);
             }
           }
-#endif
           if constexpr (refill && x == refill_at) {
             // (the last query tiles fetch the last one again, into a stage nobody reads any more)
             issue_stage(min(jt + 2, NJ - 1), buf_fill);
@@ -581,11 +556,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
           for (int u = x * NU / NM; u < (x + 1) * NU / NM; ++u) {
             if (u < 8) {
 #pragma unroll
-#ifdef TRI_ABL_NOEXP
-              for (int e = 0; e < 2; ++e) p[2 * u + e] = s_cur[2 * u + e] * c;
-#else
               for (int e = 0; e < 2; ++e) p[2 * u + e] = fast_exp2(s_cur[2 * u + e] * c);
-#endif
             } else if (u < 12) {
 #pragma unroll
               for (int e = 0; e < 4; ++e) ds[4 * (u - 8) + e] = p[4 * (u - 8) + e] * p_cur[4 * (u - 8) + e];
@@ -600,17 +571,12 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
         if constexpr (valu) {
           // dS -> one of the wave's two LDS tiles [key][query]; Q^T, dO^T for the dv, dk
           // MFMAs of this tile, which the next step starts with
-#ifndef TRI_ABL_NODQ
           *reinterpret_cast<frag*>(ds_tile + ds_w0) = dsf[0];
           *reinterpret_cast<frag*>(ds_tile + ds_w1) = dsf[1];
-#endif
-#ifndef TRI_ABL_NOACC
           if constexpr (!QD_ONCE) load_qd_tr();
-#endif
           SB();
         }
         if constexpr (has_next) { s_cur = s_nxt; p_cur = p_nxt; }
-        TRI_TS(t < 0 ? 1 : t == KT - 2 ? 6 : t < KT ? 2 : 3)
       };
       static_for<KT + 2>(step);
 
@@ -627,29 +593,18 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
           for (int e = 0; e < 4; ++e) x[e] = dqacc[mt][4 * q + e];
           *red_slot(rbuf, wave, mt, q, ln) = x;
         }
-      TRI_TS(4)
       // The stage of the next query tile was requested a whole query tile ago; since then
       // the wave has issued the loads of the stage after it and (unless the row is fully
       // masked) of two bias tiles: everything older than those has landed.  A barrier
       // without a fence: a fence would wait for the loads in flight.
       ring_sync<G2W + (FLAGGED ? 0 : 4)>();
       buf = buf == 2 ? 0 : buf + 1;
-      TRI_TS(5)
       if constexpr (NRED == 1) {
         reduce_dq(jt, 0);
         ring_sync<G2W + (FLAGGED ? 0 : 4)>();
       }
     }
     if constexpr (NRED == 2) reduce_dq(NJ - 1, (NJ - 1) & 1);
-#ifdef TRI_ROW_PROF
-    // phase tick totals of wave 0 of the first workgroup -> the front of the db partial buffer
-    if (blockIdx.x == 0 && wave == 0 && a.dbpart) {
-      prof[7] = __builtin_amdgcn_s_memtime() - tstart;
-#pragma unroll
-      for (int kk = 0; kk < 8; ++kk)
-        if (lane == kk) reinterpret_cast<uint64_t*>(a.dbpart)[kk] = prof[kk];
-    }
-#endif
 
     // ---- dk, dv of this wave's keys -------------------------------------------------------
     // (the accumulators were last written by MFMAs inside asm statements, which the compiler

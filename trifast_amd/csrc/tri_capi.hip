@@ -499,7 +499,9 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   // The pre-passes are cheap (n^2 elements) and make every single-kernel call
   // self-contained, so they run on every call.
   if ((rc = run_mask_prep(mask, mask_strides, w, b, n, st))) return rc;
-  if ((rc = run_bias_prep(bias, bias_strides, w, true, b, h, n, dtype, st))) return rc;
+  // (only the dk/dv tiles that do not also produce dq read the key-major packed bias)
+  const bool want_k = do_kv && !tri::bwd_kv_tile_writes_dq(tkv);
+  if ((rc = run_bias_prep(bias, bias_strides, w, want_k, b, h, n, dtype, st))) return rc;
 
   tri::BwdArgs a;
   a.q = q; a.k = k; a.v = v; a.o = o; a.dout = dout;
