@@ -11,12 +11,13 @@
 // recomputes for its tiles
 //   S^T = K Q^T + bias - lse, P^T = exp2(c S^T), dP^T = V dO^T - delta, dS^T = P^T dP^T
 // with every operand in its natural row-major layout: a lane owns one query
-// (column) and 16 keys of each tile.  The additive terms ride on the matrix pipe:
+// (column) and 16 keys of each tile.  The additive terms cost the vector ALU nothing:
 // the bias tiles (register-resident, fp32, raw-score domain) are the accumulator
-// init of every row's score MFMA, and the per-query terms -lse*sqrt(d) and -delta
-// enter through one extra MFMA each (see rank1_operand, OffsetMask), which leaves
-// one multiply, one exp2 and one fma per element to the vector ALU.  Masked keys get
-// a large negative score from the MFMA that adds -lse.
+// init of every row's score MFMA; -delta (per query) enters through one extra MFMA
+// (see rank1_operand); -lse is one number per lane and is the addend of the fma that
+// scales the score for exp2.  That leaves two fmas and one exp2 per element.  In a tile
+// with masked keys -lse moves to an extra MFMA that it shares with the key mask (see
+// OffsetMask): masked keys get a large negative score there.
 //
 // All workgroups of one (batch*head, chunk) read the same rows at about the same
 // time; the block index is remapped so that they run on one XCD and share its L2.
@@ -206,19 +207,14 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   ofq.make_absolute(tri_smem);
   ofk.pin();
   ofq.pin();
-  // this lane's query in the lse / delta words (lanes 32..63: the zero words behind
-  // them), as an absolute LDS address
-  int scalar_off = (g ? BJ * 4 : ((wj * WJ) * 32 + jl) * 4) + (int)(uintptr_t)(TRI_L3 const unsigned char*)tri_smem;
+  // this lane's query in the lse / delta words, as an absolute LDS address (both halves of
+  // the wave read the word of their query: lanes 32..63 zero it where it becomes a rank-1
+  // operand, and use it as it is where -lse enters as a per-lane term of the exponent)
+  int scalar_off = ((wj * WJ) * 32 + jl) * 4 + (int)(uintptr_t)(TRI_L3 const unsigned char*)tri_smem;
   asm volatile("" : "+v"(scalar_off));
-  if (wave == 0) {
-#pragma unroll
-    for (int u = 0; u < NBUF; ++u) {
-      // (the lse word shares its MFMA with the key mask: in fp32 the slot of lanes 32..63
-      // belongs to the mask and the queries operand holds a one there)
-      reinterpret_cast<uint32_t*>(tri_smem + u * STAGE + OFF_LSE + BJ * 4)[lane] = sizeof(T) == 4 ? OffsetMask<T>::ones_dword() : 0u;
-      reinterpret_cast<uint32_t*>(tri_smem + u * STAGE + OFF_DELTA + BJ * 4)[lane] = 0u;
-    }
-  }
+  // (the lse word shares its MFMA with the key mask: in fp32 the slot of lanes 32..63
+  // belongs to the mask and the queries operand holds a one there)
+  const uint32_t upper_l = sizeof(T) == 4 ? OffsetMask<T>::ones_dword() : 0u;
   // LDS reads take a 16-bit immediate offset: for ring buffers past the first 64 KiB a
   // second set of lane offsets, moved up by two stages, keeps the buffer's offset an
   // immediate (the reads of those buffers would otherwise each need an address add)
@@ -242,12 +238,6 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   for (int tj = 0; tj < WJ; ++tj) { lrank[tj].init(0u, g); drank[tj].init(); }
   typename OffsetMask<T>::Keys kop;
   kop.init(perm32(jl), g);
-  frag kop_plain = kop.plain();
-  if constexpr (sizeof(T) == 2) {
-    typename OffsetMask<T>::u32x4 t = __builtin_bit_cast(typename OffsetMask<T>::u32x4, kop_plain);
-    asm volatile("" : "+v"(t));  // kept in registers, not rebuilt from constants per use
-    kop_plain = __builtin_bit_cast(frag, t);
-  }
 
   const float c = a.c;
   const bool wave_live = j_wave < N && k_wave < N;
@@ -265,6 +255,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     const bool flagged = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const uint32_t*>(st + OFF_FLAG)) != 0;
     frag qf[WJ][DS], dof[WJ][DS], kf[WK][DS], vf[WK][DS];
     frag lf[WJ], df[WJ];  // per-query terms -lse*sqrt(d) and -delta as rank-1 MFMA operands
+    float nl2[WJ];         // -lse of this lane's query in the exponent's unit
 #pragma unroll
     for (int tj = 0; tj < WJ; ++tj) {
 #pragma unroll
@@ -272,9 +263,12 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
         qf[tj][s] = oq.natural_at(sl + OFF_Q + tj * 32 * ROWB, s);
         dof[tj][s] = oq.natural_at(sl + OFF_DO + tj * 32 * ROWB, s);
       }
-      lrank[tj].set_raw(*reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_LSE + tj * 128 + soff)));
+      const uint32_t lw = *reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_LSE + tj * 128 + soff));
+      const uint32_t dw = *reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_DELTA + tj * 128 + soff));
+      lrank[tj].set_raw(g ? upper_l : lw);
       lf[tj] = lrank[tj].get();
-      df[tj] = drank[tj].set(*reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_DELTA + tj * 128 + soff)));
+      df[tj] = drank[tj].set(g ? 0u : dw);
+      nl2[tj] = split_value<T>(lw) * c;
     }
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk)
@@ -291,13 +285,22 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
 #pragma unroll
       for (int tj = 0; tj < WJ; ++tj) {
         f32x16 s;
+        float addend = 0.f;
         // Each case ends in the MFMA that defines s from the bias tile in place (a
         // select between accumulator inits would copy 16 registers).
         if (!flagged) {
-          if (keepw == 0xffffffffu) s = E::mfma(kop_plain, lf[tj], biasr[tj][tk]);
-          else s = E::mfma(kop.masked(keepw), lf[tj], biasr[tj][tk]);  // masked keys: large negative score
+          if (keepw == 0xffffffffu) {
+            // no masked key in the tile: a lane owns one query, so -lse is one number per
+            // lane and rides on the multiply of the exponent (an fma) instead of an MFMA
+            s = E::mfma(kf[tk][0], qf[tj][0], biasr[tj][tk]);
 #pragma unroll
-          for (int sd = 0; sd < DS; ++sd) s = E::mfma(kf[tk][sd], qf[tj][sd], s);
+            for (int sd = 1; sd < DS; ++sd) s = E::mfma(kf[tk][sd], qf[tj][sd], s);
+            addend = nl2[tj];
+          } else {
+            s = E::mfma(kop.masked(keepw), lf[tj], biasr[tj][tk]);  // masked keys: large negative score
+#pragma unroll
+            for (int sd = 0; sd < DS; ++sd) s = E::mfma(kf[tk][sd], qf[tj][sd], s);
+          }
         } else {
           // rare: a fully masked row ignores q.k and the bias
           asm volatile("" ::);
@@ -308,7 +311,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
         for (int sd = 0; sd < DS; ++sd) dp = E::mfma(vf[tk][sd], dof[tj][sd], dp);
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const float p = fast_exp2(s[v] * c);
+          const float p = fast_exp2(__builtin_fmaf(s[v], c, addend));
           dbacc[tj][tk][v] = __builtin_fmaf(p, dp[v], dbacc[tj][tk][v]);
         }
       }

@@ -242,6 +242,17 @@ TRI_DEV uint32_t split_word(float x) {
     return (uint32_t)__builtin_bit_cast(uint16_t, hi) | ((uint32_t)__builtin_bit_cast(uint16_t, lo) << 16);
   }
 }
+// the number a split word stands for
+template <typename T>
+TRI_DEV float split_value(uint32_t w) {
+  if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(float, w);
+  } else {
+    const T hi = __builtin_bit_cast(T, (uint16_t)(w & 0xffffu));
+    const T lo = __builtin_bit_cast(T, (uint16_t)(w >> 16));
+    return (float)hi + (float)lo;
+  }
+}
 // Per-query offset and key mask through ONE extra MFMA of a transposed score tile
 // (rows = keys, columns = queries): the contraction slots are shared between the two
 // rank-1 terms.
