@@ -71,12 +71,17 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   // Linear block id L = 8 * slot + xcd (workgroups go to the 8 XCDs round-robin).
   // Every XCD walks its own sequence of (batch*head, chunk) groups; the launcher
   // pads the group count to a multiple of 8.
+  // With fewer than 8 groups each group gets 8 / groups XCDs (whole number) and deals its
+  // blocks to them in turn, so that no XCD stays idle: the rows are then fetched once per XCD
+  // of the group.
   const int per_group = gridDim.x * gridDim.y;
   const int L = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
   const int slot = L >> 3;
-  const int group = 8 * (slot / per_group) + (L & 7);
-  if (group >= a.BH * a.nchunks) return;
-  const int within = slot % per_group;
+  const int ngroups = a.BH * a.nchunks;
+  const int share = ngroups >= 8 ? 1 : 8 / ngroups;  // XCDs per group
+  const int group = share == 1 ? 8 * (slot / per_group) + (L & 7) : (L & 7) / share;
+  const int within = share == 1 ? slot % per_group : slot * share + (L & 7) % share;
+  if (group >= ngroups || within >= per_group) return;
   const int bh = group % a.BH, chunk = group / a.BH;
   const int b = bh / a.H, h = bh % a.H;
   const int j_blk = (within % gridDim.x) * BJ, k_blk = (within / gridDim.x) * BKB;
