@@ -31,11 +31,11 @@ def row_attention(q_i, k_i, v_i, bias, mask_i):
     return torch.einsum("hjk,hkd->hjd", torch.softmax(s, dim=-1), v_i)
 
 
-def rows_reference(q, k, v, bias, mask, do, dtype):
+def rows_reference(q, k, v, bias, mask, do, dtype, rows=ROWS):
     """o, dq, dk, dv of the chosen rows and db summed over them, computed in `dtype`."""
     out = {}
     db = torch.zeros_like(bias[0], dtype=torch.float32)
-    for i in ROWS:
+    for i in rows:
         q_i, k_i, v_i = (t[0, :, i].to(dtype).detach().requires_grad_(True) for t in (q, k, v))
         b = bias[0].to(dtype).detach().requires_grad_(True)
         o_i = row_attention(q_i, k_i, v_i, b, mask[0, i])
@@ -75,3 +75,27 @@ def test_offsets_beyond_32_bits():
     # rows that received no upstream gradient have none to give
     for i in (2, 4094):
         assert not q.grad[0, :, i].any() and not k.grad[0, :, i].any() and not v.grad[0, :, i].any()
+
+
+@pytest.mark.parametrize("n,h", [(1792, 3), (2048, 2), (2944, 1)])
+def test_bias_gradient_with_few_head_groups(n, h):
+    """Long rows with few heads: the bias-gradient kernel then has fewer (batch*head, row
+    chunk) groups than the GPU has XCDs and deals the blocks of a group to several XCDs
+    (3, 2 and 1 groups here).  db is checked through rows that carry all of the upstream
+    gradient, as above."""
+    dev, dtype = "cuda", torch.bfloat16
+    rows = (0, n // 2 + 1, n - 1)
+    g = torch.Generator(device=dev).manual_seed(n + h)
+    q, k, v = (torch.randn(1, h, n, n, D, device=dev, dtype=dtype, generator=g) * D**-0.25 for _ in range(3))
+    bias = torch.randn(1, h, n, n, device=dev, dtype=dtype, generator=g)
+    mask = torch.rand(1, n, n, device=dev, generator=g) < 0.2
+    do = torch.zeros_like(q)
+    for i in rows:
+        do[0, :, i] = torch.randn(h, n, D, device=dev, dtype=dtype, generator=g)
+    q, k, v, bias = (t.requires_grad_(True) for t in (q, k, v, bias))
+    trifast_amd.triangle_attention(q, k, v, bias, mask).backward(do)
+    torch.cuda.synchronize()
+    _, db_ref = rows_reference(q, k, v, bias, mask, do, torch.float32, rows)
+    _, db_pt = rows_reference(q, k, v, bias, mask, do, dtype, rows)
+    assert torch.isfinite(bias.grad.float()).all()
+    orc.compare_values(bias.grad[0], db_pt, db_ref, f"n={n} h={h} db", eps=orc.DTYPE_EPS[dtype])
