@@ -151,7 +151,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   using E = Elem<T>;
   using frag = typename E::frag;
   using Tile = LdsTile<T, D>;
-  using DsTile = LdsTile<T, 32>;
+  using DsTile = LdsTile<T, 32, 2>;  // the wave's dS tile: 16-byte stores of whole rows, transposed reads
   constexpr int NWV = kRowWaves;
   constexpr int KP = E::KP;
   constexpr int DS = D / (2 * KP);
@@ -310,7 +310,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   ofq.init(perm32(kl), lane);
   ofk.init(kl, lane);
   ofk.shift(wave * 32 * ROWB);  // key tile t of this wave starts (4 t + wave) * 32 rows into K
-  OperandOffsets<T, 32> ofd;
+  OperandOffsets<T, 32, 2> ofd;
   ofd.init(0, lane);
   // (one tile: the wave reads dS of a key tile back before it writes the next one)
   unsigned char* const ds_tile = tri_smem + OFF_DS + wave * 2048;

@@ -50,11 +50,15 @@ TRI_DEV void ring_sync() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(IN_FLIGHT) : "memory");
 }
 
-template <typename T, int D>
+// SWZ_ROWS: rows that share one swizzle value (0: as many as make 256 bytes, which is what
+// 16-byte operand reads of 16 rows want; a tile that is written with 16-byte stores, one row
+// per lane, and only read back transposed wants 2: measured, the stores then run without
+// bank conflicts, and transposing reads take whole rows, so any per-row swizzle suits them).
+template <typename T, int D, int SWZ_ROWS = 0>
 struct LdsTile {
   static constexpr int ROWB = D * (int)sizeof(T);  // bytes per row
   static constexpr int CPR = ROWB / 16;            // 16-byte chunks per row (power of two)
-  static constexpr int RPB = (256 / ROWB) > 0 ? 256 / ROWB : 1;  // rows per 256 bytes
+  static constexpr int RPB = SWZ_ROWS > 0 ? SWZ_ROWS : ((256 / ROWB) > 0 ? 256 / ROWB : 1);  // rows per swizzle value
   static constexpr int VEC = 16 / (int)sizeof(T);
   TRI_DEV static int swz(int r) { return (r / RPB) % CPR; }
   // byte offset, from the tile base, of byte `o` of row r (o must not straddle a chunk)
@@ -112,9 +116,9 @@ struct LdsTile {
 // the swizzle, so an operand read is (tile base + compile-time offset) + one of
 // these registers.  fp32 operands are single elements with many steps: their
 // offsets are computed where they are used.
-template <typename T, int D>
+template <typename T, int D, int SWZ_ROWS = 0>
 struct OperandOffsets {
-  using Tile = LdsTile<T, D>;
+  using Tile = LdsTile<T, D, SWZ_ROWS>;
   using frag = typename Elem<T>::frag;
   static constexpr int KP = Elem<T>::KP;
   static constexpr int DS = D / (2 * KP);
