@@ -113,17 +113,19 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk) dbacc[tj][tk] = zero16();
 
-  // The loads of one row, as a flat list of wave-sized items: 1 KiB pieces of the Q,
-  // dO, K, V tiles (16 bytes per lane), 64-float pieces of lse2 and -delta, the keep
-  // words of the key block and the row's flag (4 bytes per lane).  Wave w takes items w, w + NW, ...; every
-  // wave issues exactly XN loads per row (a wave that runs out repeats the last
-  // item, which rewrites the same bytes), so "all but the newest K rows have
-  // landed" is one s_waitcnt vmcnt(K * XN) for every wave.  Queries and keys past
+  // The loads of one row, as two lists of wave-sized items: 1 KiB pieces of the Q, dO, K,
+  // V tiles (16 bytes per lane), and 64-float pieces of lse2 and -delta, the keep words of
+  // the key block and the row's flag (4 bytes per lane).  Wave w takes items w, w + NW, ...
+  // of each list; every wave issues exactly XW wide and XF narrow loads per row, in that
+  // order (a wave that runs out repeats the last item of the list, which rewrites the same
+  // bytes), so the width of a load is known at compile time and "all but the newest K rows
+  // have landed" is one s_waitcnt vmcnt(K * XN) for every wave.  Queries and keys past
   // the end are clamped (they feed db entries that are never stored).
   constexpr int CPR = Tile::CPR;
   constexpr int GQ = BJ * CPR / 64, GKK = BKB * CPR / 64, GF = BJ / 64;
-  constexpr int TOT = 2 * GQ + 2 * GKK + 2 * GF + 2;
-  constexpr int XN = (TOT + NW - 1) / NW;
+  constexpr int TOTW = 2 * GQ + 2 * GKK, TOTF = 2 * GF + 2;
+  constexpr int XW = (TOTW + NW - 1) / NW, XF = (TOTF + NW - 1) / NW;
+  constexpr int XN = XW + XF;
   static_assert(BJ * CPR % 64 == 0 && BKB * CPR % 64 == 0 && BJ % 64 == 0, "whole wave loads only");
   auto uniform64 = [](int64_t x) -> int64_t {
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)x), hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)x >> 32));
@@ -132,7 +134,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   const char* item_ptr[XN];   // source of the next row to load (per lane)
   int64_t item_step[XN];      // bytes from one pair row to the next (wave-uniform, in scalar registers)
   int item_lds[XN];           // destination offset inside a stage (wave-uniform)
-  bool item_wide[XN];         // 16-byte (tile) or 4-byte (float / meta) lanes
+  // (items 0 .. XW-1 move 16 bytes per lane, items XW .. XN-1 4 bytes)
   {
     const int es = (int)sizeof(T);
     auto tile_item = [&](int x, int gi, const T* base, int64_t srow, int64_t si, int blk, int off) {
@@ -141,11 +143,13 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
       item_ptr[x] = reinterpret_cast<const char*>(base + (int64_t)min(blk + r, N - 1) * srow + cc * Tile::VEC) + (int64_t)i_begin * si * es;
       item_step[x] = uniform64(si * es);
       item_lds[x] = off + gi * 1024;
-      item_wide[x] = true;
     };
 #pragma unroll
     for (int x = 0; x < XN; ++x) {
-      int it = __builtin_amdgcn_readfirstlane(min(x * NW + wave, TOT - 1));
+      // position in the flat order Q | dO | K | V | lse2 | delta | keep words | flag
+      const int it = x < XW ? __builtin_amdgcn_readfirstlane(min(x * NW + wave, TOTW - 1))
+                            : TOTW + __builtin_amdgcn_readfirstlane(min((x - XW) * NW + wave, TOTF - 1));
+      constexpr int TOT = TOTW + TOTF;
       if (it < GQ) {
         tile_item(x, it, qbase, a.sq.j, a.sq.i, j_blk, OFF_Q);
       } else if (it < 2 * GQ) {
@@ -161,19 +165,16 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
         item_ptr[x] = reinterpret_cast<const char*>(base + (int64_t)i_begin * N + min(j_blk + gi * 64 + lane, N - 1));
         item_step[x] = uniform64((int64_t)N * 4);
         item_lds[x] = ((f < GF) ? OFF_LSE : OFF_DELTA) + gi * 256;
-        item_wide[x] = false;
       } else if (it < TOT - 1) {
         // the keep words of this key block (lanes past the block repeat the last word)
         item_ptr[x] = reinterpret_cast<const char*>(a.keep + ((int64_t)b * N + i_begin) * a.nwords + min(k_blk / 32 + min(lane, WKW - 1), a.nwords - 1));
         item_step[x] = uniform64((int64_t)a.nwords * 4);
         item_lds[x] = OFF_META;
-        item_wide[x] = false;
       } else {
         // the row's flag, the same word for every lane
         item_ptr[x] = reinterpret_cast<const char*>(a.rowflag + (int64_t)b * N + i_begin);
         item_step[x] = 4;
         item_lds[x] = OFF_FLAG;
-        item_wide[x] = false;
       }
     }
   }
@@ -186,7 +187,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     ++rows_issued;
 #pragma unroll
     for (int x = 0; x < XN; ++x) {
-      if (item_wide[x]) __builtin_amdgcn_global_load_lds((const TRI_G1 void*)item_ptr[x], (TRI_L3 void*)(st + item_lds[x]), 16, 0, 0);
+      if (x < XW) __builtin_amdgcn_global_load_lds((const TRI_G1 void*)item_ptr[x], (TRI_L3 void*)(st + item_lds[x]), 16, 0, 0);
       else __builtin_amdgcn_global_load_lds((const TRI_G1 void*)item_ptr[x], (TRI_L3 void*)(st + item_lds[x]), 4, 0, 0);
       item_ptr[x] += advance ? item_step[x] : 0;
     }
