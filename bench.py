@@ -37,10 +37,10 @@ PEAK_HBM_GBS = 8000.0
 # as roofline.traffic when the benchmark runs that workload with that tile (keyed by the
 # tile's index in the library's table of the kernel).
 MEASURED_TRAFFIC_MIB = {
-    ("M", "_fwd", 3): 1516.9,
-    ("M", "_bwd_q", 1): 2338.1,
-    ("M", "_bwd_kv", 7): 2691.6,
-    ("M", "_bwd_b", 4): 1649.1,
+    ("M", "_fwd", 3): 1518.5,
+    ("M", "_bwd_q", 1): 2332.5,
+    ("M", "_bwd_kv", 7): 2652.8,
+    ("M", "_bwd_b", 4): 1649.0,
 }
 
 # name -> (dtype, b, n, h, d, description)
