@@ -5,11 +5,12 @@
 // SIMD with the whole register file.  The keys of the row are dealt to the waves
 // in tiles of 32 (wave w owns key tiles w, w+4, ...; at most KT of them): their
 // dk, dv accumulators stay in registers for the whole row, their V rows too (B
-// operands), and the K row of the pair row sits in LDS for the whole workgroup
-// (read as B operand of the scores and, transposed, as A operand of dq).  The
-// queries of the row are streamed through LDS in tiles of 32 (Q, dO rows, direct
-// global->LDS loads, double-buffered).  Per (query tile, key tile), with the
-// scores un-transposed (a lane owns one key and 16 queries):
+// operands; in a private piece of LDS where the registers do not hold them all), and
+// the K row of the pair row sits in LDS for the whole workgroup (read as B operand of
+// the scores and, transposed, as A operand of dq).  The queries of the row are
+// streamed through LDS in tiles of 32 (Q, dO rows, direct global->LDS loads, three
+// stages: in use, ready, in flight).  Per (query tile, key tile), with the scores
+// un-transposed (a lane owns one key and 16 queries):
 //   S  = Q K^T + sqrt(d) (bias - lse)      every term through the matrix pipe (below)
 //   P  = exp2(c S)
 //   dP = dO V^T - delta
@@ -17,15 +18,20 @@
 //   dv^T += dO^T P,  dk^T += Q^T dS        P, dS are B operands as they are
 //   dq^T += K^T dS^T                       dS goes through a 2 KiB LDS tile of the wave
 //                                          and comes back transposed (ds_read_tr)
-// A wave alone on its SIMD issues one instruction every four cycles or so, whatever the
-// instruction is, and the matrix pipe has time to spare: so everything that can be said
-// as a matrix product is one.  The packed bias words of a tile are A operands as they
+// Everything additive is a matrix product, which leaves the per-tile vector work free of
+// conversions, selects and adds (matrix and full-rate vector time add up within a wave,
+// so this costs what it saves for the bias; it makes masked rows cost what unmasked ones
+// do and frees the registers the converted tiles took).  The packed bias words of a tile are A operands as they
 // are (a lane owns a query and eight keys) against a constant B operand that holds
 // sqrt(d) where the contraction slot is the column's key; -lse sqrt(d) and -delta (per
 // query) and the key mask (per key) are rank-1 products of operand words.  That leaves
 // the vector ALU one multiply and one exp2 per score, one multiply per dS and the two
 // conversions.  dq of a query tile is the sum of the four waves' partial tiles: they
 // meet in LDS once per query tile and are added in wave order (deterministic, no atomics).
+// The four waves share the LDS pipe, and an LDS instruction occupies it for four cycles
+// whatever its width (transposing reads move half of what 16-byte reads do): operands
+// that do not change over the key tiles of a query tile (Q^T, dO^T) are read once per
+// query tile where the registers allow.
 //
 // The prologue also computes delta = rowsum(o * do) of the row and leaves it, with
 // the row's log-sum-exp, in the per-query planes the db kernel reads.
