@@ -152,6 +152,48 @@ def test_pick_prefers_the_default_tile_on_a_near_tie(tmp_path, monkeypatch):
     tuner.reset()
 
 
+def test_pick_charges_a_tile_what_it_leaves_to_other_kernels(tmp_path, monkeypatch):
+    """dk/dv tiles that do not also produce dq are charged the dq kernel's time: the
+    row-resident tile wins although its own launch is the longest."""
+    monkeypatch.setenv("TRIFAST_CONFIG_DIR", str(tmp_path))
+    monkeypatch.setenv("TRIFAST_AUTOTUNE", "1")
+    monkeypatch.delenv("TRIFAST_FORCE_TUNE", raising=False)
+    monkeypatch.setattr(tuner, "_device_tag", lambda device=None: "Test-GPU_9-5")
+    lib = _lib.load()
+    tiles = tuner.supported_tiles(_lib.KERNEL_BWD_KV, 1024, 4, 32, torch.bfloat16)
+    fused = [t for t in tiles if lib.trifast_bwd_kv_tile_writes_dq(t)]
+    assert len(fused) == 1 and len(tiles) > 1  # 1024 keys: only the largest row-resident tile fits
+    monkeypatch.setattr(tuner, "_time_launch", lambda launch, tile, **kw: 2.1 if tile in fused else 1.6)
+    tuner.reset()
+    assert tuner.pick(_lib.KERNEL_BWD_KV, 1024, 4, 32, torch.bfloat16, lambda t: None) not in fused
+    monkeypatch.setenv("TRIFAST_FORCE_TUNE", "1")
+    extra = lambda t: 0.0 if lib.trifast_bwd_kv_tile_writes_dq(t) else 1.4
+    assert tuner.pick(_lib.KERNEL_BWD_KV, 1024, 4, 32, torch.bfloat16, lambda t: None, extra_cost=extra) == fused[0]
+    tuner.reset()
+
+
+def test_row_resident_tiles_in_the_library_tables():
+    """The row-resident kernel appears as the last four tiles of the dk/dv family, each for rows
+    of up to 256, 512, 768, 1024 keys, for 16-bit inputs, and is the default where it is fastest."""
+    lib = _lib.load()
+    nt = lib.trifast_num_tiles(_lib.KERNEL_BWD_KV)
+    fused = [t for t in range(nt) if lib.trifast_bwd_kv_tile_writes_dq(t)]
+    assert fused == list(range(nt - 4, nt))
+    assert not lib.trifast_bwd_kv_tile_writes_dq(-1) and not lib.trifast_bwd_kv_tile_writes_dq(nt)
+    for t, keys in zip(fused, (256, 512, 768, 1024)):
+        assert _lib.tile_info(_lib.KERNEL_BWD_KV, t)["BLOCK_K"] == keys
+        assert lib.trifast_supports(_lib.KERNEL_BWD_KV, t, keys, 4, 32, _lib.BF16)
+        assert lib.trifast_supports(_lib.KERNEL_BWD_KV, t, keys - 37, 2, 32, _lib.F16)
+        assert not lib.trifast_supports(_lib.KERNEL_BWD_KV, t, keys + 1, 4, 32, _lib.BF16)
+        assert not lib.trifast_supports(_lib.KERNEL_BWD_KV, t, keys, 4, 32, _lib.F32)
+        assert not lib.trifast_supports(_lib.KERNEL_BWD_KV, t, keys, 4, 128, _lib.BF16)
+    default = lambda n, d, code: lib.trifast_default_tile(_lib.KERNEL_BWD_KV, n, 4, d, code)
+    assert default(1024, 32, _lib.BF16) == fused[3] and default(300, 32, _lib.F16) == fused[1]
+    assert default(129, 32, _lib.BF16) == fused[0] and default(1025, 32, _lib.BF16) not in fused
+    assert default(128, 32, _lib.BF16) not in fused and default(512, 64, _lib.BF16) not in fused
+    assert default(512, 32, _lib.F32) not in fused
+
+
 def test_tune_cli_flags_and_sweep():
     p = tune.build_parser()
     a = p.parse_args([])
