@@ -177,6 +177,24 @@ int trifast_bwd_one(int kernel,
                     const int64_t* db_strides,
                     int tile, void* workspace, int64_t workspace_bytes, void* stream);
 
+/*
+ * Output gating of a triangle-attention block, fused with the layout change between the
+ * operator and the block's output projection.  No counterpart in the reference (its callers
+ * are only hinted at by the module of reference tests/unit/test_trifast.py:152-169): this is
+ * the caller-side step that follows trifast_fwd in an AlphaFold-style block.
+ *   forward   y[b, i, j, h, :]  = o[b, h, i, j, :] * sigmoid(g[b, i, j, h, :])
+ *   backward  do[b, h, i, j, :] = dy[b, i, j, h, :] * sigmoid(g)
+ *             dg[b, i, j, h, :] = dy * o * sigmoid(g) * (1 - sigmoid(g))
+ * o, do: the operator's layout [b, h, n, n, d]; g, dg, y, dy: [b, n, n, h, d], the layout of a
+ * linear layer over the pair representation.  All tensors contiguous, 16-byte aligned, of
+ * dtype `dtype`; arithmetic in fp32.  Nothing is allocated; the launch is asynchronous on
+ * `stream`.
+ */
+int trifast_gate_fwd(void* y, const void* o, const void* g,
+                     int64_t b, int64_t h, int64_t n, int64_t d, int dtype, void* stream);
+int trifast_gate_bwd(void* dout, void* dg, const void* dy, const void* o, const void* g,
+                     int64_t b, int64_t h, int64_t n, int64_t d, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -105,6 +105,35 @@ def test_argument_errors_come_back_as_codes_not_crashes():
     assert rc == -1 and "backward kernel" in _lib.last_error()
 
 
+def test_gate_argument_errors_come_back_as_codes():
+    """The gate entries check sizes, dtype and pointers before they launch anything."""
+    lib = _lib.load()
+    ok = 0x1000
+    assert lib.trifast_gate_fwd(ok, ok, ok, 1, 2, 8, 48, _lib.BF16, None) == -2 and "head dim" in _lib.last_error()
+    assert lib.trifast_gate_fwd(None, ok, ok, 1, 2, 8, 32, _lib.BF16, None) == -1 and "null" in _lib.last_error()
+    assert lib.trifast_gate_fwd(ok, ok + 8, ok, 1, 2, 8, 32, _lib.BF16, None) == -3 and "o is not 16-byte" in _lib.last_error()
+    assert lib.trifast_gate_bwd(ok, ok, None, ok, ok, 1, 2, 8, 32, _lib.BF16, None) == -1 and "dy" in _lib.last_error()
+    assert lib.trifast_gate_bwd(ok + 4, ok, ok, ok, ok, 1, 2, 8, 32, _lib.F32, None) == -3 and "do" in _lib.last_error()
+    assert lib.trifast_gate_bwd(ok, ok, ok, ok, ok, 1, 2, 8, 32, 7, None) < 0
+
+
+def test_gated_output_checks_shapes_on_the_host():
+    import torch
+
+    from trifast_amd import nn
+
+    o = torch.zeros(1, 2, 8, 8, 16)
+    with pytest.raises(ValueError, match="g must be"):
+        nn.gated_output(o, torch.zeros(1, 8, 8, 16))
+    with pytest.raises(TypeError):
+        nn.gated_output(o, torch.zeros(1, 8, 8, 32, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="GPU only"):  # no CPU fallback
+        nn.gated_output(o, torch.zeros(1, 8, 8, 32))
+    block = nn.TriangleAttention(24, 2, 16, ending_node=True)
+    assert block.heads(torch.zeros(3, 8, 8, 32)).shape == (3, 2, 8, 8, 16)
+    assert {n for n, _ in block.named_parameters()} == {"q.weight", "k.weight", "v.weight", "b.weight", "g.weight", "g.bias", "out.weight", "out.bias"}
+
+
 def test_output_pointers_and_strides_are_checked():
     """Gradients and lse are written / read with vector accesses: a misaligned pointer or
     a stride the kernels cannot write comes back as TRIFAST_EALIGN, not as a fault."""

@@ -1,0 +1,134 @@
+"""The gated block around the operator (trifast_amd.nn) on the GPU.
+
+The gate kernel is checked against its formula in fp64 with the rounding bound of one
+result in the tensors' dtype; the block against the same block built from the oracle and
+plain PyTorch ops with the same weights (values, input and parameter gradients).
+"""
+
+import pytest
+import torch
+
+import trifast_amd
+from oracle import triangle_oracle as orc
+from trifast_amd import nn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def gate_reference(o, g):
+    """y[*, i, j, h*d] = o[*, h, i, j, d] * sigmoid(g)."""
+    return o.movedim(-4, -2).flatten(-2) * torch.sigmoid(g)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
+@pytest.mark.parametrize("lead,h,n,d", [((2,), 4, 33, 32), ((), 1, 7, 16), ((2, 2), 3, 20, 64), ((1,), 2, 130, 128)])
+def test_gate_forward_and_backward(dtype, lead, h, n, d):
+    gen = torch.Generator().manual_seed(n * 1000 + d)
+    o = torch.randn(*lead, h, n, n, d, generator=gen).to(DEV, dtype)
+    g = (3 * torch.randn(*lead, n, n, h * d, generator=gen)).to(DEV, dtype)
+    dy = torch.randn(*lead, n, n, h * d, generator=gen).to(DEV, dtype)
+    oo, gg = o.clone().requires_grad_(True), g.clone().requires_grad_(True)
+    y = nn.gated_output(oo, gg)
+    assert y.shape == g.shape and y.dtype == dtype
+    y.backward(dy)
+    ro, rg = o.double().requires_grad_(True), g.double().requires_grad_(True)
+    ry = gate_reference(ro, rg)
+    ry.backward(dy.double())
+    # the kernel computes in fp32 (hardware exp2 of x log2 e: a few fp32 ulps) and rounds once to the dtype
+    for name, got, want in (("y", y.detach(), ry.detach()), ("do", oo.grad, ro.grad), ("dg", gg.grad, rg.grad)):
+        assert got.shape == want.shape, name
+        err = (got.double() - want).abs()
+        bound = 0.5 * torch.finfo(dtype).eps * want.abs() + 16 * 2.0**-23 * want.abs() + torch.finfo(dtype).smallest_normal
+        assert bool((err <= bound).all()), f"{name} {dtype}: max excess {(err - bound).max().item():.3e}"
+
+
+def test_gate_of_a_strided_operand_is_made_dense_first():
+    o = torch.randn(2, 2, 16, 16, 32, device=DEV, dtype=torch.bfloat16).transpose(2, 3)
+    g = torch.randn(2, 16, 16, 64, device=DEV, dtype=torch.bfloat16)
+    assert torch.equal(nn.gated_output(o, g), nn.gated_output(o.contiguous(), g))
+
+
+def test_empty_gate():
+    o = torch.zeros(0, 2, 8, 8, 16, device=DEV)
+    assert nn.gated_output(o, torch.zeros(0, 8, 8, 32, device=DEV)).shape == (0, 8, 8, 32)
+
+
+class ReferenceBlock(torch.nn.Module):
+    """trifast_amd.nn.TriangleAttention from the oracle and plain PyTorch ops, with copies
+    where the product uses views; ending node by explicit transposition of the pair dims."""
+
+    def __init__(self, c_in, h, d, ending_node):
+        super().__init__()
+        self.h, self.d, self.ending_node = h, d, ending_node
+        self.q = torch.nn.Linear(c_in, h * d, bias=False)
+        self.k = torch.nn.Linear(c_in, h * d, bias=False)
+        self.v = torch.nn.Linear(c_in, h * d, bias=False)
+        self.b = torch.nn.Linear(c_in, h, bias=False)
+        self.g = torch.nn.Linear(c_in, h * d)
+        self.out = torch.nn.Linear(h * d, c_in)
+
+    def forward(self, x, mask):
+        g = self.g(x)
+        if self.ending_node:
+            x, mask = x.transpose(-2, -3).contiguous(), mask.transpose(-1, -2).contiguous()
+        heads = lambda t: t.unflatten(-1, (self.h, self.d)).permute(0, 3, 1, 2, 4).contiguous()
+        o = orc.attention_reference(heads(self.q(x)), heads(self.k(x)), heads(self.v(x)), self.b(x).permute(0, 3, 1, 2).contiguous(), mask)
+        o = o.permute(0, 2, 3, 1, 4).flatten(-2)
+        if self.ending_node:
+            o = o.transpose(-2, -3)
+        return self.out(o * torch.sigmoid(g))
+
+
+@pytest.mark.parametrize("ending_node", [False, True], ids=["starting", "ending"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_block_matches_the_reference_block(ending_node, dtype):
+    torch.manual_seed(3)
+    bs, n, c, h, d = 2, 40, 48, 2, 32
+    x = torch.randn(bs, n, n, c, device=DEV)
+    mask = torch.rand(bs, n, n, device=DEV) < 0.2
+    label = torch.randn(bs, n, n, c, device=DEV)
+    ours = nn.TriangleAttention(c, h, d, ending_node).to(DEV)
+    ref32 = ReferenceBlock(c, h, d, ending_node).to(DEV)
+    ref32.load_state_dict(ours.state_dict())
+
+    def run(model, dt):
+        model = model.to(dt)
+        xi = x.to(dt).detach().requires_grad_(True)
+        out = model(xi, mask)
+        torch.nn.functional.mse_loss(out.float(), label).backward()
+        res = {"out": out.detach().float(), "x": xi.grad.float(), **{k: p.grad.float() for k, p in model.named_parameters()}}
+        model.zero_grad()
+        return res
+
+    want = run(ref32, torch.float32)
+    got = run(ours, dtype)
+    if dtype == torch.float32:
+        for name in want:
+            a, r = got[name], want[name]
+            assert (a - r).abs().max().item() <= 3e-5 * max(r.abs().max().item(), 1e-6) + 1e-7, f"{name}: {(a - r).abs().max().item():.3e}"
+        return
+    # low precision: our block may be at most 3x as far from fp32 as the same reference block run in that dtype
+    refl = ReferenceBlock(c, h, d, ending_node).to(DEV)
+    refl.load_state_dict({k: v.float() for k, v in ours.state_dict().items()})
+    pt = run(refl, dtype)
+    for name in want:
+        e_ours = (got[name] - want[name]).abs().max().item()
+        e_pt = (pt[name] - want[name]).abs().max().item()
+        assert e_ours <= 3 * e_pt + 1e-6, f"{name}: ours {e_ours:.3e} vs PyTorch in {dtype} {e_pt:.3e}"
+
+
+def test_block_trains():
+    """Reference tests/unit/test_trifast.py:172-210 on the gated block: every parameter moves."""
+    torch.manual_seed(0)
+    model = nn.TriangleAttention(32, 4, 32).to(DEV, torch.bfloat16)
+    x = torch.randn(1, 48, 48, 32, device=DEV, dtype=torch.bfloat16)
+    mask = torch.rand(1, 48, 48, device=DEV) < 0.3
+    opt = torch.optim.Adam(model.parameters(), lr=1e-2)
+    before = {k: p.detach().clone() for k, p in model.named_parameters()}
+    for _ in range(3):
+        opt.zero_grad()
+        model(x, mask).float().square().mean().backward()
+        opt.step()
+    for k, p in model.named_parameters():
+        assert torch.isfinite(p).all() and not torch.equal(before[k], p), k

@@ -12,6 +12,7 @@
 #include "../../include/trifast_hip.h"
 #include "tri_common.hpp"
 #include "tri_launch.hpp"
+#include "tri_gate.hpp"
 
 namespace tri {
 
@@ -564,6 +565,36 @@ int trifast_bwd_one(int kernel, void* dq, void* dk, void* dv, void* db, const vo
   return bwd_impl(kernel, dq, dk, dv, db, dout, q, k, v, bias, mask, o, lse, b, h, n, d, dtype, do_strides,
                   q_strides, k_strides, v_strides, bias_strides, mask_strides, dq_strides, dk_strides,
                   dv_strides, db_strides, tiles, workspace, workspace_bytes, stream);
+}
+
+namespace {
+int gate_impl(bool bwd, void* y_or_dg, void* dox, const void* dy, const void* o, const void* g, int64_t b, int64_t h,
+              int64_t n, int64_t d, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (int rc = check_common(b, h, n, d, dtype)) return rc;
+  const void* ptrs[5] = {y_or_dg, o, g, bwd ? dox : o, bwd ? dy : o};
+  static const char* const names[5] = {"output", "o", "g", "do", "dy"};
+  for (int x = 0; x < 5; ++x) {
+    if (!ptrs[x]) return fail(TRIFAST_EINVAL, "gate: %s is a null pointer", names[x]);
+    if ((reinterpret_cast<uintptr_t>(ptrs[x]) & 15) != 0) return fail(TRIFAST_EALIGN, "gate: %s is not 16-byte aligned", names[x]);
+  }
+  tri::GateArgs a;
+  a.y = y_or_dg; a.dox = dox; a.o = o; a.g = g; a.dy = dy;
+  a.rows = b * n * n; a.plane = n * n; a.H = (int)h; a.D = (int)d;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const hipError_t e = bwd ? tri::gate_launch<true>(a, dtype, st) : tri::gate_launch<false>(a, dtype, st);
+  if (e != hipSuccess) return hip_fail(e, "gate launch");
+  return 0;
+}
+}  // namespace
+
+int trifast_gate_fwd(void* y, const void* o, const void* g, int64_t b, int64_t h, int64_t n, int64_t d, int dtype, void* stream) {
+  return gate_impl(false, y, nullptr, nullptr, o, g, b, h, n, d, dtype, stream);
+}
+
+int trifast_gate_bwd(void* dout, void* dg, const void* dy, const void* o, const void* g, int64_t b, int64_t h, int64_t n,
+                     int64_t d, int dtype, void* stream) {
+  return gate_impl(true, dg, dout, dy, o, g, b, h, n, d, dtype, stream);
 }
 
 }  // extern "C"

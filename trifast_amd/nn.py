@@ -1,0 +1,101 @@
+"""Callers of the operator: the gated triangle-attention block of AlphaFold-style models.
+
+The reference ships the operator only; its tests hint at the surrounding module
+(reference tests/unit/test_trifast.py:152-169: linear layers for q, k, v and the bias over
+a pair representation ``x [*, n, n, c]``).  This module is that block written so that no
+tensor is copied to change its layout:
+
+* q, k, v leave their linear layers as ``[*, n, n, h*d]`` and go to the operator as
+  ``[*, h, n, n, d]`` *views* (heads interleaved, 64-byte rows for d = 32 bf16); the bias
+  as a ``[*, h, n, n]`` view of ``[*, n, n, h]``.  The operator reads them through their
+  strides and writes dq, dk, dv, db with the same strides, so autograd needs no re-layout
+  copy on the way back either.
+* The output gate ``o * sigmoid(g)`` and the layout change from the operator's
+  ``[*, h, n, n, d]`` to the ``[*, n, n, h*d]`` that the output projection consumes are one
+  streaming HIP kernel (``trifast_gate_fwd`` / ``trifast_gate_bwd``).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from trifast_amd import _lib
+from trifast_amd.torch import _dtype_code, triangle_attention, triangle_attention_ending_node
+
+
+def _gate_shapes(o: torch.Tensor, g: torch.Tensor) -> tuple[int, int, int, int]:
+    if o.dim() < 4:
+        raise ValueError(f"o must be [*, h, n, n, d], got shape {tuple(o.shape)}")
+    *lead, h, n, n2, d = o.shape
+    if n != n2:
+        raise ValueError(f"o must be square in its pair dims, got shape {tuple(o.shape)}")
+    if tuple(g.shape) != (*lead, n, n, h * d):
+        raise ValueError(f"g must be [*, n, n, h*d] = {(*lead, n, n, h * d)}, got {tuple(g.shape)}")
+    if g.dtype != o.dtype:
+        raise TypeError("o and g must share one dtype")
+    if not (o.is_cuda and g.is_cuda and o.device == g.device):
+        raise RuntimeError("gated_output runs on the GPU only (o and g on one device)")
+    b = 1
+    for s in lead:
+        b *= s
+    return b, h, n, d
+
+
+class _GatedOutput(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+        b, h, n, d = _gate_shapes(o, g)
+        o, g = o.contiguous(), g.contiguous()
+        y = torch.empty_like(g)
+        if y.numel():
+            rc = _lib.load().trifast_gate_fwd(y.data_ptr(), o.data_ptr(), g.data_ptr(), b, h, n, d, _dtype_code(o),
+                                              torch.cuda.current_stream(o.device).cuda_stream)
+            _lib.check(rc, "trifast_gate_fwd")
+        ctx.save_for_backward(o, g)
+        ctx.dims = (b, h, n, d)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy: torch.Tensor):
+        o, g = ctx.saved_tensors
+        b, h, n, d = ctx.dims
+        dy = dy.contiguous()
+        do, dg = torch.empty_like(o), torch.empty_like(g)
+        if dy.numel():
+            rc = _lib.load().trifast_gate_bwd(do.data_ptr(), dg.data_ptr(), dy.data_ptr(), o.data_ptr(), g.data_ptr(),
+                                              b, h, n, d, _dtype_code(o), torch.cuda.current_stream(o.device).cuda_stream)
+            _lib.check(rc, "trifast_gate_bwd")
+        return do, dg
+
+
+def gated_output(o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+    """``y[*, i, j, h*d] = o[*, h, i, j, d] * sigmoid(g[*, i, j, h*d])``: the operator's output
+    gated and handed to the output projection in one pass."""
+    return _GatedOutput.apply(o, g)
+
+
+class TriangleAttention(torch.nn.Module):
+    """Gated triangle self-attention around the starting node (``ending_node=False``) or the
+    ending node of a pair representation ``x [*, n, n, c_in]``; ``mask [*, n, n]`` is True
+    where a pair is masked out (the operator's polarity)."""
+
+    def __init__(self, c_in: int, h: int, d: int, ending_node: bool = False):
+        super().__init__()
+        self.h, self.d, self.ending_node = h, d, ending_node
+        self.q = torch.nn.Linear(c_in, h * d, bias=False)
+        self.k = torch.nn.Linear(c_in, h * d, bias=False)
+        self.v = torch.nn.Linear(c_in, h * d, bias=False)
+        self.b = torch.nn.Linear(c_in, h, bias=False)
+        self.g = torch.nn.Linear(c_in, h * d)
+        self.out = torch.nn.Linear(h * d, c_in)
+
+    def heads(self, t: torch.Tensor) -> torch.Tensor:
+        """``[*, n, n, h*d] -> [*, h, n, n, d]`` as a view."""
+        return t.unflatten(-1, (self.h, self.d)).movedim(-2, -4)
+
+    def forward(self, x: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
+        q, k, v = self.heads(self.q(x)), self.heads(self.k(x)), self.heads(self.v(x))
+        bias = self.b(x).movedim(-1, -3)
+        attend = triangle_attention_ending_node if self.ending_node else triangle_attention
+        o = attend(q, k, v, bias, mask)
+        return self.out(gated_output(o, self.g(x)))

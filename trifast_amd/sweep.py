@@ -5,6 +5,7 @@ A100 / RTX 3090 files.
 
     python -m trifast_amd.sweep runtime [--out benchmark] [--n-max 2048] [--step 32]
     python -m trifast_amd.sweep memory  [--out benchmark] [--n-max 2048] [--step 32]
+    python -m trifast_amd.sweep block   [--n 1024] [--c-in 128]
 
 Same protocol as reference scripts/benchmark.py:13-105 and scripts/memory.py:25-131:
 bf16, h=4, d=32, 50 % random mask, n = 32..2048 in steps of 32; "fwd" times the forward,
@@ -12,6 +13,12 @@ bf16, h=4, d=32, 50 % random mask, n = 32..2048 in steps of 32; "fwd" times the 
 milliseconds; memory is ``torch.cuda.max_memory_allocated`` around one forward
 (+ backward) in MiB.  Only the "Trifast" column is produced: the other columns of the
 reference's tables are other implementations.
+
+``block`` has no counterpart in the reference: it times the gated block of
+``trifast_amd.nn`` (projections, operator, gate, output projection; forward + backward)
+against the same block with the layout copies and the unfused gate a caller would write
+in plain PyTorch around the operator, and the gate kernels alone against the HBM bytes
+they must move.
 """
 
 from __future__ import annotations
@@ -105,15 +112,57 @@ def memory(out: Path, ns: list[int], repeat: int = 3) -> None:
     print(f"wrote {out / 'memory.parquet'} and {out / 'memory.csv'}")
 
 
+def block(n: int, c_in: int) -> None:
+    from . import nn
+
+    dev = torch.device("cuda")
+    torch.manual_seed(0)
+    fused = nn.TriangleAttention(c_in, H, D).to(dev, DTYPE)
+
+    def unfused(x, mask):
+        m = fused
+        heads = lambda t: t.unflatten(-1, (H, D)).permute(0, 3, 1, 2, 4).contiguous()
+        o = triangle_attention(heads(m.q(x)), heads(m.k(x)), heads(m.v(x)), m.b(x).permute(0, 3, 1, 2).contiguous(), mask)
+        return m.out(o.permute(0, 2, 3, 1, 4).flatten(-2) * torch.sigmoid(m.g(x)))
+
+    x = torch.randn(1, n, n, c_in, device=dev, dtype=DTYPE, requires_grad=True)
+    mask = torch.rand(1, n, n, device=dev) < 0.5
+    dy = torch.randn(1, n, n, c_in, device=dev, dtype=DTYPE)
+
+    def step(fn):
+        fn(x, mask).backward(dy)
+        x.grad = None
+        fused.zero_grad(set_to_none=True)
+
+    ms_fused = _median_ms(lambda: step(fused))
+    ms_unfused = _median_ms(lambda: step(unfused))
+    print(f"block n={n} c_in={c_in} h={H} d={D} {DTYPE}: forward+backward {ms_fused:.3f} ms with views and the fused gate, "
+          f"{ms_unfused:.3f} ms with layout copies and the gate in PyTorch ops ({ms_unfused / ms_fused:.2f}x)")
+    o = torch.randn(1, H, n, n, D, device=dev, dtype=DTYPE)
+    g = torch.randn(1, n, n, H * D, device=dev, dtype=DTYPE)
+    gy = torch.randn_like(g)
+    size = o.numel() * o.element_size()
+    ms = _median_ms(lambda: nn._GatedOutput.apply(o, g))
+    print(f"gate forward  {ms * 1e3:8.1f} us  {3 * size / ms / 1e6:7.1f} GB/s of 3 tensors x {size / 2**20:.0f} MiB")
+    oo, gg = o.clone().requires_grad_(True), g.clone().requires_grad_(True)
+    y = nn.gated_output(oo, gg)
+    ms = _median_ms(lambda: torch.autograd.grad(y, (oo, gg), gy, retain_graph=True))
+    print(f"gate backward {ms * 1e3:8.1f} us  {5 * size / ms / 1e6:7.1f} GB/s of 5 tensors x {size / 2**20:.0f} MiB")
+
+
 def main() -> None:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("what", choices=["runtime", "memory"])
+    ap.add_argument("what", choices=["runtime", "memory", "block"])
     ap.add_argument("--out", default="benchmark")
     ap.add_argument("--n-max", type=int, default=2048)
     ap.add_argument("--step", type=int, default=32)
+    ap.add_argument("--n", type=int, default=1024, help="block: sequence length")
+    ap.add_argument("--c-in", type=int, default=128, help="block: channels of the pair representation")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("the sweeps need a GPU: the operator has no CPU path")
+    if args.what == "block":
+        return block(args.n, args.c_in)
     ns = list(range(args.step, args.n_max + 1, args.step))
     (runtime if args.what == "runtime" else memory)(Path(args.out), ns)
 
