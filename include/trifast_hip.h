@@ -24,7 +24,8 @@
  *       lse         : contiguous float32 [b, h, n, n], natural log, indexed [i, j]
  *     Vector accesses need 16-byte alignment: base pointers of q, k, v, do, o, dq, dk,
  *     dv, db must be 16-byte aligned and the si/sj/sh/sb strides of the q-like ones
- *     multiples of 16/sizeof(elem); lse must be 4-byte aligned.  Outputs must not
+ *     multiples of 16/sizeof(elem), with 0 <= sj * sizeof(elem) < 2^24 (the rows of a tile
+ *     are addressed with 32-bit offsets); lse must be 4-byte aligned.  Outputs must not
  *     overlap themselves or each other (no zero strides over a dim larger than 1).
  *     bias and mask are re-tiled by pre-pass kernels into the workspace, so they
  *     carry no alignment or contiguity requirement.

@@ -100,6 +100,9 @@ def test_argument_errors_come_back_as_codes_not_crashes():
     bad_stride = _lib.i64_array([0, 0, 0, 32, 2])
     rc = lib.trifast_fwd(0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 1, 1, 8, 32, _lib.BF16, bad_stride, st5, st5, st4, st3, -1, None, 0, None)
     assert rc == -3 and "last stride" in _lib.last_error()
+    far_rows = _lib.i64_array([0, 0, 32, 1 << 23, 1])  # 16 MiB between the rows of a bf16 tile
+    rc = lib.trifast_fwd(0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 1, 1, 8, 32, _lib.BF16, st5, far_rows, st5, st4, st3, -1, None, 0, None)
+    assert rc == -2 and "stride 3" in _lib.last_error()
     none4 = (None, None, None, None)
     rc = lib.trifast_bwd_one(0, *([0x1000] * 12), 1, 1, 8, 32, _lib.BF16, st5, st5, st5, st5, st4, st3, *none4, -1, None, 0, None)
     assert rc == -1 and "backward kernel" in _lib.last_error()

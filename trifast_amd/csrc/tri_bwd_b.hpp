@@ -35,7 +35,7 @@
 namespace tri {
 
 // LDS bytes of one stage (one pair row) of the kernel below
-constexpr int bwd_b_stage_bytes(int BJ, int BKB, int ROWB) { return 2 * (BJ * 4 + 256) + 512 + (2 * BJ + 2 * BKB) * ROWB; }
+constexpr int bwd_b_stage_bytes(int BJ, int BKB, int ROWB) { return 2 * (BJ * 4 + 256) + (2 * BJ + 2 * BKB) * ROWB; }
 
 template <typename T, int D, int GJ, int GK, int WJ, int WK, int NBUF>
 __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a) {
@@ -47,18 +47,14 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   constexpr int NW = GJ * GK;
   constexpr int BJ = GJ * WJ * 32, BKB = GK * WK * 32;  // queries / keys per workgroup
   constexpr int ROWB = Tile::ROWB;
-  // one stage: lse2[BJ] | 64 zero words | -delta[BJ] | 64 zero words | keep words of the
-  // key block (64 words) | the row's flag (64 copies) | Q rows | dO rows | K rows | V rows.
-  // The small arrays come first so that their offsets in every ring buffer fit the
-  // 16-bit immediate of an LDS read; the zero words are what lanes 32..63 read as
-  // their (empty) half of a rank-1 operand.
+  // one stage: lse2[BJ] | 64 spare words | -delta[BJ] | 64 spare words | Q rows | dO rows |
+  // K rows | V rows.  The small arrays come first so that their offsets in every ring
+  // buffer fit the 16-bit immediate of an LDS read.  (The row's flag and keep words do not
+  // pass through LDS: they are wave-uniform and come by scalar loads.)
   constexpr int OFF_LSE = 0, OFF_DELTA = OFF_LSE + BJ * 4 + 256;
-  constexpr int OFF_META = OFF_DELTA + BJ * 4 + 256, OFF_FLAG = OFF_META + 256;
-  constexpr int OFF_Q = OFF_FLAG + 256, OFF_DO = OFF_Q + BJ * ROWB, OFF_K = OFF_DO + BJ * ROWB, OFF_V = OFF_K + BKB * ROWB;
+  constexpr int OFF_Q = OFF_DELTA + BJ * 4 + 256, OFF_DO = OFF_Q + BJ * ROWB, OFF_K = OFF_DO + BJ * ROWB, OFF_V = OFF_K + BKB * ROWB;
   constexpr int STAGE = OFF_V + BKB * ROWB;
   static_assert(STAGE == bwd_b_stage_bytes(BJ, BKB, ROWB), "the launcher sizes LDS with bwd_b_stage_bytes");
-  constexpr int WKW = BKB / 32;
-  static_assert(WKW <= 64, "the keep words of the key block are one 64-lane load");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
 
@@ -114,8 +110,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     for (int tk = 0; tk < WK; ++tk) dbacc[tj][tk] = zero16();
 
   // The loads of one row, as two lists of wave-sized items: 1 KiB pieces of the Q, dO, K,
-  // V tiles (16 bytes per lane), and 64-float pieces of lse2 and -delta, the keep words of
-  // the key block and the row's flag (4 bytes per lane).  Wave w takes items w, w + NW, ...
+  // V tiles (16 bytes per lane), and 64-float pieces of lse2 and -delta (4 bytes per lane).  Wave w takes items w, w + NW, ...
   // of each list; every wave issues exactly XW wide and XF narrow loads per row, in that
   // order (a wave that runs out repeats the last item of the list, which rewrites the same
   // bytes), so the width of a load is known at compile time and "all but the newest K rows
@@ -123,7 +118,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   // the end are clamped (they feed db entries that are never stored).
   constexpr int CPR = Tile::CPR;
   constexpr int GQ = BJ * CPR / 64, GKK = BKB * CPR / 64, GF = BJ / 64;
-  constexpr int TOTW = 2 * GQ + 2 * GKK, TOTF = 2 * GF + 2;
+  constexpr int TOTW = 2 * GQ + 2 * GKK, TOTF = 2 * GF;
   constexpr int XW = (TOTW + NW - 1) / NW, XF = (TOTF + NW - 1) / NW;
   constexpr int XN = XW + XF;
   static_assert(BJ * CPR % 64 == 0 && BKB * CPR % 64 == 0 && BJ % 64 == 0, "whole wave loads only");
@@ -131,8 +126,11 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)x), hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)x >> 32));
     return (int64_t)(((uint64_t)hi << 32) | lo);
   };
-  const char* item_ptr[XN];   // source of the next row to load (per lane)
-  int64_t item_step[XN];      // bytes from one pair row to the next (wave-uniform, in scalar registers)
+  // An item's source is a 64-bit base (wave-uniform, scalar registers, stepped from one pair
+  // row to the next with scalar adds) plus a 32-bit byte offset per lane that never changes.
+  const char* item_base[XN];
+  uint32_t item_voff[XN];
+  int64_t item_step[XN];      // bytes from one pair row to the next (wave-uniform)
   int item_lds[XN];           // destination offset inside a stage (wave-uniform)
   // (items 0 .. XW-1 move 16 bytes per lane, items XW .. XN-1 4 bytes)
   {
@@ -140,16 +138,16 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     auto tile_item = [&](int x, int gi, const T* base, int64_t srow, int64_t si, int blk, int off) {
       const int p = gi * 64 + lane;
       const int r = p / CPR, cc = (p % CPR) ^ Tile::swz(r);
-      item_ptr[x] = reinterpret_cast<const char*>(base + (int64_t)min(blk + r, N - 1) * srow + cc * Tile::VEC) + (int64_t)i_begin * si * es;
+      item_base[x] = reinterpret_cast<const char*>(uniform64((int64_t)(uintptr_t)(base + (int64_t)blk * srow + (int64_t)i_begin * si)));
+      item_voff[x] = (uint32_t)(min(r, N - 1 - blk) * (int)srow + cc * Tile::VEC) * (uint32_t)es;
       item_step[x] = uniform64(si * es);
       item_lds[x] = off + gi * 1024;
     };
 #pragma unroll
     for (int x = 0; x < XN; ++x) {
-      // position in the flat order Q | dO | K | V | lse2 | delta | keep words | flag
+      // position in the flat order Q | dO | K | V | lse2 | delta
       const int it = x < XW ? __builtin_amdgcn_readfirstlane(min(x * NW + wave, TOTW - 1))
                             : TOTW + __builtin_amdgcn_readfirstlane(min((x - XW) * NW + wave, TOTF - 1));
-      constexpr int TOT = TOTW + TOTF;
       if (it < GQ) {
         tile_item(x, it, qbase, a.sq.j, a.sq.i, j_blk, OFF_Q);
       } else if (it < 2 * GQ) {
@@ -158,38 +156,38 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
         tile_item(x, it - 2 * GQ, kbase, a.sk.j, a.sk.i, k_blk, OFF_K);
       } else if (it < 2 * GQ + 2 * GKK) {
         tile_item(x, it - 2 * GQ - GKK, vbase, a.sv.j, a.sv.i, k_blk, OFF_V);
-      } else if (it < 2 * GQ + 2 * GKK + 2 * GF) {
+      } else {
         const int f = it - 2 * GQ - 2 * GKK;
         const int gi = f % GF;
         const float* base = (f < GF) ? lse2_bh : delta_bh;
-        item_ptr[x] = reinterpret_cast<const char*>(base + (int64_t)i_begin * N + min(j_blk + gi * 64 + lane, N - 1));
+        const int j0 = min(j_blk + gi * 64, N - 1);
+        item_base[x] = reinterpret_cast<const char*>(uniform64((int64_t)(uintptr_t)(base + (int64_t)i_begin * N + j0)));
+        item_voff[x] = (uint32_t)(min(lane, N - 1 - j0) * 4);
         item_step[x] = uniform64((int64_t)N * 4);
         item_lds[x] = ((f < GF) ? OFF_LSE : OFF_DELTA) + gi * 256;
-      } else if (it < TOT - 1) {
-        // the keep words of this key block (lanes past the block repeat the last word)
-        item_ptr[x] = reinterpret_cast<const char*>(a.keep + ((int64_t)b * N + i_begin) * a.nwords + min(k_blk / 32 + min(lane, WKW - 1), a.nwords - 1));
-        item_step[x] = uniform64((int64_t)a.nwords * 4);
-        item_lds[x] = OFF_META;
-      } else {
-        // the row's flag, the same word for every lane
-        item_ptr[x] = reinterpret_cast<const char*>(a.rowflag + (int64_t)b * N + i_begin);
-        item_step[x] = 4;
-        item_lds[x] = OFF_FLAG;
       }
     }
   }
+  // all ones if x > 0, else zero, as a 64-bit scalar (written out: the compiler would keep the
+  // condition as a lane mask and turn it into a number with vector instructions in every row)
+  auto ones_while_positive = [](int x) -> int64_t {
+    int64_t m;
+    asm volatile("s_cmp_gt_i32 %1, 0\n\ts_cselect_b64 %0, -1, 0" : "=s"(m) : "s"(__builtin_amdgcn_readfirstlane(x)) : "scc");
+    return m;
+  };
   // issue the loads of the next row into stage buffer `buf`; past the last row of
-  // the chunk the pointers stop and the last row is loaded again (never used)
+  // the chunk the bases stop and the last row is loaded again (never used)
   int rows_issued = 0;
   auto issue_row = [&](int buf) {
-    unsigned char* st = tri_smem + buf * STAGE;
-    const bool advance = rows_issued + 1 < nrows;
+    const uint32_t st = (uint32_t)(uintptr_t)(TRI_L3 unsigned char*)(tri_smem + buf * STAGE);
+    const int64_t advance = ones_while_positive(nrows - 1 - rows_issued);
     ++rows_issued;
 #pragma unroll
     for (int x = 0; x < XN; ++x) {
-      if (x < XW) __builtin_amdgcn_global_load_lds((const TRI_G1 void*)item_ptr[x], (TRI_L3 void*)(st + item_lds[x]), 16, 0, 0);
-      else __builtin_amdgcn_global_load_lds((const TRI_G1 void*)item_ptr[x], (TRI_L3 void*)(st + item_lds[x]), 4, 0, 0);
-      item_ptr[x] += advance ? item_step[x] : 0;
+      const uint32_t dst = __builtin_amdgcn_readfirstlane(st + (uint32_t)item_lds[x]);
+      if (x < XW) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(item_voff[x]), "s"(item_base[x]) : "memory", "m0");
+      else asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(dst), "v"(item_voff[x]), "s"(item_base[x]) : "memory", "m0");
+      item_base[x] += advance & item_step[x];
     }
   };
   // wait until at most the newest `K` rows of this wave's loads are in flight and
@@ -246,11 +244,45 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   kop.init(perm32(jl), g);
 
   const float c = a.c;
-  const bool wave_live = j_wave < N && k_wave < N;
+  // (an integer that the compiler cannot see through: a boolean would be kept as a lane mask
+  // and negated with vector instructions in every row)
+  int wave_live = __builtin_amdgcn_readfirstlane((int)(j_wave < N && k_wave < N));
+  asm volatile("" : "+s"(wave_live));
 
-  auto compute_row = [&](int buf) __attribute__((always_inline)) {
-    const unsigned char* st = tri_smem + buf * STAGE;
-    const uint32_t* meta = reinterpret_cast<const uint32_t*>(st + OFF_META);
+  // The row's flag and the keep words of the wave's key tiles are the same for every lane:
+  // they are read from global memory with scalar loads, one row ahead of their use (rows
+  // past the end of the chunk repeat the last one and are not used).
+  struct RowMeta {
+    uint32_t flag;
+    uint32_t keep[WK];
+  };
+  typedef const __attribute__((address_space(4))) uint32_t* const_words;
+  const int64_t keep_step = uniform64((int64_t)a.nwords * 4);
+  const_words flag_word = (const_words)(uintptr_t)(a.rowflag + (int64_t)b * N + i_begin);
+  // (a key tile past the last word of the row has no attended key: its word is never read)
+  const_words keep_word = (const_words)(uintptr_t)(a.keep + ((int64_t)b * N + i_begin) * a.nwords + min(k_wave / 32, a.nwords - 1));
+  int word_at[WK];         // offset of tile tk's word from keep_word (clamped to the row)
+  uint32_t word_mask[WK];  // zero for a tile past the last word
+#pragma unroll
+  for (int tk = 0; tk < WK; ++tk) {
+    word_at[tk] = __builtin_amdgcn_readfirstlane(min(k_wave / 32 + tk, a.nwords - 1) - min(k_wave / 32, a.nwords - 1));
+    word_mask[tk] = __builtin_amdgcn_readfirstlane(k_wave / 32 + tk < a.nwords ? 0xffffffffu : 0u);
+  }
+  int meta_rows = 0;
+  // the words of the next row (the first call gives those of row 0)
+  auto load_meta = [&]() -> RowMeta {
+    RowMeta m;
+    m.flag = *flag_word;
+#pragma unroll
+    for (int tk = 0; tk < WK; ++tk) m.keep[tk] = keep_word[word_at[tk]] & word_mask[tk];
+    const int64_t advance = ones_while_positive(nrows - 1 - meta_rows);
+    ++meta_rows;
+    flag_word = (const_words)((uintptr_t)flag_word + (uintptr_t)(advance & 4));
+    keep_word = (const_words)((uintptr_t)keep_word + (uintptr_t)(advance & keep_step));
+    return m;
+  };
+
+  auto compute_row = [&](int buf, const RowMeta& meta) __attribute__((always_inline)) {
     const bool high = kHighSet && buf >= 2;  // (a constant once the ring loop is unrolled)
     const int sl = buf * STAGE - (high ? HIGH : 0);  // offset of the buffer for reads through the lane offsets
     const OperandOffsets<T, D>& oq = high ? ofq_hi : ofq;
@@ -258,10 +290,11 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     const int soff = high ? scalar_off_hi : scalar_off;
     // (wave-uniform values are pinned to scalar registers so that the branches on
     // them are real branches and not lane masks)
-    const bool flagged = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const uint32_t*>(st + OFF_FLAG)) != 0;
+    const bool flagged = meta.flag != 0;
     frag qf[WJ][DS], dof[WJ][DS], kf[WK][DS], vf[WK][DS];
     frag lf[WJ], df[WJ];  // per-query terms -lse*sqrt(d) and -delta as rank-1 MFMA operands
     float nl2[WJ];         // -lse of this lane's query in the exponent's unit
+    uint32_t lw[WJ], dw[WJ];
 #pragma unroll
     for (int tj = 0; tj < WJ; ++tj) {
 #pragma unroll
@@ -269,12 +302,8 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
         qf[tj][s] = oq.natural_at(sl + OFF_Q + tj * 32 * ROWB, s);
         dof[tj][s] = oq.natural_at(sl + OFF_DO + tj * 32 * ROWB, s);
       }
-      const uint32_t lw = *reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_LSE + tj * 128 + soff));
-      const uint32_t dw = *reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_DELTA + tj * 128 + soff));
-      lrank[tj].set_raw(g ? upper_l : lw);
-      lf[tj] = lrank[tj].get();
-      df[tj] = drank[tj].set(g ? 0u : dw);
-      nl2[tj] = split_value<T>(lw) * c;
+      lw[tj] = *reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_LSE + tj * 128 + soff));
+      dw[tj] = *reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_DELTA + tj * 128 + soff));
     }
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk)
@@ -283,10 +312,28 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
         kf[tk][s] = ok.natural_at(sl + OFF_K + tk * 32 * ROWB, s);
         vf[tk][s] = ok.natural_at(sl + OFF_V + tk * 32 * ROWB, s);
       }
+    // every LDS read of the row is issued before the first branch on the row's keep words
+    // (read where they are used, they would return in several waited-for batches)
+#pragma unroll
+    for (int tj = 0; tj < WJ; ++tj) {
+#pragma unroll
+      for (int s = 0; s < DS; ++s) asm volatile("" : "+v"(qf[tj][s]), "+v"(dof[tj][s]));
+      asm volatile("" : "+v"(lw[tj]), "+v"(dw[tj]));
+    }
+#pragma unroll
+    for (int tk = 0; tk < WK; ++tk)
+#pragma unroll
+      for (int s = 0; s < DS; ++s) asm volatile("" : "+v"(kf[tk][s]), "+v"(vf[tk][s]));
+#pragma unroll
+    for (int tj = 0; tj < WJ; ++tj) {
+      lrank[tj].set_raw(g ? upper_l : lw[tj]);
+      lf[tj] = lrank[tj].get();
+      df[tj] = drank[tj].set(g ? 0u : dw[tj]);
+      nl2[tj] = split_value<T>(lw[tj]) * c;
+    }
 #pragma unroll
     for (int tk = 0; tk < WK; ++tk) {
-      // a key tile past the last word of the row has no attended key
-      const uint32_t keepw = __builtin_amdgcn_readfirstlane((k_wave / 32 + tk < a.nwords) ? meta[wk * WK + tk] : 0u);
+      const uint32_t keepw = meta.keep[tk];
       if (keepw == 0) continue;  // no attended key in this tile: dS = 0
 #pragma unroll
       for (int tj = 0; tj < WJ; ++tj) {
@@ -303,14 +350,14 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
             for (int sd = 1; sd < DS; ++sd) s = E::mfma(kf[tk][sd], qf[tj][sd], s);
             addend = nl2[tj];
           } else {
-            s = E::mfma(kop.masked(keepw), lf[tj], biasr[tj][tk]);  // masked keys: large negative score
+            s = E::mfma(kop.masked_copy(keepw), lf[tj], biasr[tj][tk]);  // masked keys: large negative score
 #pragma unroll
             for (int sd = 0; sd < DS; ++sd) s = E::mfma(kf[tk][sd], qf[tj][sd], s);
           }
         } else {
           // rare: a fully masked row ignores q.k and the bias
           asm volatile("" ::);
-          s = E::mfma(kop.masked(keepw), lf[tj], zero16());
+          s = E::mfma(kop.masked_copy(keepw), lf[tj], zero16());
         }
         f32x16 dp = E::mfma(ones, df[tj], zero16());
 #pragma unroll
@@ -332,14 +379,17 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     constexpr int P = NBUF - 1;
 #pragma unroll
     for (int u = 0; u < P; ++u) issue_row(u);
+    RowMeta meta = load_meta();
     sync_rows(std::integral_constant<int, P - 1>{});  // row 0 has landed
     for (int r = 0; r < nrows; r += NBUF) {
 #pragma unroll
       for (int u = 0; u < NBUF; ++u) {
         if (r + u < nrows) {
           issue_row((u + P) % NBUF);
-          if (wave_live) compute_row(u);
+          const RowMeta next = load_meta();
+          if (wave_live != 0) compute_row(u, meta);
           sync_rows(std::integral_constant<int, P - 1>{});  // the next row has landed
+          meta = next;
         }
       }
     }
@@ -347,13 +397,14 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     // one stage only (two do not fit in LDS): load, then compute
     for (int ir = 0; ir < nrows; ++ir) {
       issue_row(0);
+      const RowMeta meta = load_meta();
       sync_rows(std::integral_constant<int, 0>{});
-      if (wave_live) compute_row(0);
+      if (wave_live != 0) compute_row(0, meta);
       sync_rows(std::integral_constant<int, 0>{});
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the spare rows loaded past the end
-  if (!wave_live) return;
+  if (wave_live == 0) return;
 
   // a single chunk writes db itself; several chunks write fp32 partials.  The lane
   // owns query j; its 16 values are two runs of 8 consecutive keys.

@@ -219,6 +219,11 @@ int check_qlike(const char* name, const void* p, const int64_t* s, int dtype) {
   if ((reinterpret_cast<uintptr_t>(p) & 15) != 0) return fail(TRIFAST_EALIGN, "%s: base pointer is not 16-byte aligned", name);
   for (int t = 0; t < 4; ++t)
     if (s[t] % vec != 0) return fail(TRIFAST_EALIGN, "%s: stride %d (%lld) is not a multiple of %d elements", name, t, (long long)s[t], vec);
+  // the stage loads address the rows of a tile (up to 256 of them) with 32-bit byte offsets
+  // from the tile's first row
+  const int64_t max_row_stride = (int64_t(1) << 24) / elem_size(dtype);
+  if (s[3] < 0 || s[3] >= max_row_stride)
+    return fail(TRIFAST_EUNSUPPORTED, "%s: stride 3 (%lld) must be in [0, %lld) elements", name, (long long)s[3], (long long)max_row_stride);
   return 0;
 }
 

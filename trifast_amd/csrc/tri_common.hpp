@@ -302,6 +302,18 @@ struct OffsetMask {
         return as_frag(v);
       }
     }
+    // the same as a new value: for callers whose tiles are rarely masked (the operand in
+    // place would be carried, and copied, through the unmasked path as well)
+    TRI_DEV frag masked_copy(uint32_t keepw) const {
+      const uint32_t m = (keepw & bit) ? 0u : mask_dword();
+      u32x4 t = v;
+      if constexpr (sizeof(T) == 4) {
+        if (g) t[0] = m;
+      } else {
+        t[1] = m;
+      }
+      return as_frag(t);
+    }
   };
   // queries operand of the lane that owns a query
   struct Queries {
