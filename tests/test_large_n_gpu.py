@@ -99,3 +99,57 @@ def test_bias_gradient_with_few_head_groups(n, h):
     _, db_pt = rows_reference(q, k, v, bias, mask, do, dtype, rows)
     assert torch.isfinite(bias.grad.float()).all()
     orc.compare_values(bias.grad[0], db_pt, db_ref, f"n={n} h={h} db", eps=orc.DTYPE_EPS[dtype])
+
+
+@pytest.mark.parametrize("n,h,dtype", [(1030, 2, torch.bfloat16), (2048, 1, torch.bfloat16), (1500, 1, torch.float16), (2100, 1, torch.bfloat16)],
+                         ids=["n1030_two_passes_ragged", "n2048_two_passes", "n1500_f16", "n2100_three_passes"])
+def test_row_resident_backward_in_several_passes(n, h, dtype, monkeypatch):
+    """Rows longer than the row-resident kernel holds at once run it once per 1024 keys: dk, dv
+    of each pass's keys and the dq summed over the passes are checked on a few pair rows, among
+    them a fully masked one, one whose attended keys all lie in the last pass and one whose
+    attended keys all lie in the first; db (from the db kernel, which reads the planes the first
+    pass leaves) through the rows that carry the upstream gradient.  Two runs give the same bits."""
+    from trifast_amd import _lib, tuner
+
+    lib = _lib.load()
+    code = _lib.BF16 if dtype == torch.bfloat16 else _lib.F16
+    nt = lib.trifast_num_tiles(_lib.KERNEL_BWD_KV)
+    tile = nt - 1
+    assert lib.trifast_bwd_kv_tile_writes_dq(tile) and lib.trifast_supports(_lib.KERNEL_BWD_KV, tile, n, h, D, code)
+    real_pick = tuner.pick
+    monkeypatch.setattr(tuner, "pick", lambda kern, *a, **kw: tile if kern == _lib.KERNEL_BWD_KV else real_pick(kern, *a, **kw))
+    dev = "cuda"
+    rows = (0, 3, 4, 5, n // 2, n - 1)
+    g = torch.Generator(device=dev).manual_seed(n)
+    q, k, v = (torch.randn(1, h, n, n, D, device=dev, dtype=dtype, generator=g) * D**-0.25 for _ in range(3))
+    bias = torch.randn(1, h, n, n, device=dev, dtype=dtype, generator=g)
+    mask = torch.rand(1, n, n, device=dev, generator=g) < 0.2
+    mask[0, 3, :] = True          # fully masked
+    mask[0, 4, :1024] = True      # nothing to attend to in the first pass
+    mask[0, 5, 1000:] = True      # nothing in the later passes (and a ragged edge inside the first)
+    do = torch.zeros_like(q)
+    for i in rows:
+        do[0, :, i] = torch.randn(h, n, D, device=dev, dtype=dtype, generator=g)
+    grads = []
+    for _ in range(2):
+        leaves = [t.detach().clone().requires_grad_(True) for t in (q, k, v, bias)]
+        o = trifast_amd.triangle_attention(*leaves, mask)
+        o.backward(do)
+        torch.cuda.synchronize()
+        grads.append([t.grad for t in leaves])
+    for a, c in zip(*grads):
+        assert torch.equal(a, c), "two runs differ"
+    dq, dk, dv, db = grads[0]
+    ref, db_ref = rows_reference(q, k, v, bias, mask, do, torch.float32, rows)
+    pt, db_pt = rows_reference(q, k, v, bias, mask, do, dtype, rows)
+    eps = orc.DTYPE_EPS[dtype]
+    for i in rows:
+        got = (dq[0, :, i], dk[0, :, i], dv[0, :, i])
+        for name, x, p, r in zip(("dq", "dk", "dv"), got, pt[i][1:], ref[i][1:]):
+            assert torch.isfinite(x.float()).all(), f"row {i} {name}: non-finite values"
+            orc.compare_values(x.detach(), p, r, f"n={n} row {i} {name}", eps=eps)
+    orc.compare_values(db[0], db_pt, db_ref, f"n={n} db", eps=eps)
+    # masked-out keys get exactly zero dk, dv (row 4: the whole first pass)
+    assert not dk[0, :, 4, :1024].any() and not dv[0, :, 4, :1024].any()
+    # rows without upstream gradient have none to give
+    assert not dq[0, :, 1].any() and not dk[0, :, n - 2].any()

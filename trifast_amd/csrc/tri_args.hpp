@@ -66,6 +66,10 @@ struct BwdArgs {
   float c;                   // log2(e) / sqrt(d)
   float sqrt_d;
   float scale;               // 1 / sqrt(d)
+  // row-resident kernel run in several passes over the keys (rows longer than one pass holds)
+  int key_tile0;             // first 32-key tile of this pass
+  int pass_flags;            // 1: not the first pass, 2: not the last pass
+  void* dq_lo;               // [b*h, n, n, d]: between passes dq is kept as dq (high part) + dq_lo
 };
 
 }  // namespace tri

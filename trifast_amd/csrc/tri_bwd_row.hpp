@@ -36,8 +36,13 @@
 // The prologue also computes delta = rowsum(o * do) of the row and leaves it, with
 // the row's log-sum-exp, in the per-query planes the db kernel reads.
 //
-// Rows up to 128*KT keys fit (1024 keys at head dim 32); longer rows use the dq and
-// dk/dv kernels.  Replaces _bwd_q and _bwd_kv of reference
+// Rows up to 128*KT keys fit (1024 keys at head dim 32).  Longer rows run the kernel in
+// several passes (MULTI), one launch per 128*KT keys: dk and dv of a pass's keys are complete
+// after it, dq is the sum over the passes and travels from one to the next as two numbers of
+// the element type per value (the rounded running sum in dq itself, the rounding error in a
+// workspace plane), which keeps 16 bits of it.  The per-query words are then read from the
+// global planes (the first pass writes them) instead of LDS, where the longer row leaves
+// them no room.  Replaces _bwd_q and _bwd_kv of reference
 // src/trifast/triton.py:274-383 and :143-263 in one pass.
 #pragma once
 #include <type_traits>
@@ -143,15 +148,15 @@ constexpr int bwd_row_v_lds_tiles(int D, int KT) { return KT * (D / 16) < 16 ? 0
 // dq partial buffers: two (one barrier per query tile) unless the longest rows need the room
 constexpr int bwd_row_red_buffers(int D, int KT) { return D <= 32 && KT * (D / 16) < 16 ? 2 : 1; }
 // LDS bytes of the kernel below
-constexpr int bwd_row_base_lds_bytes(int D, int es, int KT) {
+constexpr int bwd_row_base_lds_bytes(int D, int es, int KT, bool multi) {
   const int rowb = D * es, dm = (D + 31) / 32, keys = kRowWaves * KT * 32;
   const int nred = bwd_row_red_buffers(D, KT);
-  return keys * rowb + 3 * (2 * 32 * rowb) + kRowWaves * 2048 + nred * kRowWaves * dm * 4096 + 2 * keys * 4 +
+  return keys * rowb + 3 * (2 * 32 * rowb) + kRowWaves * 2048 + nred * kRowWaves * dm * 4096 + (multi ? 0 : 2 * keys * 4) +
          kRowWaves * bwd_row_v_lds_tiles(D, KT) * (D / 16) * 1024;
 }
-constexpr int bwd_row_lds_bytes(int D, int es, int KT) { return bwd_row_base_lds_bytes(D, es, KT); }
+constexpr int bwd_row_lds_bytes(int D, int es, int KT, bool multi = false) { return bwd_row_base_lds_bytes(D, es, KT, multi); }
 
-template <typename T, int D, int KT>
+template <typename T, int D, int KT, bool MULTI = false>
 __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const BwdArgs a) {
   static_assert(sizeof(T) == 2, "16-bit inputs only (the transposing LDS reads)");
   using E = Elem<T>;
@@ -172,13 +177,14 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   constexpr int OFF_DS = OFF_ST + 3 * STAGE;  // three stages: in use, ready, in flight
   constexpr int OFF_RED = OFF_DS + NWV * 2048;
   constexpr int OFF_NL = OFF_RED + NRED * NWV * DM * 4096;
-  constexpr int OFF_ND = OFF_NL + KEYS * 4;
+  constexpr int PLANE = MULTI ? 0 : KEYS * 4;  // per-query words of the row (single pass only)
+  constexpr int OFF_ND = OFF_NL + PLANE;
   constexpr int G2W = (2 * 32 * (ROWB / 16) / 64 + NWV - 1) / NWV;  // global->LDS loads per wave and stage
   constexpr int VL = bwd_row_v_lds_tiles(D, KT);  // this wave's last VL key tiles keep V in LDS
   constexpr int VR = KT - VL;
-  constexpr int OFF_V = OFF_ND + KEYS * 4;
-  static_assert(OFF_V + NWV * VL * DS * 1024 == bwd_row_lds_bytes(D, (int)sizeof(T), KT), "the launcher sizes LDS with bwd_row_lds_bytes");
-  static_assert(bwd_row_lds_bytes(D, (int)sizeof(T), KT) <= 160 * 1024, "LDS of one compute unit");
+  constexpr int OFF_V = OFF_ND + PLANE;
+  static_assert(OFF_V + NWV * VL * DS * 1024 == bwd_row_lds_bytes(D, (int)sizeof(T), KT, MULTI), "the launcher sizes LDS with bwd_row_lds_bytes");
+  static_assert(bwd_row_lds_bytes(D, (int)sizeof(T), KT, MULTI) <= 160 * 1024, "LDS of one compute unit");
   static_assert((KT - 1) * NWV * 32 * ROWB + 32 * ROWB <= 65536, "key tile offsets are LDS immediates");
   extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
 
@@ -188,6 +194,9 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   const int kl = lane & 31, g = lane >> 5;
   const int N = a.N;
   const int NJ = a.nwords;  // 32-tiles of the row (queries and keys)
+  // this pass: key tiles KT0 .. KT0 + 4 KT - 1 of the row (tiles past the row's end are empty)
+  const int KT0 = MULTI ? a.key_tile0 : 0;
+  const bool first_pass = !MULTI || (a.pass_flags & 1) == 0, last_pass = !MULTI || (a.pass_flags & 2) == 0;
 
   // Workgroups go to the 8 XCDs round-robin by linear id.  Every XCD walks its own
   // contiguous run of (batch*head, row) items, so that at any time it works on one
@@ -212,7 +221,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
 
   // ---- prologue -----------------------------------------------------------------
   // K row -> LDS (rows past the end repeat the last key; their keep bits are clear)
-  Tile::template fill<KEYS, NWV>(lds_k, [&](int r) { return krow + (int64_t)min(r, N - 1) * a.sk.j; }, wave, lane);
+  Tile::template fill<KEYS, NWV>(lds_k, [&](int r) { return krow + (int64_t)min(32 * KT0 + r, N - 1) * a.sk.j; }, wave, lane);
   // query tiles 0 (and 1) -> the two stage buffers
   // (per-lane source pointers for query tile 0, computed once; a tile inside the row adds
   // one uniform offset, the ragged last one clamps the query index)
@@ -257,7 +266,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   uint32_t kw[KT];
 #pragma unroll
   for (int t = 0; t < KT; ++t) {
-    const int kt = NWV * t + wave;
+    const int kt = KT0 + NWV * t + wave;
     kw[t] = __builtin_amdgcn_readfirstlane(kt < NJ ? a.keep[((int64_t)b * N + i) * a.nwords + kt] : 0u);
   }
   const uint32_t lanebit = 1u << kl;
@@ -268,7 +277,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   frag* const v_lds = reinterpret_cast<frag*>(tri_smem + OFF_V + wave * VL * DS * 1024) + lane;
 #pragma unroll
   for (int t = 0; t < KT; ++t) {
-    const int key = min(32 * (NWV * t + wave) + kl, N - 1);
+    const int key = min(32 * (KT0 + NWV * t + wave) + kl, N - 1);
 #pragma unroll
     for (int s = 0; s < DS; ++s) {
       const frag x = *reinterpret_cast<const frag*>(vrow + (int64_t)key * a.sv.j + 2 * KP * s + KP * g);
@@ -279,13 +288,13 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
 
   // per-query terms of the row: -delta and -lse*sqrt(d) (ln n for lse in a fully masked
   // row) as MFMA operand words, kept in LDS for this kernel and written for the db kernel
-  {
+  uint32_t* const dplane = a.delta + ((int64_t)bh * N + i) * N;
+  uint32_t* const lplane = a.lse2 + ((int64_t)bh * N + i) * N;
+  if (first_pass) {
     const T* orow = reinterpret_cast<const T*>(a.o) + ((int64_t)bh * N + i) * N * D;
     const float* lserow = a.lse + ((int64_t)bh * N + i) * N;
-    uint32_t* dplane = a.delta + ((int64_t)bh * N + i) * N;
-    uint32_t* lplane = a.lse2 + ((int64_t)bh * N + i) * N;
     const float flat = -__builtin_amdgcn_logf((float)N) * (kLn2 * a.sqrt_d);
-    for (int j = tid; j < KEYS; j += NWV * 64) {
+    for (int j = tid; j < (MULTI ? N : KEYS); j += NWV * 64) {
       float nlv = E::kMaskElem, ndv = 0.f;  // queries past the end: P = dS = 0
       if (j < N) {
         float dsum = 0.f;
@@ -304,10 +313,24 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
         dplane[j] = dw;
         lplane[j] = lw;
       }
-      nl[j] = lw;
-      nd[j] = dw;
+      if constexpr (!MULTI) {
+        nl[j] = lw;
+        nd[j] = dw;
+      }
     }
   }
+  // (several passes: the words come back from the global planes, which the first pass has just
+  // written: its stores are waited for, with the loads, before the barrier below; the loads
+  // are made at device scope so that no stale copy in the first-level cache can serve them)
+  auto fetch_words = [&](int jt, uint32_t& lw, uint32_t& dw) {
+    const int j = 32 * min(jt, NJ - 1) + perm32(kl);
+    lw = split_word<T>(E::kMaskElem);  // queries past the end: P = dS = 0
+    dw = split_word<T>(0.f);
+    if (j < N) {
+      lw = __hip_atomic_load(lplane + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      dw = __hip_atomic_load(dplane + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
 
   // lane-constant LDS offsets.  Q, dO tiles: natural A operands (tile row m stands for
   // query perm32(m)) and transposed A operands; K tiles: natural B operand of this lane's
@@ -328,7 +351,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   // (as A operand: operand row m stands for query perm32(m), like the Q and dO operands)
   const T* bias_lane = pack_bh + (perm32(kl) + 32 * g) * 8;
   auto bias_load = [&](int jt, int t, u32x4v* dst) {
-    const int kt = min(NWV * t + wave, a.NP - 1);
+    const int kt = min(KT0 + NWV * t + wave, a.NP - 1);
     const T* p = bias_lane + ((int64_t)min(jt, a.NP - 1) * a.NP + kt) * 1024;
     dst[0] = *reinterpret_cast<const u32x4v*>(p);
     dst[1] = *reinterpret_cast<const u32x4v*>(p + 512);
@@ -379,7 +402,25 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   // key-tile steps they would be spilled, and a reload from scratch waits for every load
   // in flight.
   T* dqrow = reinterpret_cast<T*>(a.dq) + b * a.sdq.b + h * a.sdq.h + i * a.sdq.i;
-  auto reduce_dq = [&](int jt, int buf) {
+  T* lorow = reinterpret_cast<T*>(a.dq_lo) + ((int64_t)bh * N + i) * N * D;  // (several passes only)
+  typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
+  // what the passes before this one left for this lane's elements of query tile jt: fetched at
+  // the start of the query tile, added when its dq is summed
+  struct DqCarry {
+    typename E::vec4 hi[DM], lo[DM];
+  };
+  auto fetch_carry = [&](int jt, DqCarry& cy) {
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const int j = min(32 * jt + (ln & 31), N - 1);
+#pragma unroll
+    for (int mt = 0; mt < DM; ++mt) {
+      const int d0 = min(32 * mt + 8 * wave + 4 * (ln >> 5), D - 4);
+      cy.hi[mt] = *reinterpret_cast<const typename E::vec4*>(dqrow + (int64_t)j * a.sdq.j + d0);
+      cy.lo[mt] = *reinterpret_cast<const typename E::vec4*>(lorow + (int64_t)j * D + d0);
+    }
+  };
+  auto reduce_dq = [&](int jt, int buf, const DqCarry& cy) {
     int ln = lane;
     asm volatile("" : "+v"(ln));
     const int j = 32 * jt + (ln & 31);
@@ -389,13 +430,30 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
       f32x4 acc = *red_slot(buf, 0, mt, wave, ln);
 #pragma unroll
       for (int w = 1; w < NWV; ++w) acc += *red_slot(buf, w, mt, wave, ln);
+      float out[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) out[e] = acc[e] * a.scale;
+      if constexpr (MULTI) {
+        if (!first_pass) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) out[e] += (float)cy.hi[mt][e] + (float)cy.lo[mt][e];
+        }
+      }
       typename E::vec4 ov;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) ov[e] = (T)(acc[e] * a.scale);
+      for (int e = 0; e < 4; ++e) ov[e] = (T)out[e];
       if (d0 < D && j < N) {
-        typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
         T* dst = dqrow + (int64_t)j * a.sdq.j + d0;
         asm volatile("global_store_dwordx2 %0, %1, off" : : "v"(dst), "v"(__builtin_bit_cast(u32x2v, ov)) : "memory");
+        if constexpr (MULTI) {
+          if (!last_pass) {
+            typename E::vec4 lv;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) lv[e] = (T)(out[e] - (float)ov[e]);
+            T* ldst = lorow + (int64_t)j * D + d0;
+            asm volatile("global_store_dwordx2 %0, %1, off" : : "v"(ldst), "v"(__builtin_bit_cast(u32x2v, lv)) : "memory");
+          }
+        }
       }
     }
   };
@@ -437,18 +495,32 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
     };
     fetch_bias(0, 0);
     fetch_bias(0, 1);
+    uint32_t lw_next = 0u, dw_next = 0u;  // several passes: the words of the next query tile
+    if constexpr (MULTI) fetch_words(0, lw_next, dw_next);
+    DqCarry carry;
     int buf = 0;  // jt % 3: the stage of this query tile
     for (int jt = 0; jt < NJ; ++jt) {
       const int buf_fill = buf == 0 ? 2 : buf - 1;  // (jt + 2) % 3: the stage to refill
       if (jt > 0) {
-        if constexpr (NRED == 2) reduce_dq(jt - 1, (jt - 1) & 1);
+        if constexpr (NRED == 2) reduce_dq(jt - 1, (jt - 1) & 1, carry);
+      }
+      if constexpr (MULTI) {
+        if (!first_pass) fetch_carry(jt, carry);
       }
       const unsigned char* qt = tri_smem + OFF_ST + buf * STAGE;
       const unsigned char* dot = qt + 32 * ROWB;
 
       // operand words of this lane's query (lanes 32..63 carry zeros)
       {
-        const uint32_t lw = nl[32 * jt + perm32(kl)], dw = nd[32 * jt + perm32(kl)];
+        uint32_t lw, dw;
+        if constexpr (MULTI) {
+          lw = lw_next;
+          dw = dw_next;
+          fetch_words(jt + 1, lw_next, dw_next);
+        } else {
+          lw = nl[32 * jt + perm32(kl)];
+          dw = nd[32 * jt + perm32(kl)];
+        }
         s_off.set_raw(g ? 0u : lw);
         d_off.v[0] = g ? 0u : dw;
       }
@@ -606,11 +678,11 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
       ring_sync<G2W + (FLAGGED ? 0 : 4)>();
       buf = buf == 2 ? 0 : buf + 1;
       if constexpr (NRED == 1) {
-        reduce_dq(jt, 0);
+        reduce_dq(jt, 0, carry);
         ring_sync<G2W + (FLAGGED ? 0 : 4)>();
       }
     }
-    if constexpr (NRED == 2) reduce_dq(NJ - 1, (NJ - 1) & 1);
+    if constexpr (NRED == 2) reduce_dq(NJ - 1, (NJ - 1) & 1, carry);
 
     // ---- dk, dv of this wave's keys -------------------------------------------------------
     // (the accumulators were last written by MFMAs inside asm statements, which the compiler
@@ -619,7 +691,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
     T* dvrow = reinterpret_cast<T*>(a.dv) + b * a.sdv.b + h * a.sdv.h + i * a.sdv.i;
   #pragma unroll
     for (int t = 0; t < KT; ++t) {
-      const int key = 32 * (NWV * t + wave) + kl;
+      const int key = 32 * (KT0 + NWV * t + wave) + kl;
   #pragma unroll
       for (int mt = 0; mt < DM; ++mt) {
         asm volatile("s_nop 15" : "+a"(dkacc[t][mt]));

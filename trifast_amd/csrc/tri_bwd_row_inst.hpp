@@ -7,7 +7,7 @@
 namespace tri {
 
 // tile index -> key tiles per wave; a workgroup holds rows of up to 128 * KT keys
-constexpr int kRowKT[kBwdRowTiles] = {2, 4, 6, 8};
+constexpr int kRowKT[kBwdRowTiles] = {2, 4, 6, 8, 8};  // (the last one: several passes of 8)
 
 template <typename T, int D, int KT>
 hipError_t bwd_row_run(const BwdArgs& a, int bh, hipStream_t st, bool dry) {
@@ -25,6 +25,35 @@ hipError_t bwd_row_run(const BwdArgs& a, int bh, hipStream_t st, bool dry) {
   }
 }
 
+// Rows of up to kRowMaxPasses * 1024 keys at head dim 32: one launch per 1024 keys (8 key
+// tiles per wave), each complete for dk and dv of its keys and adding its part to dq.
+constexpr int kRowMaxPasses = 4;
+template <typename T, int D>
+hipError_t bwd_row_run_multi(const BwdArgs& a, int bh, hipStream_t st, bool dry) {
+  if constexpr (D == 32) {
+    constexpr int KT = 8;
+    constexpr int lds = bwd_row_lds_bytes(D, (int)sizeof(T), KT, true);
+    const int per_pass = kRowWaves * KT;  // key tiles of one pass
+    const int passes = (a.nwords + per_pass - 1) / per_pass;
+    // (a row that one pass holds is the single-pass tile's)
+    if (a.N <= per_pass * 32 || a.N > kRowMaxPasses * per_pass * 32) return hipErrorInvalidConfiguration;
+    if (dry) return hipSuccess;
+    if (!a.dq_lo) return hipErrorInvalidValue;
+    const int total = bh * a.N;
+    dim3 grid((unsigned)((total + 7) / 8 * 8));
+    for (int p = 0; p < passes; ++p) {
+      BwdArgs ap = a;
+      ap.key_tile0 = p * per_pass;
+      ap.pass_flags = (p > 0 ? 1 : 0) | (p + 1 < passes ? 2 : 0);
+      const hipError_t e = launch_dyn(tri_bwd_row_kernel<T, D, KT, true>, grid, dim3(kRowWaves * 64), lds, st, ap);
+      if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+  } else {
+    return hipErrorInvalidConfiguration;
+  }
+}
+
 template <typename T, int D>
 hipError_t bwd_row_dispatch_kt(const BwdArgs& a, int bh, int tile, hipStream_t st, bool dry) {
   switch (tile) {
@@ -32,6 +61,7 @@ hipError_t bwd_row_dispatch_kt(const BwdArgs& a, int bh, int tile, hipStream_t s
     case 1: return bwd_row_run<T, D, kRowKT[1]>(a, bh, st, dry);
     case 2: return bwd_row_run<T, D, kRowKT[2]>(a, bh, st, dry);
     case 3: return bwd_row_run<T, D, kRowKT[3]>(a, bh, st, dry);
+    case 4: return bwd_row_run_multi<T, D>(a, bh, st, dry);
   }
   return hipErrorInvalidValue;
 }

@@ -344,6 +344,8 @@ int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype)
       // 64-byte rows of 129..1024 keys: the row-resident tile that also produces dq, with as
       // few key tiles per wave as hold the row (ids follow the four streaming tiles)
       if (row_bytes == 64 && dtype != TRIFAST_F32 && n > 128 && n <= 1024) pick = 4 + (int)((n - 1) / 256);
+      // longer rows of head dim 32: the same kernel in passes of 1024 keys
+      if (d == 32 && dtype != TRIFAST_F32 && n > 1024 && n <= 4096) pick = 8;
       break;
     case TRIFAST_KERNEL_BWD_B:  // 128 x 128 block of 16 waves; 8 waves, then 64 x 64 of 4 waves, as rows widen or n shrinks
       pick = (n <= 128 || row_bytes >= 256) ? 2 : (row_bytes == 128 ? 3 : 4);
@@ -369,12 +371,20 @@ int64_t trifast_fwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, 
   return ws_mask_bytes(b, n) + ws_pack_bytes(b, h, n, dtype);
 }
 
-int64_t trifast_bwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype) {
-  (void)d;
-  if (b < 1 || h < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
+// The tail of the backward workspace serves two kernels that run one after the other: the
+// low parts of dq between the passes of the row-resident kernel over a long row (where a tile
+// of that kind supports the shape), then the db partials of the row chunks.
+static int64_t ws_tail_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype) {
   const int64_t chunks = tri::bwd_b_chunks(n, b * h);
-  return ws_mask_bytes(b, n) + 2 * ws_pack_bytes(b, h, n, dtype) + 2 * align256(b * h * n * n * 4) +
-         (chunks > 1 ? align256(chunks * b * h * n * n * 4) : 0);
+  const int64_t parts = chunks > 1 ? align256(chunks * b * h * n * n * 4) : 0;
+  const bool passes = tri::head_dim_ok((int)d) && tri::bwd_kv_supports(tri::bwd_kv_num_tiles() - 1, n, (int)d, dtype);
+  const int64_t lo = passes ? align256(b * h * n * n * d * elem_size(dtype)) : 0;
+  return parts > lo ? parts : lo;
+}
+
+int64_t trifast_bwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype) {
+  if (b < 1 || h < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
+  return ws_mask_bytes(b, n) + 2 * ws_pack_bytes(b, h, n, dtype) + 2 * align256(b * h * n * n * 4) + ws_tail_bytes(b, h, n, d, dtype);
 }
 
 // Forward with the workspace either given by the caller or (use_static) taken from the
@@ -518,6 +528,8 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   a.nchunks = tri::bwd_b_chunks(n, b * h);
   a.rows_per_chunk = (int)((n + a.nchunks - 1) / a.nchunks);
   a.dq = dq; a.dk = dk; a.dv = dv; a.db = db;
+  a.key_tile0 = 0; a.pass_flags = 0;
+  a.dq_lo = w.dbpart;  // (shared with the db partials, which are written after the last pass has read it)
   a.sq = str5(q_strides); a.sk = str5(k_strides); a.sv = str5(v_strides); a.sdo = str5(do_strides);
   a.sdq = str5(dq_strides); a.sdk = str5(dk_strides); a.sdv = str5(dv_strides);
   a.sdb_b = db_strides[0]; a.sdb_h = db_strides[1]; a.sdb_j = db_strides[2]; a.sdb_k = db_strides[3];
