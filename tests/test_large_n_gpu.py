@@ -101,8 +101,9 @@ def test_bias_gradient_with_few_head_groups(n, h):
     orc.compare_values(bias.grad[0], db_pt, db_ref, f"n={n} h={h} db", eps=orc.DTYPE_EPS[dtype])
 
 
-@pytest.mark.parametrize("n,h,dtype", [(1030, 2, torch.bfloat16), (2048, 1, torch.bfloat16), (1500, 1, torch.float16), (2100, 1, torch.bfloat16)],
-                         ids=["n1030_two_passes_ragged", "n2048_two_passes", "n1500_f16", "n2100_three_passes"])
+# (the last pass runs with 2, 8, 4, 6, 2 and 2 key tiles per wave)
+@pytest.mark.parametrize("n,h,dtype", [(1030, 2, torch.bfloat16), (2048, 1, torch.bfloat16), (1500, 1, torch.float16), (1700, 1, torch.bfloat16), (2100, 1, torch.bfloat16), (4200, 1, torch.bfloat16)],
+                         ids=["n1030_two_passes_ragged", "n2048_two_passes", "n1500_f16", "n1700", "n2100_three_passes", "n4200_five_passes"])
 def test_row_resident_backward_in_several_passes(n, h, dtype, monkeypatch):
     """Rows longer than the row-resident kernel holds at once run it once per 1024 keys: dk, dv
     of each pass's keys and the dq summed over the passes are checked on a few pair rows, among

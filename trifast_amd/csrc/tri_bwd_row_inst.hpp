@@ -26,26 +26,35 @@ hipError_t bwd_row_run(const BwdArgs& a, int bh, hipStream_t st, bool dry) {
 }
 
 // Rows of up to kRowMaxPasses * 1024 keys at head dim 32: one launch per 1024 keys (8 key
-// tiles per wave), each complete for dk and dv of its keys and adding its part to dq.
-constexpr int kRowMaxPasses = 4;
+// tiles per wave), each complete for dk and dv of its keys and adding its part to dq; the
+// last pass runs with as few key tiles per wave as hold what is left of the row.
+constexpr int kRowMaxPasses = 8;
+template <typename T, int D, int KT>
+hipError_t bwd_row_pass(const BwdArgs& ap, int bh, hipStream_t st) {
+  constexpr int lds = bwd_row_lds_bytes(D, (int)sizeof(T), KT, true);
+  const int total = bh * ap.N;
+  dim3 grid((unsigned)((total + 7) / 8 * 8));
+  return launch_dyn(tri_bwd_row_kernel<T, D, KT, true>, grid, dim3(kRowWaves * 64), lds, st, ap);
+}
 template <typename T, int D>
 hipError_t bwd_row_run_multi(const BwdArgs& a, int bh, hipStream_t st, bool dry) {
   if constexpr (D == 32) {
-    constexpr int KT = 8;
-    constexpr int lds = bwd_row_lds_bytes(D, (int)sizeof(T), KT, true);
-    const int per_pass = kRowWaves * KT;  // key tiles of one pass
-    const int passes = (a.nwords + per_pass - 1) / per_pass;
+    constexpr int per_pass = kRowWaves * 8;  // key tiles of a full pass
     // (a row that one pass holds is the single-pass tile's)
     if (a.N <= per_pass * 32 || a.N > kRowMaxPasses * per_pass * 32) return hipErrorInvalidConfiguration;
     if (dry) return hipSuccess;
     if (!a.dq_lo) return hipErrorInvalidValue;
-    const int total = bh * a.N;
-    dim3 grid((unsigned)((total + 7) / 8 * 8));
+    const int passes = (a.nwords + per_pass - 1) / per_pass;
     for (int p = 0; p < passes; ++p) {
       BwdArgs ap = a;
       ap.key_tile0 = p * per_pass;
       ap.pass_flags = (p > 0 ? 1 : 0) | (p + 1 < passes ? 2 : 0);
-      const hipError_t e = launch_dyn(tri_bwd_row_kernel<T, D, KT, true>, grid, dim3(kRowWaves * 64), lds, st, ap);
+      const int left = a.nwords - p * per_pass;  // key tiles from this pass on
+      hipError_t e;
+      if (left <= 2 * kRowWaves) e = bwd_row_pass<T, D, 2>(ap, bh, st);
+      else if (left <= 4 * kRowWaves) e = bwd_row_pass<T, D, 4>(ap, bh, st);
+      else if (left <= 6 * kRowWaves) e = bwd_row_pass<T, D, 6>(ap, bh, st);
+      else e = bwd_row_pass<T, D, 8>(ap, bh, st);
       if (e != hipSuccess) return e;
     }
     return hipSuccess;
