@@ -96,7 +96,11 @@ int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype)
  */
 int trifast_bwd_kv_tile_writes_dq(int tile);
 
-/* Bytes of caller-provided workspace (256-byte aligned) each call needs. */
+/* Bytes of caller-provided workspace (256-byte aligned) each call needs: O(b h n^2); the
+ * backward's is b h n^2 (12 + 4 chunks) bytes for 16-bit inputs (chunks of pair rows of the
+ * bias gradient, at most 8) or, for rows of 1025..8192 keys at head dim 32, b h n^2 (12 + 2 d)
+ * (the row-resident kernel then keeps dq between its passes over the keys as two 16-bit
+ * numbers per value, the second of them in the workspace). */
 int64_t trifast_fwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype);
 int64_t trifast_bwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype);
 
