@@ -183,6 +183,18 @@ int trifast_bwd_one(int kernel,
                     int tile, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * Weight gradient of a linear layer over a pair representation: dw[n, k] = sum over r of
+ * dy[r, n] x[r, k] for x [rows, k], dy [rows, n], dw [n, k], all dense, of one 16-bit dtype,
+ * rows = b n^2 in the millions and k in {32, 64, 128, 256}: the rows are split over
+ * workgroups, whose fp32 partials (the workspace) are added in a fixed order.  No counterpart
+ * in the reference, whose callers are only hinted at by the module of
+ * tests/unit/test_trifast.py:152-169 (its q, k, v, bias linear layers, trained in :172-210).
+ */
+int64_t trifast_linear_dw_workspace_bytes(int64_t rows, int64_t k, int64_t n);
+int trifast_linear_dw(void* dw, const void* dy, const void* x, int64_t rows, int64_t k, int64_t n, int dtype,
+                      void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * Output gating of a triangle-attention block, fused with the layout change between the
  * operator and the block's output projection.  No counterpart in the reference (its callers
  * are only hinted at by the module of reference tests/unit/test_trifast.py:152-169): this is

@@ -124,6 +124,23 @@ def test_gate_argument_errors_come_back_as_codes():
     assert lib.trifast_gate_bwd(ok, ok, ok, ok, ok, 1, 2, 8, 32, 7, None) < 0
 
 
+def test_weight_gradient_argument_errors_come_back_as_codes():
+    lib = _lib.load()
+    ok = 0x1000
+    call = lambda dw, dy, x, rows, k, n, dtype=_lib.BF16, ws=ok, nbytes=1 << 40: lib.trifast_linear_dw(dw, dy, x, rows, k, n, dtype, ws, nbytes, None)
+    assert call(ok, ok, ok, 100, 48, 8) == -2 and "input channels" in _lib.last_error()
+    assert call(ok, ok, ok, 100, 64, 8, _lib.F32) == -2 and "16-bit" in _lib.last_error()
+    assert call(ok, ok, ok, 0, 64, 8) == -1 and "positive" in _lib.last_error()
+    assert call(None, ok, ok, 100, 64, 8) == -1 and "null" in _lib.last_error()
+    assert call(ok, ok + 8, ok, 100, 64, 8) == -3 and "aligned" in _lib.last_error()
+    assert call(ok, ok, ok, 100, 64, 8, nbytes=16) == -4 and "workspace" in _lib.last_error()
+    # the partials: one [n, k] fp32 matrix per chunk of rows, at most 1024 chunks
+    assert lib.trifast_linear_dw_workspace_bytes(1024, 128, 128) == 128 * 128 * 4
+    assert lib.trifast_linear_dw_workspace_bytes(1 << 20, 128, 128) == 1024 * 128 * 128 * 4
+    assert lib.trifast_linear_dw_workspace_bytes(1 << 24, 128, 4) <= 1024 * 128 * 4 * 4
+    assert lib.trifast_linear_dw_workspace_bytes(0, 128, 4) < 0
+
+
 def test_gated_output_checks_shapes_on_the_host():
     import torch
 
@@ -138,6 +155,8 @@ def test_gated_output_checks_shapes_on_the_host():
         nn.gated_output(o, torch.zeros(1, 8, 8, 32))
     block = nn.TriangleAttention(24, 2, 16, ending_node=True)
     assert block.heads(torch.zeros(3, 8, 8, 32)).shape == (3, 2, 8, 8, 16)
+    # linear layers over CPU tensors are torch's own
+    assert nn.linear(torch.zeros(2, 24), block.b).shape == (2, 2)
     assert {n for n, _ in block.named_parameters()} == {"q.weight", "k.weight", "v.weight", "b.weight", "g.weight", "g.bias", "out.weight", "out.bias"}
 
 

@@ -132,3 +132,58 @@ def test_block_trains():
         opt.step()
     for k, p in model.named_parameters():
         assert torch.isfinite(p).all() and not torch.equal(before[k], p), k
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("rows,k,n", [(33 * 31, 128, 128), (5, 32, 6), (70000, 64, 4), (4099, 256, 260), (2 * 2048 + 1, 128, 36)])
+def test_weight_gradient_against_float64(dtype, rows, k, n):
+    """dy^T x with the rows split over workgroups: ragged row counts (the last chunk and its last
+    32-row step are partial), output rows that are not a multiple of 8 or of 32, more than one
+    group of 128 output rows, every compiled k."""
+    gen = torch.Generator().manual_seed(rows + n)
+    x = torch.randn(rows, k, generator=gen).to(DEV, dtype)
+    dy = torch.randn(rows, n, generator=gen).to(DEV, dtype)
+    got = nn.linear_weight_grad(dy, x)
+    assert got.shape == (n, k) and got.dtype == dtype
+    want = dy.double().t() @ x.double()
+    size = dy.double().abs().t() @ x.double().abs()
+    # fp32 accumulation of exact products in a fixed order, one rounding to the dtype
+    bound = 0.5 * torch.finfo(dtype).eps * want.abs() + max(rows, 64) ** 0.5 * 2.0**-22 * size + torch.finfo(dtype).smallest_normal
+    err = (got.double() - want).abs()
+    assert bool((err <= bound).all()), f"max excess {(err - bound).max().item():.3e}"
+    assert torch.equal(got, nn.linear_weight_grad(dy, x)), "two runs differ"
+
+
+def test_linear_gradients_are_those_of_the_layer():
+    torch.manual_seed(5)
+    dtype = torch.bfloat16
+    x = torch.randn(3, 50, 50, 64, device=DEV, dtype=dtype)
+    for n, wb in ((64, False), (4, False), (32, True)):
+        m = torch.nn.Linear(64, n, bias=wb).to(DEV, dtype)
+        dy = torch.randn(3, 50, 50, n, device=DEV, dtype=dtype)
+
+        def grads(fn):
+            xi = x.clone().requires_grad_(True)
+            m.zero_grad()
+            y = fn(xi)
+            y.backward(dy)
+            return [y.detach().float(), xi.grad.float()] + [p.grad.float().clone() for p in m.parameters()]
+
+        got = grads(lambda xi: nn.linear(xi, m))
+        want = grads(m)
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])  # the same library products
+        for a, r in zip(got[2:], want[2:]):
+            assert a.shape == r.shape
+            # the same products, summed in another order and rounded to bf16 once
+            assert (a - r).abs().max().item() <= 2.0**-7 * r.abs().max().item(), f"{(a - r).abs().max().item():.3e} of {r.abs().max().item():.3e}"
+
+
+def test_linear_falls_back_to_torch_where_the_kernel_has_no_instance():
+    x = torch.randn(10, 48, device=DEV, dtype=torch.bfloat16, requires_grad=True)  # 48 input channels are not compiled
+    m = torch.nn.Linear(48, 8).to(DEV, torch.bfloat16)
+    assert not nn._dw_ready(x, m.weight)
+    nn.linear(x, m).sum().backward()
+    assert m.weight.grad is not None and x.grad is not None
+    x32 = torch.randn(10, 64, device=DEV)
+    m32 = torch.nn.Linear(64, 8).to(DEV)
+    assert torch.equal(nn.linear(x32, m32), m32(x32))

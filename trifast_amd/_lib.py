@@ -65,6 +65,8 @@ SIGNATURES = {
          _I64P, _I64P, _I64P, _I64P,
          c_int, c_void_p, c_int64, c_void_p],
     ),
+    "trifast_linear_dw_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64]),
+    "trifast_linear_dw": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p]),
     "trifast_gate_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "trifast_gate_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
 }

@@ -13,6 +13,7 @@
 #include "tri_common.hpp"
 #include "tri_launch.hpp"
 #include "tri_gate.hpp"
+#include "tri_linear.hpp"
 
 namespace tri {
 
@@ -604,6 +605,31 @@ int gate_impl(bool bwd, void* y_or_dg, void* dox, const void* dy, const void* o,
   return 0;
 }
 }  // namespace
+
+int64_t trifast_linear_dw_workspace_bytes(int64_t rows, int64_t k, int64_t n) {
+  if (rows < 1 || k < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
+  return align256(tri::linear_dw_chunks(rows) * n * k * 4);
+}
+
+int trifast_linear_dw(void* dw, const void* dy, const void* x, int64_t rows, int64_t k, int64_t n, int dtype,
+                      void* workspace, int64_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  if (dtype != TRIFAST_BF16 && dtype != TRIFAST_F16) return fail(TRIFAST_EUNSUPPORTED, "linear_dw: 16-bit element types only (dtype code %d)", dtype);
+  if (rows < 1 || n < 1 || n > 65535 * 128) return fail(TRIFAST_EINVAL, "linear_dw: rows and n must be positive (rows=%lld n=%lld)", (long long)rows, (long long)n);
+  if (!tri::linear_dw_k_ok(k)) return fail(TRIFAST_EUNSUPPORTED, "linear_dw: %lld input channels (32, 64, 128 or 256 are compiled)", (long long)k);
+  if (!dw || !dy || !x) return fail(TRIFAST_EINVAL, "linear_dw: null pointer argument");
+  if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(dy) & 15) != 0)
+    return fail(TRIFAST_EALIGN, "linear_dw: x and dy must be 16-byte aligned");
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 || workspace_bytes < trifast_linear_dw_workspace_bytes(rows, k, n))
+    return fail(TRIFAST_EWORKSPACE, "linear_dw: workspace missing, misaligned or smaller than trifast_linear_dw_workspace_bytes");
+  tri::LinearDwArgs a{};
+  a.x = x; a.dy = dy; a.dw = dw; a.part = static_cast<float*>(workspace);
+  a.rows = rows; a.rows_per_chunk = tri::linear_dw_rows_per_chunk(rows); a.chunks = (int)tri::linear_dw_chunks(rows);
+  a.K = (int)k; a.N = (int)n;
+  const hipError_t e = tri::linear_dw_launch(a, dtype, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "linear_dw launch");
+  return 0;
+}
 
 int trifast_gate_fwd(void* y, const void* o, const void* g, int64_t b, int64_t h, int64_t n, int64_t d, int dtype, void* stream) {
   return gate_impl(false, y, nullptr, nullptr, o, g, b, h, n, d, dtype, stream);

@@ -1,0 +1,214 @@
+// Weight gradient of a linear layer over a pair representation,
+//   dW[n, k] = sum over r of dY[r, n] * x[r, k]        x [rows, K], dY [rows, N], dW [N, K]
+// for the tall, narrow shapes a triangle-attention block has: rows = b n^2 in the millions,
+// K and N a few hundred at most.  The contraction runs over the long dimension and the
+// result is tiny, which is the one shape of the block's six linear layers that a BLAS library
+// serves badly (one or two workgroups walk all the rows: 1.7 ms per layer at rows = 2^20,
+// K = N = 128, against 0.15 ms for the layer's other two products).  Here the rows are
+// split into chunks, one workgroup per (chunk, group of 128 output rows n): it streams its
+// rows of dY and x through LDS 32 at a time (both operands have the contraction index as
+// their memory row, so both are read back transposed, ds_read_tr), keeps its part of dW in
+// fp32 accumulators (wave w: rows n of its 32-block, all K columns), and writes it as an fp32
+// partial; a second kernel adds the partials in a fixed order (deterministic, no atomics)
+// and rounds once.  Bound by HBM: every element of dY and x is read once per group of n.
+// No counterpart in the reference: the linear layers around its operator are only hinted
+// at by the module of reference tests/unit/test_trifast.py:152-169.
+#pragma once
+#include <type_traits>
+
+#include "tri_common.hpp"
+
+namespace tri {
+
+struct LinearDwArgs {
+  const void* x;    // [rows, K]
+  const void* dy;   // [rows, N]
+  float* part;      // [chunks, N, K] partial sums
+  void* dw;         // [N, K]
+  int64_t rows;
+  int64_t rows_per_chunk;  // multiple of 32
+  int chunks;
+  int K, N;
+};
+
+constexpr int kLinearRowsPerStep = 32;
+
+// rows of one chunk: enough chunks to fill the GPU several times, few enough that the
+// partials stay small (at most 1024)
+inline int64_t linear_dw_rows_per_chunk(int64_t rows) {
+  int64_t per = 1024;
+  while ((rows + per - 1) / per > 1024) per *= 2;
+  return per;
+}
+inline int64_t linear_dw_chunks(int64_t rows) {
+  const int64_t per = linear_dw_rows_per_chunk(rows);
+  return (rows + per - 1) / per;
+}
+
+// KD: columns of x (K, one of 32, 64, 128, 256); the group of output rows is 128 wide
+template <typename T, int KD>
+__global__ __launch_bounds__(256) void linear_dw_kernel(const LinearDwArgs a) {
+  using E = Elem<T>;
+  using frag = typename E::frag;
+  using vec = typename E::vec;
+  constexpr int ND = 128;                // output rows n per workgroup
+  constexpr int KB = KD / 32;            // 32-column blocks of x
+  constexpr int LDX = KD + 8, LDY = ND + 8;  // padded rows (16-byte multiples)
+  constexpr int XCH = 32 * KD / 8, YCH = 32 * ND / 8;          // 16-byte chunks of a step's tiles
+  constexpr int XC = (XCH + 255) / 256, YC = (YCH + 255) / 256;  // ... per lane
+  __shared__ __attribute__((aligned(16))) T xs[2][32][LDX];
+  __shared__ __attribute__((aligned(16))) T ys[2][32][LDY];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = lane >> 5;
+  const int K = KD, N = a.N;
+  const int n_grp = blockIdx.y * ND;  // first output row of this workgroup
+  const int64_t r_begin = (int64_t)blockIdx.x * a.rows_per_chunk;
+  const int64_t r_end = min(a.rows, r_begin + a.rows_per_chunk);
+  const int steps = (int)((r_end - r_begin + 31) / 32);
+  const T* xg = reinterpret_cast<const T*>(a.x);
+  const T* yg = reinterpret_cast<const T*>(a.dy);
+  const bool y_vec = (N % 8) == 0;  // rows of dY keep 16-byte alignment
+
+  // this lane's chunks of a step's tiles (tile row, first column), fetched two steps ahead of
+  // their use: one set of registers per step in flight
+  vec xr2[2][XC], yr2[2][YC];
+  auto load_step = [&](int s, vec* xr, vec* yr) {
+    const int64_t r0 = r_begin + 32 * (int64_t)s;
+#pragma unroll
+    for (int c = 0; c < XC; ++c) {
+      const int p = c * 256 + tid, r = p / (KD / 8), col = 8 * (p % (KD / 8));
+      vec v = {};
+      if (p < XCH && r0 + r < r_end) v = *reinterpret_cast<const vec*>(xg + (r0 + r) * K + col);
+      xr[c] = v;
+    }
+#pragma unroll
+    for (int c = 0; c < YC; ++c) {
+      const int p = c * 256 + tid, r = p / (ND / 8), col = n_grp + 8 * (p % (ND / 8));
+      vec v = {};
+      if (r0 + r < r_end && col < N) {
+        const T* src = yg + (r0 + r) * N + col;
+        if (y_vec) {
+          v = *reinterpret_cast<const vec*>(src);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (col + e < N) v[e] = src[e];
+        }
+      }
+      yr[c] = v;
+    }
+  };
+  auto store_step = [&](int buf, const vec* xr, const vec* yr) {
+#pragma unroll
+    for (int c = 0; c < XC; ++c) {
+      const int p = c * 256 + tid, r = p / (KD / 8), col = 8 * (p % (KD / 8));
+      if (p < XCH) *reinterpret_cast<vec*>(&xs[buf][r][col]) = xr[c];
+    }
+#pragma unroll
+    for (int c = 0; c < YC; ++c) {
+      const int p = c * 256 + tid, r = p / (ND / 8), col = 8 * (p % (ND / 8));
+      *reinterpret_cast<vec*>(&ys[buf][r][col]) = yr[c];
+    }
+  };
+
+  f32x16 acc[KB];
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb) acc[kb] = zero16();
+  // (a wave whose 32 output rows lie past N has nothing to compute; it still stages)
+  const bool wave_live = __builtin_amdgcn_readfirstlane((int)(n_grp + 32 * wave < N)) != 0;
+
+  load_step(0, xr2[0], yr2[0]);
+  if (steps > 1) load_step(1, xr2[1], yr2[1]);
+  store_step(0, xr2[0], yr2[0]);
+  __syncthreads();
+  auto one_step = [&](int s, auto parity) __attribute__((always_inline)) {
+    constexpr int buf = decltype(parity)::value;  // s % 2: the LDS buffer of step s, the register set of step s + 2
+    if (s + 2 < steps) load_step(s + 2, xr2[buf], yr2[buf]);
+    if (wave_live) {
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        // A: dY^T (output row n in the lane, 8 memory rows as contraction slots); B: x^T
+        const frag af = lds_tr_frag<T, LDY>(ys[buf], 16 * s2 + 8 * g, 32 * wave, lane);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          const frag bf = lds_tr_frag<T, LDX>(xs[buf], 16 * s2 + 8 * g, 32 * kb, lane);
+          acc[kb] = E::mfma(af, bf, acc[kb]);
+        }
+      }
+    }
+    // the other buffer was last read in step s - 1, which every wave left before the
+    // barrier that ended it
+    if (s + 1 < steps) store_step(buf ^ 1, xr2[buf ^ 1], yr2[buf ^ 1]);
+    __syncthreads();
+  };
+  for (int s = 0; s < steps; s += 2) {
+    one_step(s, std::integral_constant<int, 0>{});
+    if (s + 1 < steps) one_step(s + 1, std::integral_constant<int, 1>{});
+  }
+  if (!wave_live) return;
+  // partial [chunk][n][k]: the lane holds column k = 32 kb + lane % 32 and rows
+  // n = 32 wave + 8 q + 4 g + e of the group
+  float* part = a.part + (int64_t)blockIdx.x * N * K;
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int n = n_grp + 32 * wave + 8 * (v / 4) + 4 * g + (v % 4);
+      if (n < N) part[(int64_t)n * K + 32 * kb + (lane & 31)] = acc[kb][v];
+    }
+}
+
+// dW = sum of the partials, rounded once.  A workgroup sums 32 elements: lane group c of 8
+// adds the chunks c, c + 8, ... in increasing order, then the 8 sums are added in order of c
+// (one fixed association, whatever the timing).
+template <typename T>
+__global__ __launch_bounds__(256) void linear_dw_reduce_kernel(const LinearDwArgs a) {
+  __shared__ float sums[8][32];
+  const int64_t count = (int64_t)a.N * a.K;
+  const int e = threadIdx.x & 31, c0 = threadIdx.x >> 5;
+  const int64_t idx = (int64_t)blockIdx.x * 32 + e;
+  float sum = 0.f;
+  if (idx < count) {
+#pragma unroll 4
+    for (int c = c0; c < a.chunks; c += 8) sum += a.part[(int64_t)c * count + idx];
+  }
+  sums[c0][e] = sum;
+  __syncthreads();
+  if (c0 == 0 && idx < count) {
+    float total = sums[0][e];
+#pragma unroll
+    for (int c = 1; c < 8; ++c) total += sums[c][e];
+    reinterpret_cast<T*>(a.dw)[idx] = (T)total;
+  }
+}
+
+inline bool linear_dw_k_ok(int64_t k) { return k == 32 || k == 64 || k == 128 || k == 256; }
+
+template <typename T>
+inline hipError_t linear_dw_launch_t(const LinearDwArgs& a, hipStream_t st) {
+  const dim3 grid((unsigned)a.chunks, (unsigned)((a.N + 127) / 128)), block(256);
+  switch (a.K) {
+    case 32: hipLaunchKernelGGL((linear_dw_kernel<T, 32>), grid, block, 0, st, a); break;
+    case 64: hipLaunchKernelGGL((linear_dw_kernel<T, 64>), grid, block, 0, st, a); break;
+    case 128: hipLaunchKernelGGL((linear_dw_kernel<T, 128>), grid, block, 0, st, a); break;
+    case 256: hipLaunchKernelGGL((linear_dw_kernel<T, 256>), grid, block, 0, st, a); break;
+    default: return hipErrorInvalidConfiguration;
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  const int64_t count = (int64_t)a.N * a.K;
+  hipLaunchKernelGGL((linear_dw_reduce_kernel<T>), dim3((unsigned)((count + 31) / 32)), block, 0, st, a);
+  return hipGetLastError();
+}
+
+inline hipError_t linear_dw_launch(const LinearDwArgs& a, int dtype, hipStream_t st) {
+  switch (dtype) {
+    case kBF16: return linear_dw_launch_t<__bf16>(a, st);
+    case kF16: return linear_dw_launch_t<_Float16>(a, st);
+  }
+  return hipErrorInvalidConfiguration;
+}
+
+}  // namespace tri

@@ -10,6 +10,10 @@ tensor is copied to change its layout:
   as a ``[*, h, n, n]`` view of ``[*, n, n, h]``.  The operator reads them through their
   strides and writes dq, dk, dv, db with the same strides, so autograd needs no re-layout
   copy on the way back either.
+* The weight gradients of the six linear layers come from ``trifast_linear_dw``: for rows in
+  the millions and a few hundred channels the BLAS library runs that product (a contraction
+  over all rows into a tiny matrix) on one or two workgroups, ten times slower than the
+  layer's other two products.
 * The output gate ``o * sigmoid(g)`` and the layout change from the operator's
   ``[*, h, n, n, d]`` to the ``[*, n, n, h*d]`` that the output projection consumes are one
   streaming HIP kernel (``trifast_gate_fwd`` / ``trifast_gate_bwd``).
@@ -74,6 +78,61 @@ def gated_output(o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
     return _GatedOutput.apply(o, g)
 
 
+_DW_K = (32, 64, 128, 256)
+
+
+def _dw_ready(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Shapes and types the weight-gradient kernel takes; anything else is torch's product."""
+    return x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and weight.dtype == x.dtype and x.shape[-1] in _DW_K and x.numel() > 0
+
+
+def linear_weight_grad(dy: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """``dy^T x`` for ``dy [rows, n]``, ``x [rows, k]``: the weight gradient of a linear layer, with
+    the long contraction over the rows split over the whole GPU (``trifast_linear_dw``)."""
+    dy, x = dy.contiguous(), x.contiguous()
+    rows, n = dy.shape
+    k = x.shape[1]
+    lib = _lib.load()
+    dw = torch.empty(n, k, dtype=x.dtype, device=x.device)
+    ws = torch.empty(lib.trifast_linear_dw_workspace_bytes(rows, k, n), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.trifast_linear_dw(dw.data_ptr(), dy.data_ptr(), x.data_ptr(), rows, k, n, _dtype_code(x), ws.data_ptr(), ws.numel(),
+                                   torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, "trifast_linear_dw")
+    return dw
+
+
+class _Linear(torch.autograd.Function):
+    """``linear(x, weight, bias)`` whose weight gradient comes from ``trifast_linear_dw``; the
+    forward and the input gradient are the BLAS library's products, which run at memory speed
+    for these shapes."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        return torch.nn.functional.linear(x, weight, bias)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight = ctx.saved_tensors
+        dy2 = dy.reshape(-1, dy.shape[-1])
+        dx = (dy2 @ weight).view(x.shape) if ctx.needs_input_grad[0] else None
+        dw = linear_weight_grad(dy2, x.reshape(-1, x.shape[-1])) if ctx.needs_input_grad[1] else None
+        db = dy2.sum(0) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        return dx, dw, db
+
+
+def linear(x: torch.Tensor, layer: torch.nn.Linear) -> torch.Tensor:
+    """``layer(x)`` for a linear layer over a pair representation ``x [*, k]``; on the GPU, for
+    16-bit tensors with k in (32, 64, 128, 256), its weight gradient is computed by this
+    library's kernel (the BLAS library runs that one product, a contraction over millions of
+    rows into a tiny result, on one or two workgroups)."""
+    if not _dw_ready(x, layer.weight):
+        return layer(x)
+    return _Linear.apply(x, layer.weight, layer.bias)
+
+
 class TriangleAttention(torch.nn.Module):
     """Gated triangle self-attention around the starting node (``ending_node=False``) or the
     ending node of a pair representation ``x [*, n, n, c_in]``; ``mask [*, n, n]`` is True
@@ -94,8 +153,8 @@ class TriangleAttention(torch.nn.Module):
         return t.unflatten(-1, (self.h, self.d)).movedim(-2, -4)
 
     def forward(self, x: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
-        q, k, v = self.heads(self.q(x)), self.heads(self.k(x)), self.heads(self.v(x))
-        bias = self.b(x).movedim(-1, -3)
+        q, k, v = self.heads(linear(x, self.q)), self.heads(linear(x, self.k)), self.heads(linear(x, self.v))
+        bias = linear(x, self.b).movedim(-1, -3)
         attend = triangle_attention_ending_node if self.ending_node else triangle_attention
         o = attend(q, k, v, bias, mask)
-        return self.out(gated_output(o, self.g(x)))
+        return linear(gated_output(o, linear(x, self.g)), self.out)

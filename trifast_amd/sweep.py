@@ -16,9 +16,9 @@ reference's tables are other implementations.
 
 ``block`` has no counterpart in the reference: it times the gated block of
 ``trifast_amd.nn`` (projections, operator, gate, output projection; forward + backward)
-against the same block with the layout copies and the unfused gate a caller would write
-in plain PyTorch around the operator, and the gate kernels alone against the HBM bytes
-they must move.
+against the same block with the layout copies, the unfused gate and the linear layers a
+caller would write in plain PyTorch around the operator, and the gate and weight-gradient
+kernels alone against the HBM bytes they must move.
 """
 
 from __future__ import annotations
@@ -148,6 +148,14 @@ def block(n: int, c_in: int) -> None:
     y = nn.gated_output(oo, gg)
     ms = _median_ms(lambda: torch.autograd.grad(y, (oo, gg), gy, retain_graph=True))
     print(f"gate backward {ms * 1e3:8.1f} us  {5 * size / ms / 1e6:7.1f} GB/s of 5 tensors x {size / 2**20:.0f} MiB")
+    x2 = x.detach().reshape(-1, c_in)
+    for n_out in (H * D, H):
+        dy2 = torch.randn(x2.shape[0], n_out, device=dev, dtype=DTYPE)
+        nbytes = (x2.numel() + dy2.numel()) * x2.element_size()
+        ms = _median_ms(lambda: nn.linear_weight_grad(dy2, x2))
+        ms_blas = _median_ms(lambda: dy2.t() @ x2)
+        print(f"weight gradient [{n_out} x {c_in}] over {x2.shape[0]} rows {ms * 1e3:8.1f} us  {nbytes / ms / 1e6:7.1f} GB/s of x and dy "
+              f"({nbytes / 2**20:.0f} MiB); the BLAS library's product {ms_blas * 1e3:8.1f} us")
 
 
 def main() -> None:
