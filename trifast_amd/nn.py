@@ -52,8 +52,9 @@ class _GatedOutput(torch.autograd.Function):
         o, g = o.contiguous(), g.contiguous()
         y = torch.empty_like(g)
         if y.numel():
-            rc = _lib.load().trifast_gate_fwd(y.data_ptr(), o.data_ptr(), g.data_ptr(), b, h, n, d, _dtype_code(o),
-                                              torch.cuda.current_stream(o.device).cuda_stream)
+            with torch.cuda.device(o.device):
+                rc = _lib.load().trifast_gate_fwd(y.data_ptr(), o.data_ptr(), g.data_ptr(), b, h, n, d, _dtype_code(o),
+                                                  torch.cuda.current_stream(o.device).cuda_stream)
             _lib.check(rc, "trifast_gate_fwd")
         ctx.save_for_backward(o, g)
         ctx.dims = (b, h, n, d)
@@ -66,8 +67,9 @@ class _GatedOutput(torch.autograd.Function):
         dy = dy.contiguous()
         do, dg = torch.empty_like(o), torch.empty_like(g)
         if dy.numel():
-            rc = _lib.load().trifast_gate_bwd(do.data_ptr(), dg.data_ptr(), dy.data_ptr(), o.data_ptr(), g.data_ptr(),
-                                              b, h, n, d, _dtype_code(o), torch.cuda.current_stream(o.device).cuda_stream)
+            with torch.cuda.device(o.device):
+                rc = _lib.load().trifast_gate_bwd(do.data_ptr(), dg.data_ptr(), dy.data_ptr(), o.data_ptr(), g.data_ptr(),
+                                                  b, h, n, d, _dtype_code(o), torch.cuda.current_stream(o.device).cuda_stream)
             _lib.check(rc, "trifast_gate_bwd")
         return do, dg
 
