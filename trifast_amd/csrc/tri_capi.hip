@@ -376,7 +376,7 @@ int64_t trifast_fwd_workspace_bytes(int64_t b, int64_t h, int64_t n, int64_t d, 
 // low parts of dq between the passes of the row-resident kernel over a long row (where a tile
 // of that kind supports the shape), then the db partials of the row chunks.
 static int64_t ws_tail_bytes(int64_t b, int64_t h, int64_t n, int64_t d, int dtype) {
-  const int64_t chunks = tri::bwd_b_chunks(n, b * h);
+  const int64_t chunks = tri::bwd_b_chunks(n, b * h, (int)d * elem_size(dtype));
   const int64_t parts = chunks > 1 ? align256(chunks * b * h * n * n * 4) : 0;
   const bool passes = tri::head_dim_ok((int)d) && tri::bwd_kv_supports(tri::bwd_kv_num_tiles() - 1, n, (int)d, dtype);
   const int64_t lo = passes ? align256(b * h * n * n * d * elem_size(dtype)) : 0;
@@ -526,7 +526,7 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   a.lse = lse;
   a.keep = w.keep; a.rowflag = w.rowflag; a.delta = w.delta; a.lse2 = w.lse2; a.dbpart = w.dbpart;
   a.BH = (int)(b * h);
-  a.nchunks = tri::bwd_b_chunks(n, b * h);
+  a.nchunks = tri::bwd_b_chunks(n, b * h, (int)d * elem_size(dtype));
   a.rows_per_chunk = (int)((n + a.nchunks - 1) / a.nchunks);
   a.dq = dq; a.dk = dk; a.dv = dv; a.db = db;
   a.key_tile0 = 0; a.pass_flags = 0;
