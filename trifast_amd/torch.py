@@ -245,6 +245,8 @@ def backwards(ctx, *grad):
     # reference src/trifast/torch.py:185-207
     do = grad[0]
     q, k, v, b, mask, o, l = ctx.saved_tensors
+    if do is None:  # only lse was used downstream: nothing flows back through o
+        do = torch.zeros_like(o)
     dq, dk, dv, db, _ = triangle_attention_bwd(do, q, k, v, b, o, l, mask)
     return dq, dk, dv, db, None
 
@@ -254,6 +256,8 @@ def setup_context(ctx, inputs, output) -> None:
     q, k, v, b, mask, *_ = inputs
     o, l = output
     ctx.save_for_backward(q, k, v, b, mask, o, l)
+    # lse takes no gradient: without this autograd fills a zero tensor of its size for every backward
+    ctx.set_materialize_grads(False)
 
 
 _triangle_attention.register_autograd(backwards, setup_context=setup_context)
