@@ -30,11 +30,24 @@ __global__ __launch_bounds__(64) void mask_prep_kernel(const MaskPrepArgs a) {
   const uint8_t* row = a.mask + b * a.sb + i * a.si;
   uint32_t* out = a.keep + ((int64_t)b * a.n + i) * a.nwords;
   bool any_kept = false;
+  // (contiguous, 16-byte aligned rows: the 32 bytes of a word are two vector loads)
+  const bool vec_rows = a.sk == 1 && (reinterpret_cast<uintptr_t>(row) & 15) == 0;
   for (int w = lane; w < a.nwords; w += 64) {
     uint32_t bits = 0;
-    for (int t = 0; t < 32; ++t) {
-      const int key = 32 * w + t;
-      if (key < a.n && row[key * a.sk] == 0) bits |= 1u << t;
+    if (vec_rows && 32 * w + 32 <= a.n) {
+      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(row + 32 * w + 16 * half);
+#pragma unroll
+        for (int t = 0; t < 16; ++t)
+          if (((v[t / 4] >> (8 * (t % 4))) & 0xffu) == 0) bits |= 1u << (16 * half + t);
+      }
+    } else {
+      for (int t = 0; t < 32; ++t) {
+        const int key = 32 * w + t;
+        if (key < a.n && row[key * a.sk] == 0) bits |= 1u << t;
+      }
     }
     out[w] = bits;
     any_kept |= bits != 0;
@@ -71,13 +84,18 @@ __global__ __launch_bounds__(256) void bias_prep_kernel(const BiasPrepArgs a) {
   const int l32 = lane & 31, g = lane >> 5;
   const T* src = reinterpret_cast<const T*>(a.bias) + b * a.sb + h * a.sh;
   const int64_t out = ((int64_t)bh * a.NP * a.NP * 128 + slot) * 8;
+  typedef T tvec __attribute__((ext_vector_type(8)));
   if (a.packq) {
     T* dst = reinterpret_cast<T*>(a.packq) + out;
     const int j = 32 * jt + l32;
+    const int key0 = 32 * kt + 16 * r + 8 * g;
+    const T* p = src + j * a.sj + key0 * a.sk;
+    // (eight consecutive keys of a row with contiguous keys: one vector load where it is aligned)
+    if (a.sk == 1 && j < a.N && key0 + 8 <= a.N && (reinterpret_cast<uintptr_t>(p) & (sizeof(tvec) - 1)) == 0) {
+      *reinterpret_cast<tvec*>(dst) = *reinterpret_cast<const tvec*>(p);
+    } else {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int key = 32 * kt + 16 * r + 8 * g + e;
-      dst[e] = (j < a.N && key < a.N) ? src[j * a.sj + key * a.sk] : (T)0.f;
+      for (int e = 0; e < 8; ++e) dst[e] = (j < a.N && key0 + e < a.N) ? p[e * a.sk] : (T)0.f;
     }
   }
   if (a.packk) {
