@@ -134,10 +134,11 @@ def test_weight_gradient_argument_errors_come_back_as_codes():
     assert call(None, ok, ok, 100, 64, 8) == -1 and "null" in _lib.last_error()
     assert call(ok, ok + 8, ok, 100, 64, 8) == -3 and "aligned" in _lib.last_error()
     assert call(ok, ok, ok, 100, 64, 8, nbytes=16) == -4 and "workspace" in _lib.last_error()
-    # the partials: one [n, k] fp32 matrix per chunk of rows, at most 1024 chunks
+    # the partials: one [n, k] fp32 matrix per chunk of at least 1024 rows, at most 768 chunks
     assert lib.trifast_linear_dw_workspace_bytes(1024, 128, 128) == 128 * 128 * 4
-    assert lib.trifast_linear_dw_workspace_bytes(1 << 20, 128, 128) == 1024 * 128 * 128 * 4
-    assert lib.trifast_linear_dw_workspace_bytes(1 << 24, 128, 4) <= 1024 * 128 * 4 * 4
+    assert lib.trifast_linear_dw_workspace_bytes(3000, 128, 128) == 3 * 128 * 128 * 4
+    assert 700 * 128 * 128 * 4 <= lib.trifast_linear_dw_workspace_bytes(1 << 20, 128, 128) <= 768 * 128 * 128 * 4
+    assert lib.trifast_linear_dw_workspace_bytes(1 << 24, 128, 4) <= 768 * 128 * 4 * 4
     assert lib.trifast_linear_dw_workspace_bytes(0, 128, 4) < 0
 
 

@@ -135,7 +135,7 @@ def test_block_trains():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
-@pytest.mark.parametrize("rows,k,n", [(33 * 31, 128, 128), (5, 32, 6), (70000, 64, 4), (4099, 256, 260), (2 * 2048 + 1, 128, 36)])
+@pytest.mark.parametrize("rows,k,n", [(33 * 31, 128, 128), (5, 32, 6), (70000, 64, 4), (4099, 256, 260), (2 * 2048 + 1, 128, 36), (5000, 256, 32), (900001, 128, 4)])
 def test_weight_gradient_against_float64(dtype, rows, k, n):
     """dy^T x with the rows split over workgroups: ragged row counts (the last chunk and its last
     32-row step are partial), output rows that are not a multiple of 8 or of 32, more than one

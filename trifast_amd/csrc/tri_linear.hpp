@@ -33,26 +33,29 @@ struct LinearDwArgs {
 
 constexpr int kLinearRowsPerStep = 32;
 
-// rows of one chunk: enough chunks to fill the GPU several times, few enough that the
-// partials stay small (at most 1024)
+// rows of one chunk: at least 1024 (the partials of a chunk cost as much traffic as 128 rows),
+// and at most 768 chunks: three workgroups per CU are resident at once, and a grid that is not
+// a whole number of such rounds leaves CUs idle in the last one
 inline int64_t linear_dw_rows_per_chunk(int64_t rows) {
-  int64_t per = 1024;
-  while ((rows + per - 1) / per > 1024) per *= 2;
-  return per;
+  const int64_t per = ((rows + 767) / 768 + 31) / 32 * 32;
+  return per < 1024 ? 1024 : per;
 }
 inline int64_t linear_dw_chunks(int64_t rows) {
   const int64_t per = linear_dw_rows_per_chunk(rows);
   return (rows + per - 1) / per;
 }
 
-// KD: columns of x (K, one of 32, 64, 128, 256); the group of output rows is 128 wide
-template <typename T, int KD>
+// KD: columns of x (K, one of 32, 64, 128, 256); ND: output rows n per workgroup, 128 (wave w
+// owns rows 32 w .. 32 w + 31 and every column block of x) or, for layers of up to 32 outputs,
+// 32 (the four waves share the column blocks of x)
+template <typename T, int KD, int ND>
 __global__ __launch_bounds__(256) void linear_dw_kernel(const LinearDwArgs a) {
   using E = Elem<T>;
   using frag = typename E::frag;
   using vec = typename E::vec;
-  constexpr int ND = 128;                // output rows n per workgroup
   constexpr int KB = KD / 32;            // 32-column blocks of x
+  constexpr bool SPLIT_K = ND == 32;
+  constexpr int KBW = SPLIT_K ? (KB + 3) / 4 : KB;  // column blocks of one wave
   constexpr int LDX = KD + 8, LDY = ND + 8;  // padded rows (16-byte multiples)
   constexpr int XCH = 32 * KD / 8, YCH = 32 * ND / 8;          // 16-byte chunks of a step's tiles
   constexpr int XC = (XCH + 255) / 256, YC = (YCH + 255) / 256;  // ... per lane
@@ -87,7 +90,7 @@ __global__ __launch_bounds__(256) void linear_dw_kernel(const LinearDwArgs a) {
     for (int c = 0; c < YC; ++c) {
       const int p = c * 256 + tid, r = p / (ND / 8), col = n_grp + 8 * (p % (ND / 8));
       vec v = {};
-      if (r0 + r < r_end && col < N) {
+      if (p < YCH && r0 + r < r_end && col < N) {
         const T* src = yg + (r0 + r) * N + col;
         if (y_vec) {
           v = *reinterpret_cast<const vec*>(src);
@@ -109,15 +112,17 @@ __global__ __launch_bounds__(256) void linear_dw_kernel(const LinearDwArgs a) {
 #pragma unroll
     for (int c = 0; c < YC; ++c) {
       const int p = c * 256 + tid, r = p / (ND / 8), col = 8 * (p % (ND / 8));
-      *reinterpret_cast<vec*>(&ys[buf][r][col]) = yr[c];
+      if (p < YCH) *reinterpret_cast<vec*>(&ys[buf][r][col]) = yr[c];
     }
   };
 
-  f32x16 acc[KB];
+  f32x16 acc[KBW];
 #pragma unroll
-  for (int kb = 0; kb < KB; ++kb) acc[kb] = zero16();
-  // (a wave whose 32 output rows lie past N has nothing to compute; it still stages)
-  const bool wave_live = __builtin_amdgcn_readfirstlane((int)(n_grp + 32 * wave < N)) != 0;
+  for (int i = 0; i < KBW; ++i) acc[i] = zero16();
+  const int n_blk = SPLIT_K ? 0 : wave;                          // this wave's 32 output rows
+  auto col_block = [&](int i) { return SPLIT_K ? wave + 4 * i : i; };  // ... and its column blocks of x
+  // (a wave whose output rows lie past N, or that has no column block, only stages)
+  const bool wave_live = __builtin_amdgcn_readfirstlane((int)(n_grp + 32 * n_blk < N && col_block(0) < KB)) != 0;
 
   load_step(0, xr2[0], yr2[0]);
   if (steps > 1) load_step(1, xr2[1], yr2[1]);
@@ -130,11 +135,13 @@ __global__ __launch_bounds__(256) void linear_dw_kernel(const LinearDwArgs a) {
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         // A: dY^T (output row n in the lane, 8 memory rows as contraction slots); B: x^T
-        const frag af = lds_tr_frag<T, LDY>(ys[buf], 16 * s2 + 8 * g, 32 * wave, lane);
+        const frag af = lds_tr_frag<T, LDY>(ys[buf], 16 * s2 + 8 * g, 32 * n_blk, lane);
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb) {
-          const frag bf = lds_tr_frag<T, LDX>(xs[buf], 16 * s2 + 8 * g, 32 * kb, lane);
-          acc[kb] = E::mfma(af, bf, acc[kb]);
+        for (int i = 0; i < KBW; ++i) {
+          if (col_block(i) < KB) {
+            const frag bf = lds_tr_frag<T, LDX>(xs[buf], 16 * s2 + 8 * g, 32 * col_block(i), lane);
+            acc[i] = E::mfma(af, bf, acc[i]);
+          }
         }
       }
     }
@@ -152,12 +159,14 @@ __global__ __launch_bounds__(256) void linear_dw_kernel(const LinearDwArgs a) {
   // n = 32 wave + 8 q + 4 g + e of the group
   float* part = a.part + (int64_t)blockIdx.x * N * K;
 #pragma unroll
-  for (int kb = 0; kb < KB; ++kb)
+  for (int i = 0; i < KBW; ++i) {
+    if (col_block(i) >= KB) continue;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      const int n = n_grp + 32 * wave + 8 * (v / 4) + 4 * g + (v % 4);
-      if (n < N) part[(int64_t)n * K + 32 * kb + (lane & 31)] = acc[kb][v];
+      const int n = n_grp + 32 * n_blk + 8 * (v / 4) + 4 * g + (v % 4);
+      if (n < N) part[(int64_t)n * K + 32 * col_block(i) + (lane & 31)] = acc[i][v];
     }
+  }
 }
 
 // dW = sum of the partials, rounded once.  A workgroup sums 32 elements: lane group c of 8
@@ -188,13 +197,25 @@ inline bool linear_dw_k_ok(int64_t k) { return k == 32 || k == 64 || k == 128 ||
 
 template <typename T>
 inline hipError_t linear_dw_launch_t(const LinearDwArgs& a, hipStream_t st) {
-  const dim3 grid((unsigned)a.chunks, (unsigned)((a.N + 127) / 128)), block(256);
-  switch (a.K) {
-    case 32: hipLaunchKernelGGL((linear_dw_kernel<T, 32>), grid, block, 0, st, a); break;
-    case 64: hipLaunchKernelGGL((linear_dw_kernel<T, 64>), grid, block, 0, st, a); break;
-    case 128: hipLaunchKernelGGL((linear_dw_kernel<T, 128>), grid, block, 0, st, a); break;
-    case 256: hipLaunchKernelGGL((linear_dw_kernel<T, 256>), grid, block, 0, st, a); break;
-    default: return hipErrorInvalidConfiguration;
+  const dim3 block(256);
+  if (a.N <= 32) {
+    const dim3 grid((unsigned)a.chunks, 1);
+    switch (a.K) {
+      case 32: hipLaunchKernelGGL((linear_dw_kernel<T, 32, 32>), grid, block, 0, st, a); break;
+      case 64: hipLaunchKernelGGL((linear_dw_kernel<T, 64, 32>), grid, block, 0, st, a); break;
+      case 128: hipLaunchKernelGGL((linear_dw_kernel<T, 128, 32>), grid, block, 0, st, a); break;
+      case 256: hipLaunchKernelGGL((linear_dw_kernel<T, 256, 32>), grid, block, 0, st, a); break;
+      default: return hipErrorInvalidConfiguration;
+    }
+  } else {
+    const dim3 grid((unsigned)a.chunks, (unsigned)((a.N + 127) / 128));
+    switch (a.K) {
+      case 32: hipLaunchKernelGGL((linear_dw_kernel<T, 32, 128>), grid, block, 0, st, a); break;
+      case 64: hipLaunchKernelGGL((linear_dw_kernel<T, 64, 128>), grid, block, 0, st, a); break;
+      case 128: hipLaunchKernelGGL((linear_dw_kernel<T, 128, 128>), grid, block, 0, st, a); break;
+      case 256: hipLaunchKernelGGL((linear_dw_kernel<T, 256, 128>), grid, block, 0, st, a); break;
+      default: return hipErrorInvalidConfiguration;
+    }
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
