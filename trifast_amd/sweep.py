@@ -148,6 +148,8 @@ def block(n: int, c_in: int) -> None:
     y = nn.gated_output(oo, gg)
     ms = _median_ms(lambda: torch.autograd.grad(y, (oo, gg), gy, retain_graph=True))
     print(f"gate backward {ms * 1e3:8.1f} us  {5 * size / ms / 1e6:7.1f} GB/s of 5 tensors x {size / 2**20:.0f} MiB")
+    ms = _median_ms(lambda: gy.copy_(g))
+    print(f"(a plain device copy of one such tensor {ms * 1e3:8.1f} us  {2 * size / ms / 1e6:7.1f} GB/s read + written)")
     x2 = x.detach().reshape(-1, c_in)
     for n_out in (H * D, H):
         dy2 = torch.randn(x2.shape[0], n_out, device=dev, dtype=DTYPE)
