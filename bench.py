@@ -398,7 +398,7 @@ def main():
         # the backward as a whole, counted as the five GEMMs it needs (10 b h n^3 d) whatever the
         # kernels recompute, over the launch durations of its kernels
         "bwd_credited": {"ms": bwd_ms, "tflops": f_bwd / bwd_ms / 1e9, "frac_of_peak": f_bwd / bwd_ms / 1e9 / peak},
-        "kernel_ms_include": "mask and bias pre-passes (and the db partial reduce), about 0.02 ms at n=1024",
+        "kernel_ms_include": "mask and bias pre-passes (and the db partial reduce where rows are split), about 0.01 ms at n=1024",
         "roofline": roofline,
         "autotune": tuner.autotune_enabled(),
     }
