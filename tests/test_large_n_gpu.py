@@ -154,3 +154,31 @@ def test_row_resident_backward_in_several_passes(n, h, dtype, monkeypatch):
     assert not dk[0, :, 4, :1024].any() and not dv[0, :, 4, :1024].any()
     # rows without upstream gradient have none to give
     assert not dq[0, :, 1].any() and not dk[0, :, n - 2].any()
+
+
+def test_passes_write_strided_gradients():
+    """The ending-node entry at a row length that needs two passes: q, k, v, dO and the gradients
+    are pair-transposed views there, and dq travels between the passes through the strided dq
+    tensor itself.  The same numbers must come out as from contiguous copies of the views."""
+    n, h, dtype, dev = 1040, 1, torch.bfloat16, "cuda"
+    g = torch.Generator(device=dev).manual_seed(7)
+    q, k, v, do = (torch.randn(1, h, n, n, D, device=dev, dtype=dtype, generator=g) * D**-0.25 for _ in range(4))
+    bias = torch.randn(1, h, n, n, device=dev, dtype=dtype, generator=g)
+    mask = torch.rand(1, n, n, device=dev, generator=g) < 0.1
+
+    def run(fn, *tensors):
+        leaves = [t.detach().clone().requires_grad_(True) for t in tensors]
+        out = fn(*leaves)
+        return out, leaves
+
+    o1, l1 = run(lambda a, b_, c, d_: trifast_amd.triangle_attention_ending_node(a, b_, c, d_, mask), q, k, v, bias)
+    o1.backward(do)
+    t = lambda x: x.transpose(2, 3).contiguous()
+    o2, l2 = run(lambda a, b_, c, d_: trifast_amd.triangle_attention(a, b_, c, d_, mask.transpose(1, 2).contiguous()),
+                 t(q), t(k), t(v), bias.transpose(2, 3).contiguous())
+    o2.backward(t(do))
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2.transpose(2, 3))
+    for name, a, c in zip(("dq", "dk", "dv"), l1[:3], l2[:3]):
+        assert torch.equal(a.grad, c.grad.transpose(2, 3)), name
+    assert torch.equal(l1[3].grad, l2[3].grad.transpose(2, 3)), "db"
