@@ -349,12 +349,17 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   // packed bias tiles of this lane: tile (jt, kt) is 2 x 16 bytes per lane
   typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
   // (as A operand: operand row m stands for query perm32(m), like the Q and dO operands)
-  const T* bias_lane = pack_bh + (perm32(kl) + 32 * g) * 8;
+  // (a tile's address is a wave-uniform base, computed on the scalar unit, plus this lane's
+  // constant 32-bit byte offset: no vector arithmetic per tile)
+  uint32_t bias_lane = (uint32_t)((perm32(kl) + 32 * g) * 8 * sizeof(T));
+  asm volatile("" : "+v"(bias_lane));
   auto bias_load = [&](int jt, int t, u32x4v* dst) {
     const int kt = min(KT0 + NWV * t + wave, a.NP - 1);
-    const T* p = bias_lane + ((int64_t)min(jt, a.NP - 1) * a.NP + kt) * 1024;
-    dst[0] = *reinterpret_cast<const u32x4v*>(p);
-    dst[1] = *reinterpret_cast<const u32x4v*>(p + 512);
+    const char* tile = reinterpret_cast<const char*>(pack_bh + ((int64_t)min(jt, a.NP - 1) * a.NP + kt) * 1024);
+    uint32_t vo = bias_lane;
+    asm volatile("" : "+v"(vo));  // (opaque here: the sum of the lane offset and the head's base is not hoisted as a 64-bit vector)
+    dst[0] = *reinterpret_cast<const u32x4v*>(tile + (uint64_t)vo);
+    dst[1] = *reinterpret_cast<const u32x4v*>(tile + (uint64_t)vo + 512 * sizeof(T));
   };
   const float c = a.c;
 
