@@ -191,6 +191,15 @@ int trifast_bwd_one(int kernel,
  * tests/unit/test_trifast.py:152-169 (its q, k, v, bias linear layers, trained in :172-210).
  */
 int64_t trifast_linear_dw_workspace_bytes(int64_t rows, int64_t k, int64_t n);
+/*
+ * Input gradient of up to 6 linear layers over the same pair representation in one pass:
+ * dx[r, :] = sum over layers p of dy_p[r, :] W_p, with dy_p [rows, n_p] and the weights given
+ * transposed, wt_p = W_p^T [k, n_p] (all dense, one 16-bit dtype, k in {32, 64, 128}); every
+ * dy_p is read once and dx [rows, k] written once.  dy, wt, n are host arrays of nlayers
+ * entries.  No counterpart in the reference (see trifast_linear_dw).
+ */
+int trifast_linear_dx(void* dx, int64_t rows, int64_t k, int nlayers, const void* const* dy, const void* const* wt,
+                      const int64_t* n, int dtype, void* stream);
 int trifast_linear_dw(void* dw, const void* dy, const void* x, int64_t rows, int64_t k, int64_t n, int dtype,
                       void* workspace, int64_t workspace_bytes, void* stream);
 

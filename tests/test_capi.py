@@ -142,6 +142,24 @@ def test_weight_gradient_argument_errors_come_back_as_codes():
     assert lib.trifast_linear_dw_workspace_bytes(0, 128, 4) < 0
 
 
+def test_input_gradient_argument_errors_come_back_as_codes():
+    import ctypes
+
+    lib = _lib.load()
+    ok = 0x1000
+    vp = lambda *v: (ctypes.c_void_p * len(v))(*v)
+    n1 = _lib.i64_array([8])
+    call = lambda dx, k, nl, dy, wt, n, dtype=_lib.BF16, rows=4: lib.trifast_linear_dx(dx, rows, k, nl, dy, wt, n, dtype, None)
+    assert call(ok, 256, 1, vp(ok), vp(ok), n1) == -2 and "input channels" in _lib.last_error()
+    assert call(ok, 64, 1, vp(ok), vp(ok), n1, _lib.F32) == -2 and "16-bit" in _lib.last_error()
+    assert call(ok, 64, 7, vp(*[ok] * 7), vp(*[ok] * 7), _lib.i64_array([8] * 7)) == -1 and "layers per call" in _lib.last_error()
+    assert call(ok + 8, 64, 1, vp(ok), vp(ok), n1) == -3 and "dx is not" in _lib.last_error()
+    assert call(ok, 64, 1, vp(ok), vp(ok + 4), n1) == -3 and "layer 0" in _lib.last_error()
+    assert call(ok, 64, 1, vp(None), vp(ok), n1) == -1 and "null" in _lib.last_error()
+    assert call(ok, 64, 1, vp(ok), vp(ok), _lib.i64_array([0])) == -1 and "outputs" in _lib.last_error()
+    assert call(ok, 64, 1, vp(ok), vp(ok), n1, rows=0) == -1 and "rows" in _lib.last_error()
+
+
 def test_gated_output_checks_shapes_on_the_host():
     import torch
 
@@ -158,6 +176,7 @@ def test_gated_output_checks_shapes_on_the_host():
     assert block.heads(torch.zeros(3, 8, 8, 32)).shape == (3, 2, 8, 8, 16)
     # linear layers over CPU tensors are torch's own
     assert nn.linear(torch.zeros(2, 24), block.b).shape == (2, 2)
+    assert [t.shape for t in nn.project(torch.zeros(2, 24), (block.q, block.b))] == [(2, 32), (2, 2)]
     assert {n for n, _ in block.named_parameters()} == {"q.weight", "k.weight", "v.weight", "b.weight", "g.weight", "g.bias", "out.weight", "out.bias"}
 
 

@@ -187,3 +187,48 @@ def test_linear_falls_back_to_torch_where_the_kernel_has_no_instance():
     x32 = torch.randn(10, 64, device=DEV)
     m32 = torch.nn.Linear(64, 8).to(DEV)
     assert torch.equal(nn.linear(x32, m32), m32(x32))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("rows,k,ns", [(33 * 31, 128, (128, 128, 128, 4, 128)), (5, 32, (6,)), (70001, 64, (64, 36, 4)), (300, 128, (260, 32))])
+def test_input_gradient_against_float64(dtype, rows, k, ns):
+    """sum_p dy_p W_p in one pass: the block's five layers on a ragged row count, fewer rows than
+    a tile, output widths that are not multiples of 8 or 32 (scalar loads, partial chunks) and
+    wider than one staging chunk."""
+    gen = torch.Generator().manual_seed(rows + len(ns))
+    dys = [torch.randn(rows, n, generator=gen).to(DEV, dtype) for n in ns]
+    ws = [(torch.randn(n, k, generator=gen) * n**-0.5).to(DEV, dtype) for n in ns]
+    got = nn.linear_input_grad(dys, ws)
+    assert got.shape == (rows, k) and got.dtype == dtype
+    want = sum(dy.double() @ w.double() for dy, w in zip(dys, ws))
+    size = sum(dy.double().abs() @ w.double().abs() for dy, w in zip(dys, ws))
+    # fp32 accumulation of exact products, one rounding to the dtype
+    bound = 0.5 * torch.finfo(dtype).eps * want.abs() + sum(ns) * 2.0**-23 * size + torch.finfo(dtype).smallest_normal
+    err = (got.double() - want).abs()
+    assert bool((err <= bound).all()), f"max excess {(err - bound).max().item():.3e}"
+
+
+def test_projection_gradients_are_those_of_the_layers():
+    """project(x, layers) against the layers themselves: equal outputs (the same library products),
+    input and parameter gradients within bf16 rounding, also when one output is unused."""
+    torch.manual_seed(6)
+    dtype = torch.bfloat16
+    x = torch.randn(2, 40, 40, 64, device=DEV, dtype=dtype)
+    layers = [torch.nn.Linear(64, n, bias=wb).to(DEV, dtype) for n, wb in ((64, False), (4, False), (32, True))]
+    dys = [torch.randn(2, 40, 40, m.out_features, device=DEV, dtype=dtype) for m in layers]
+    for used in ((0, 1, 2), (0, 2)):
+        def grads(fn):
+            xi = x.clone().requires_grad_(True)
+            for m in layers:
+                m.zero_grad()
+            outs = fn(xi)
+            torch.autograd.backward([outs[u] for u in used], [dys[u] for u in used])
+            return [o.detach().float() for o in outs], [xi.grad.float()] + [None if p.grad is None else p.grad.float().clone() for m in layers for p in m.parameters()]
+
+        (o1, g1), (o2, g2) = grads(lambda xi: nn.project(xi, layers)), grads(lambda xi: [m(xi) for m in layers])
+        for a, r in zip(o1, o2):
+            assert torch.equal(a, r)
+        for a, r in zip(g1, g2):
+            assert (a is None) == (r is None)
+            if a is not None:
+                assert (a - r).abs().max().item() <= 2.0**-7 * r.abs().max().item(), f"{(a - r).abs().max().item():.3e} of {r.abs().max().item():.3e}"

@@ -649,6 +649,29 @@ int trifast_linear_dw(void* dw, const void* dy, const void* x, int64_t rows, int
   return 0;
 }
 
+int trifast_linear_dx(void* dx, int64_t rows, int64_t k, int nlayers, const void* const* dy, const void* const* wt,
+                      const int64_t* n, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (dtype != TRIFAST_BF16 && dtype != TRIFAST_F16) return fail(TRIFAST_EUNSUPPORTED, "linear_dx: 16-bit element types only (dtype code %d)", dtype);
+  if (rows < 1) return fail(TRIFAST_EINVAL, "linear_dx: rows must be positive (%lld)", (long long)rows);
+  if (!tri::linear_dx_k_ok(k)) return fail(TRIFAST_EUNSUPPORTED, "linear_dx: %lld input channels (32, 64 or 128 are compiled)", (long long)k);
+  if (nlayers < 1 || nlayers > tri::kLinearLayers) return fail(TRIFAST_EINVAL, "linear_dx: 1 to %d layers per call (got %d)", tri::kLinearLayers, nlayers);
+  if (!dx || !dy || !wt || !n) return fail(TRIFAST_EINVAL, "linear_dx: null pointer argument");
+  if ((reinterpret_cast<uintptr_t>(dx) & 15) != 0) return fail(TRIFAST_EALIGN, "linear_dx: dx is not 16-byte aligned");
+  tri::LinearDxArgs a{};
+  a.dx = dx; a.rows = rows; a.K = (int)k; a.nlayers = nlayers;
+  for (int p = 0; p < nlayers; ++p) {
+    if (!dy[p] || !wt[p]) return fail(TRIFAST_EINVAL, "linear_dx: layer %d: null pointer", p);
+    if (n[p] < 1 || n[p] > (1 << 20)) return fail(TRIFAST_EINVAL, "linear_dx: layer %d: %lld outputs", p, (long long)n[p]);
+    if ((reinterpret_cast<uintptr_t>(dy[p]) & 15) != 0 || (reinterpret_cast<uintptr_t>(wt[p]) & 15) != 0)
+      return fail(TRIFAST_EALIGN, "linear_dx: layer %d: dy and the transposed weight must be 16-byte aligned", p);
+    a.dy[p] = dy[p]; a.wt[p] = wt[p]; a.n[p] = (int)n[p];
+  }
+  const hipError_t e = tri::linear_dx_launch(a, dtype, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "linear_dx launch");
+  return 0;
+}
+
 int trifast_gate_fwd(void* y, const void* o, const void* g, int64_t b, int64_t h, int64_t n, int64_t d, int dtype, void* stream) {
   return gate_impl(false, y, nullptr, nullptr, o, g, b, h, n, d, dtype, stream);
 }

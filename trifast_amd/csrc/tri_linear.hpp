@@ -233,3 +233,181 @@ inline hipError_t linear_dw_launch(const LinearDwArgs& a, int dtype, hipStream_t
 }
 
 }  // namespace tri
+
+namespace tri {
+
+// ---------------------------------------------------------------------------------------
+// Input gradient of several linear layers over one input,
+//   dx[r, :] = sum over layers p of dy_p[r, :] W_p            dy_p [rows, N_p], W_p [N_p, K]
+// in one pass: every dy_p is read once and dx is written once (the BLAS library runs one
+// product per layer and autograd adds them up, which moves dx through memory nine times
+// for five layers).  A workgroup owns 256 rows (wave w: rows 64 w .. 64 w + 63 as two 32-row
+// tiles) and all K columns, accumulated in fp32 registers over the layers; the dy rows are
+// staged through LDS 32 columns at a time (coalesced 16-byte loads, two stages ahead in
+// registers), the weights come as W_p^T [K, N_p] (made once per call by the caller: a few
+// tens of KiB) so that their operand fragments are plain 16-byte loads, served by the
+// caches.  The product is computed transposed (W^T dy^T): a lane ends up with one row of dx
+// and 4 x 4 consecutive columns per column block, stored as 8-byte pieces.
+// ---------------------------------------------------------------------------------------
+constexpr int kLinearLayers = 6;
+
+struct LinearDxArgs {
+  const void* dy[kLinearLayers];   // [rows, n[p]]
+  const void* wt[kLinearLayers];   // [K, n[p]]: W_p transposed
+  int n[kLinearLayers];
+  int nlayers;
+  void* dx;                        // [rows, K]
+  int64_t rows;
+  int K;
+};
+
+template <typename T, int KD>
+__global__ __launch_bounds__(256) void linear_dx_kernel(const LinearDxArgs a) {
+  using E = Elem<T>;
+  using frag = typename E::frag;
+  using vec = typename E::vec;
+  constexpr int KB = KD / 32;       // 32-column blocks of dx
+  constexpr int RT = 2;             // 32-row tiles per wave
+  constexpr int ROWS = 4 * RT * 32;  // rows per workgroup
+  constexpr int LD = 32 + 8;        // padded row of a staged chunk (32 columns of dy)
+  constexpr int CH = ROWS * 32 / 8 / 256;  // 16-byte pieces of a chunk per lane
+  __shared__ __attribute__((aligned(16))) T ys[2][ROWS][LD];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int cl = lane & 31, g = lane >> 5;
+  const int64_t row0 = (int64_t)blockIdx.x * ROWS;
+
+  // the chunks of all layers, in order: chunk c of layer p covers its columns 32 c .. 32 c + 31
+  int total = 0;
+  for (int p = 0; p < a.nlayers; ++p) total += (a.n[p] + 31) / 32;
+
+  vec yr[2][CH];
+  // (layer, first column) of chunk number q, walked incrementally by the two users below
+  struct Cursor {
+    int p, c;
+  };
+  auto advance = [&](Cursor& cur) {
+    if (32 * (cur.c + 1) < a.n[cur.p]) ++cur.c;
+    else { ++cur.p; cur.c = 0; }
+  };
+  auto load_chunk = [&](const Cursor& cur, vec* dst) {
+    const T* src = reinterpret_cast<const T*>(a.dy[cur.p]);
+    const int N = a.n[cur.p];
+    const bool vec_ok = (N % 8) == 0;
+#pragma unroll
+    for (int x = 0; x < CH; ++x) {
+      const int q = x * 256 + tid, r = q / 4, col = 32 * cur.c + 8 * (q % 4);
+      vec v = {};
+      if (row0 + r < a.rows && col < N) {
+        const T* s = src + (row0 + r) * N + col;
+        if (vec_ok) {
+          v = *reinterpret_cast<const vec*>(s);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (col + e < N) v[e] = s[e];
+        }
+      }
+      dst[x] = v;
+    }
+  };
+  auto store_chunk = [&](int buf, const vec* src) {
+#pragma unroll
+    for (int x = 0; x < CH; ++x) {
+      const int q = x * 256 + tid, r = q / 4, col = 8 * (q % 4);
+      *reinterpret_cast<vec*>(&ys[buf][r][col]) = src[x];
+    }
+  };
+
+  f32x16 acc[RT][KB];
+#pragma unroll
+  for (int t = 0; t < RT; ++t)
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) acc[t][kb] = zero16();
+
+  Cursor ld{0, 0}, use{0, 0};
+  load_chunk(ld, yr[0]);
+  advance(ld);
+  if (total > 1) { load_chunk(ld, yr[1]); advance(ld); }
+  store_chunk(0, yr[0]);
+  __syncthreads();
+  auto one_chunk = [&](int q, auto parity) __attribute__((always_inline)) {
+    constexpr int buf = decltype(parity)::value;
+    if (q + 2 < total) { load_chunk(ld, yr[buf]); advance(ld); }
+    // weights of this chunk: W^T[k][32 c + 16 s2 + 8 g ..], k = 32 kb + lane % 32 (columns past
+    // N_p read the last valid piece: they meet zeros of the staged dy)
+    const T* wt = reinterpret_cast<const T*>(a.wt[use.p]);
+    const int N = a.n[use.p];
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      const int n0 = 32 * use.c + 16 * s2 + 8 * g;
+      frag bf[RT];
+#pragma unroll
+      for (int t = 0; t < RT; ++t) bf[t] = *reinterpret_cast<const frag*>(&ys[buf][64 * wave + 32 * t + cl][16 * s2 + 8 * g]);
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        const T* wp = wt + (int64_t)(32 * kb + cl) * N + n0;
+        frag af = {};
+        if ((N % 8) == 0) {
+          if (n0 < N) af = *reinterpret_cast<const frag*>(wp);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (n0 + e < N) af[e] = wp[e];
+        }
+#pragma unroll
+        for (int t = 0; t < RT; ++t) acc[t][kb] = E::mfma(af, bf[t], acc[t][kb]);
+      }
+    }
+    advance(use);
+    if (q + 1 < total) store_chunk(buf ^ 1, yr[buf ^ 1]);
+    __syncthreads();
+  };
+  for (int q = 0; q < total; q += 2) {
+    one_chunk(q, std::integral_constant<int, 0>{});
+    if (q + 1 < total) one_chunk(q + 1, std::integral_constant<int, 1>{});
+  }
+
+  // dx: the lane holds row 64 wave + 32 t + lane % 32 and columns 32 kb + 8 q + 4 g + 0..3
+  T* dx = reinterpret_cast<T*>(a.dx);
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    const int64_t row = row0 + 64 * wave + 32 * t + cl;
+    if (row >= a.rows) continue;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        typename E::vec4 ov;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ov[e] = (T)acc[t][kb][4 * q + e];
+        *reinterpret_cast<typename E::vec4*>(dx + row * KD + 32 * kb + 8 * q + 4 * g) = ov;
+      }
+  }
+}
+
+template <typename T>
+inline hipError_t linear_dx_launch_t(const LinearDxArgs& a, hipStream_t st) {
+  const dim3 grid((unsigned)((a.rows + 255) / 256)), block(256);
+  switch (a.K) {
+    case 32: hipLaunchKernelGGL((linear_dx_kernel<T, 32>), grid, block, 0, st, a); break;
+    case 64: hipLaunchKernelGGL((linear_dx_kernel<T, 64>), grid, block, 0, st, a); break;
+    case 128: hipLaunchKernelGGL((linear_dx_kernel<T, 128>), grid, block, 0, st, a); break;
+    default: return hipErrorInvalidConfiguration;
+  }
+  return hipGetLastError();
+}
+
+// (the accumulators of 64 rows x K columns per wave stay in registers: K up to 128)
+inline bool linear_dx_k_ok(int64_t k) { return k == 32 || k == 64 || k == 128; }
+
+inline hipError_t linear_dx_launch(const LinearDxArgs& a, int dtype, hipStream_t st) {
+  switch (dtype) {
+    case kBF16: return linear_dx_launch_t<__bf16>(a, st);
+    case kF16: return linear_dx_launch_t<_Float16>(a, st);
+  }
+  return hipErrorInvalidConfiguration;
+}
+
+}  // namespace tri

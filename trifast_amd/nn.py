@@ -13,7 +13,8 @@ tensor is copied to change its layout:
 * The weight gradients of the six linear layers come from ``trifast_linear_dw``: for rows in
   the millions and a few hundred channels the BLAS library runs that product (a contraction
   over all rows into a tiny matrix) on one or two workgroups, ten times slower than the
-  layer's other two products.
+  layer's other two products.  The input gradient of the five projections of x is one pass
+  (``trifast_linear_dx``) instead of five products and four additions.
 * The output gate ``o * sigmoid(g)`` and the layout change from the operator's
   ``[*, h, n, n, d]`` to the ``[*, n, n, h*d]`` that the output projection consumes are one
   streaming HIP kernel (``trifast_gate_fwd`` / ``trifast_gate_bwd``).
@@ -125,6 +126,67 @@ class _Linear(torch.autograd.Function):
         return dx, dw, db
 
 
+_DX_K = (32, 64, 128)
+_DX_LAYERS = 6
+
+
+def linear_input_grad(dys, weights) -> torch.Tensor:
+    """``sum_p dys[p] @ weights[p]`` for ``dys[p] [rows, n_p]``, ``weights[p] [n_p, k]``: the input
+    gradient of several linear layers over one input, every ``dys[p]`` read once and the sum
+    written once (``trifast_linear_dx``)."""
+    dys = [dy.contiguous() for dy in dys]
+    wts = [w.t().contiguous() for w in weights]  # [k, n_p]: a few tens of KiB each
+    rows, k = dys[0].shape[0], weights[0].shape[1]
+    dx = torch.empty(rows, k, dtype=dys[0].dtype, device=dys[0].device)
+    ptrs = lambda ts: (_lib.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    with torch.cuda.device(dx.device):
+        rc = _lib.load().trifast_linear_dx(dx.data_ptr(), rows, k, len(dys), ptrs(dys), ptrs(wts), _lib.i64_array([dy.shape[1] for dy in dys]),
+                                           _dtype_code(dx), torch.cuda.current_stream(dx.device).cuda_stream)
+    _lib.check(rc, "trifast_linear_dx")
+    return dx
+
+
+class _Project(torch.autograd.Function):
+    """Several linear layers over one input.  Forward: the BLAS library's product per layer.
+    Backward: one pass for the input gradient of all layers (``trifast_linear_dx``), this
+    library's kernel for each weight gradient (``trifast_linear_dw``)."""
+
+    @staticmethod
+    def forward(ctx, x, n_layers, *params):
+        weights, biases = params[:n_layers], params[n_layers:]
+        ctx.save_for_backward(x, *weights)
+        ctx.has_bias = [b is not None for b in biases]
+        ctx.set_materialize_grads(False)  # an unused output gives None, not a tensor of zeros to multiply
+        return tuple(torch.nn.functional.linear(x, w, b) for w, b in zip(weights, biases))
+
+    @staticmethod
+    def backward(ctx, *dys):
+        x, *weights = ctx.saved_tensors
+        x2 = x.reshape(-1, x.shape[-1])
+        # (a layer whose output took no part in the loss has no gradient to give)
+        live = [(dy.reshape(-1, dy.shape[-1]), w) for dy, w in zip(dys, weights) if dy is not None]
+        dx = None
+        if ctx.needs_input_grad[0] and live:
+            if x.shape[-1] in _DX_K:
+                dx = linear_input_grad([dy for dy, _ in live], [w for _, w in live]).view(x.shape)
+            else:
+                dx = sum(dy @ w for dy, w in live).view(x.shape)
+        dws = [None if dy is None else linear_weight_grad(dy.reshape(-1, dy.shape[-1]), x2) for dy in dys]
+        dbs = [dy.reshape(-1, dy.shape[-1]).sum(0) if (dy is not None and has) else None for dy, has in zip(dys, ctx.has_bias)]
+        return (dx, None, *dws, *dbs)
+
+
+def project(x: torch.Tensor, layers) -> tuple[torch.Tensor, ...]:
+    """``tuple(layer(x) for layer in layers)`` for up to 6 ``torch.nn.Linear`` layers over the
+    same pair representation ``x [*, k]``, with a backward that reads every output gradient
+    once for the input gradient and computes the weight gradients with this library's kernel
+    (GPU, 16-bit, k in (32, 64, 128, 256)); anything else is the layers themselves."""
+    layers = list(layers)
+    if not layers or len(layers) > _DX_LAYERS or not all(_dw_ready(x, m.weight) for m in layers):
+        return tuple(m(x) for m in layers)
+    return _Project.apply(x, len(layers), *[m.weight for m in layers], *[m.bias for m in layers])
+
+
 def linear(x: torch.Tensor, layer: torch.nn.Linear) -> torch.Tensor:
     """``layer(x)`` for a linear layer over a pair representation ``x [*, k]``; on the GPU, for
     16-bit tensors with k in (32, 64, 128, 256), its weight gradient is computed by this
@@ -155,8 +217,7 @@ class TriangleAttention(torch.nn.Module):
         return t.unflatten(-1, (self.h, self.d)).movedim(-2, -4)
 
     def forward(self, x: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
-        q, k, v = self.heads(linear(x, self.q)), self.heads(linear(x, self.k)), self.heads(linear(x, self.v))
-        bias = linear(x, self.b).movedim(-1, -3)
+        q, k, v, bias, g = project(x, (self.q, self.k, self.v, self.b, self.g))
         attend = triangle_attention_ending_node if self.ending_node else triangle_attention
-        o = attend(q, k, v, bias, mask)
-        return linear(gated_output(o, linear(x, self.g)), self.out)
+        o = attend(self.heads(q), self.heads(k), self.heads(v), bias.movedim(-1, -3), mask)
+        return linear(gated_output(o, g), self.out)

@@ -151,6 +151,22 @@ def block(n: int, c_in: int) -> None:
     ms = _median_ms(lambda: gy.copy_(g))
     print(f"(a plain device copy of one such tensor {ms * 1e3:8.1f} us  {2 * size / ms / 1e6:7.1f} GB/s read + written)")
     x2 = x.detach().reshape(-1, c_in)
+    widths = (H * D, H * D, H * D, H, H * D)  # q, k, v, bias, gate
+    dys = [torch.randn(x2.shape[0], w, device=dev, dtype=DTYPE) for w in widths]
+    ws = [torch.randn(w, c_in, device=dev, dtype=DTYPE) for w in widths]
+    nbytes = (sum(t.numel() for t in dys) + x2.numel()) * x2.element_size()
+    ms = _median_ms(lambda: nn.linear_input_grad(dys, ws))
+
+    def blas_dx():
+        dx = dys[0] @ ws[0]
+        for dy, w in zip(dys[1:], ws[1:]):
+            dx = dx + dy @ w  # (what autograd does with the layers' separate input gradients)
+        return dx
+
+    ms_blas = _median_ms(blas_dx)
+    print(f"input gradient of the five projections {ms * 1e3:8.1f} us  {nbytes / ms / 1e6:7.1f} GB/s of the dy and dx ({nbytes / 2**20:.0f} MiB); "
+          f"the BLAS library's five products and four additions {ms_blas * 1e3:8.1f} us")
+    del dys, ws
     for n_out in (H * D, H):
         dy2 = torch.randn(x2.shape[0], n_out, device=dev, dtype=DTYPE)
         nbytes = (x2.numel() + dy2.numel()) * x2.element_size()
