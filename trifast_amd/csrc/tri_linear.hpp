@@ -244,9 +244,10 @@ namespace tri {
 // for five layers).  A workgroup owns 256 rows (wave w: rows 64 w .. 64 w + 63 as two 32-row
 // tiles) and all K columns, accumulated in fp32 registers over the layers; the dy rows are
 // staged through LDS 32 columns at a time (coalesced 16-byte loads, two stages ahead in
-// registers), the weights come as W_p^T [K, N_p] (made once per call by the caller: a few
-// tens of KiB) so that their operand fragments are plain 16-byte loads, served by the
-// caches.  The product is computed transposed (W^T dy^T): a lane ends up with one row of dx
+// registers), and so are the same 32 columns of the weights, which come as W_p^T [K, N_p]
+// (made once per call by the caller: a few tens of KiB) so that the operand fragments of both
+// are plain 16-byte LDS reads.  (Weight fragments loaded straight from global memory, eight
+// per chunk and wave, were waited for one by one: 0.59 ms for the block's five layers.)  The product is computed transposed (W^T dy^T): a lane ends up with one row of dx
 // and 4 x 4 consecutive columns per column block, stored as 8-byte pieces.
 // ---------------------------------------------------------------------------------------
 constexpr int kLinearLayers = 6;
@@ -271,7 +272,11 @@ __global__ __launch_bounds__(256) void linear_dx_kernel(const LinearDxArgs a) {
   constexpr int ROWS = 4 * RT * 32;  // rows per workgroup
   constexpr int LD = 32 + 8;        // padded row of a staged chunk (32 columns of dy)
   constexpr int CH = ROWS * 32 / 8 / 256;  // 16-byte pieces of a chunk per lane
-  __shared__ __attribute__((aligned(16))) T ys[2][ROWS][LD];
+  constexpr int PF = 2;             // chunks in flight: one register set and one LDS buffer each
+  constexpr int WPC = KD * 32 / 8;  // 16-byte pieces of a chunk of W^T (KD rows of 32 columns)
+  constexpr int WCH = (WPC + 255) / 256;
+  __shared__ __attribute__((aligned(16))) T ys[PF][ROWS][LD];
+  __shared__ __attribute__((aligned(16))) T ws[PF][KD][LD];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -282,7 +287,7 @@ __global__ __launch_bounds__(256) void linear_dx_kernel(const LinearDxArgs a) {
   int total = 0;
   for (int p = 0; p < a.nlayers; ++p) total += (a.n[p] + 31) / 32;
 
-  vec yr[2][CH];
+  vec yr[PF][CH], wr[PF][WCH];
   // (layer, first column) of chunk number q, walked incrementally by the two users below
   struct Cursor {
     int p, c;
@@ -291,10 +296,28 @@ __global__ __launch_bounds__(256) void linear_dx_kernel(const LinearDxArgs a) {
     if (32 * (cur.c + 1) < a.n[cur.p]) ++cur.c;
     else { ++cur.p; cur.c = 0; }
   };
-  auto load_chunk = [&](const Cursor& cur, vec* dst) {
+  auto load_chunk = [&](const Cursor& cur, vec* dst, vec* wdst) {
     const T* src = reinterpret_cast<const T*>(a.dy[cur.p]);
+    const T* wsrc = reinterpret_cast<const T*>(a.wt[cur.p]);
     const int N = a.n[cur.p];
     const bool vec_ok = (N % 8) == 0;
+    // the same 32 columns of W^T (columns past N_p are zero, like those of dy)
+#pragma unroll
+    for (int x = 0; x < WCH; ++x) {
+      const int q = x * 256 + tid, k = q / 4, col = 32 * cur.c + 8 * (q % 4);
+      vec v = {};
+      if (q < WPC && col < N) {
+        const T* s = wsrc + (int64_t)k * N + col;
+        if (vec_ok) {
+          v = *reinterpret_cast<const vec*>(s);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (col + e < N) v[e] = s[e];
+        }
+      }
+      wdst[x] = v;
+    }
 #pragma unroll
     for (int x = 0; x < CH; ++x) {
       const int q = x * 256 + tid, r = q / 4, col = 32 * cur.c + 8 * (q % 4);
@@ -312,11 +335,16 @@ __global__ __launch_bounds__(256) void linear_dx_kernel(const LinearDxArgs a) {
       dst[x] = v;
     }
   };
-  auto store_chunk = [&](int buf, const vec* src) {
+  auto store_chunk = [&](int buf, const vec* src, const vec* wsrc) {
 #pragma unroll
     for (int x = 0; x < CH; ++x) {
       const int q = x * 256 + tid, r = q / 4, col = 8 * (q % 4);
       *reinterpret_cast<vec*>(&ys[buf][r][col]) = src[x];
+    }
+#pragma unroll
+    for (int x = 0; x < WCH; ++x) {
+      const int q = x * 256 + tid, k = q / 4, col = 8 * (q % 4);
+      if (q < WPC) *reinterpret_cast<vec*>(&ws[buf][k][col]) = wsrc[x];
     }
   };
 
@@ -326,45 +354,36 @@ __global__ __launch_bounds__(256) void linear_dx_kernel(const LinearDxArgs a) {
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) acc[t][kb] = zero16();
 
-  Cursor ld{0, 0}, use{0, 0};
-  load_chunk(ld, yr[0]);
-  advance(ld);
-  if (total > 1) { load_chunk(ld, yr[1]); advance(ld); }
-  store_chunk(0, yr[0]);
+  Cursor ld{0, 0};
+#pragma unroll
+  for (int q = 0; q < PF; ++q)
+    if (q < total) { load_chunk(ld, yr[q], wr[q]); advance(ld); }
+  store_chunk(0, yr[0], wr[0]);
   __syncthreads();
-  auto one_chunk = [&](int q, auto parity) __attribute__((always_inline)) {
-    constexpr int buf = decltype(parity)::value;
-    if (q + 2 < total) { load_chunk(ld, yr[buf]); advance(ld); }
-    // weights of this chunk: W^T[k][32 c + 16 s2 + 8 g ..], k = 32 kb + lane % 32 (columns past
-    // N_p read the last valid piece: they meet zeros of the staged dy)
-    const T* wt = reinterpret_cast<const T*>(a.wt[use.p]);
-    const int N = a.n[use.p];
+  // chunk q: registers and LDS buffer q % PF.  Its registers went to LDS at the end of the
+  // step before, so they take the loads of chunk q + PF; the buffer of chunk q + 1 was last
+  // read in step q + 1 - PF, which every wave left at least one barrier ago.
+  auto one_chunk = [&](int q, auto which) __attribute__((always_inline)) {
+    constexpr int buf = decltype(which)::value;
+    constexpr int nxt = (buf + 1) % PF;
+    if (q + PF < total) { load_chunk(ld, yr[buf], wr[buf]); advance(ld); }
 #pragma unroll
     for (int s2 = 0; s2 < 2; ++s2) {
-      const int n0 = 32 * use.c + 16 * s2 + 8 * g;
       frag bf[RT];
 #pragma unroll
       for (int t = 0; t < RT; ++t) bf[t] = *reinterpret_cast<const frag*>(&ys[buf][64 * wave + 32 * t + cl][16 * s2 + 8 * g]);
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb) {
-        const T* wp = wt + (int64_t)(32 * kb + cl) * N + n0;
-        frag af = {};
-        if ((N % 8) == 0) {
-          if (n0 < N) af = *reinterpret_cast<const frag*>(wp);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (n0 + e < N) af[e] = wp[e];
-        }
+        // W^T[k][32 c + 16 s2 + 8 g ..], k = 32 kb + lane % 32
+        const frag af = *reinterpret_cast<const frag*>(&ws[buf][32 * kb + cl][16 * s2 + 8 * g]);
 #pragma unroll
         for (int t = 0; t < RT; ++t) acc[t][kb] = E::mfma(af, bf[t], acc[t][kb]);
       }
     }
-    advance(use);
-    if (q + 1 < total) store_chunk(buf ^ 1, yr[buf ^ 1]);
+    if (q + 1 < total) store_chunk(nxt, yr[nxt], wr[nxt]);
     __syncthreads();
   };
-  for (int q = 0; q < total; q += 2) {
+  for (int q = 0; q < total; q += PF) {
     one_chunk(q, std::integral_constant<int, 0>{});
     if (q + 1 < total) one_chunk(q + 1, std::integral_constant<int, 1>{});
   }
