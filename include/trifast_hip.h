@@ -192,6 +192,15 @@ int trifast_bwd_one(int kernel,
  */
 int64_t trifast_linear_dw_workspace_bytes(int64_t rows, int64_t k, int64_t n);
 /*
+ * Up to 6 linear layers over the same pair representation in one pass that reads x once:
+ * y_p = x W_p^T + bias_p for x [rows, k], W_p [n_p, k], bias_p [n_p] or null, y_p [rows, n_p]
+ * (all dense, one 16-bit dtype, k in {32, 64, 128}).  w, bias, y, n are host arrays of nlayers
+ * entries (bias itself may be null: no layer has one).  No counterpart in the reference (see
+ * trifast_linear_dw).
+ */
+int trifast_linear_fwd(const void* x, int64_t rows, int64_t k, int nlayers, const void* const* w, const void* const* bias,
+                       void* const* y, const int64_t* n, int dtype, void* stream);
+/*
  * Input gradient of up to 6 linear layers over the same pair representation in one pass:
  * dx[r, :] = sum over layers p of dy_p[r, :] W_p, with dy_p [rows, n_p] and the weights given
  * transposed, wt_p = W_p^T [k, n_p] (all dense, one 16-bit dtype, k in {32, 64, 128}); every

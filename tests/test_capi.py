@@ -142,6 +142,23 @@ def test_weight_gradient_argument_errors_come_back_as_codes():
     assert lib.trifast_linear_dw_workspace_bytes(0, 128, 4) < 0
 
 
+def test_linear_forward_argument_errors_come_back_as_codes():
+    import ctypes
+
+    lib = _lib.load()
+    ok = 0x1000
+    vp = lambda *v: (ctypes.c_void_p * len(v))(*v)
+    n1 = _lib.i64_array([8])
+    call = lambda x, k, nl, w, y, n, dtype=_lib.BF16, rows=4: lib.trifast_linear_fwd(x, rows, k, nl, w, None, y, n, dtype, None)
+    assert call(ok, 256, 1, vp(ok), vp(ok), n1) == -2 and "input channels" in _lib.last_error()
+    assert call(ok, 64, 1, vp(ok), vp(ok), n1, _lib.F32) == -2 and "16-bit" in _lib.last_error()
+    assert call(ok, 64, 7, vp(*[ok] * 7), vp(*[ok] * 7), _lib.i64_array([8] * 7)) == -1 and "layers per call" in _lib.last_error()
+    assert call(ok + 8, 64, 1, vp(ok), vp(ok), n1) == -3 and "x is not" in _lib.last_error()
+    assert call(ok, 64, 1, vp(ok), vp(ok + 4), n1) == -3 and "layer 0" in _lib.last_error()
+    assert call(ok, 64, 1, vp(None), vp(ok), n1) == -1 and "null" in _lib.last_error()
+    assert call(ok, 64, 1, vp(ok), vp(ok), n1, rows=0) == -1 and "rows" in _lib.last_error()
+
+
 def test_input_gradient_argument_errors_come_back_as_codes():
     import ctypes
 

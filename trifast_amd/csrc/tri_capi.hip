@@ -649,6 +649,30 @@ int trifast_linear_dw(void* dw, const void* dy, const void* x, int64_t rows, int
   return 0;
 }
 
+int trifast_linear_fwd(const void* x, int64_t rows, int64_t k, int nlayers, const void* const* w, const void* const* bias,
+                       void* const* y, const int64_t* n, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (dtype != TRIFAST_BF16 && dtype != TRIFAST_F16) return fail(TRIFAST_EUNSUPPORTED, "linear_fwd: 16-bit element types only (dtype code %d)", dtype);
+  if (rows < 1) return fail(TRIFAST_EINVAL, "linear_fwd: rows must be positive (%lld)", (long long)rows);
+  if (!tri::linear_fwd_k_ok(k)) return fail(TRIFAST_EUNSUPPORTED, "linear_fwd: %lld input channels (32, 64 or 128 are compiled)", (long long)k);
+  if (nlayers < 1 || nlayers > tri::kLinearLayers) return fail(TRIFAST_EINVAL, "linear_fwd: 1 to %d layers per call (got %d)", tri::kLinearLayers, nlayers);
+  if (!x || !w || !y || !n) return fail(TRIFAST_EINVAL, "linear_fwd: null pointer argument");
+  if ((reinterpret_cast<uintptr_t>(x) & 15) != 0) return fail(TRIFAST_EALIGN, "linear_fwd: x is not 16-byte aligned");
+  tri::LinearFwdArgs a{};
+  a.x = x; a.rows = rows; a.K = (int)k; a.nlayers = nlayers;
+  for (int p = 0; p < nlayers; ++p) {
+    if (!w[p] || !y[p]) return fail(TRIFAST_EINVAL, "linear_fwd: layer %d: null pointer", p);
+    if (n[p] < 1 || n[p] > (1 << 20)) return fail(TRIFAST_EINVAL, "linear_fwd: layer %d: %lld outputs", p, (long long)n[p]);
+    if ((reinterpret_cast<uintptr_t>(w[p]) & 15) != 0 || (reinterpret_cast<uintptr_t>(y[p]) & 15) != 0)
+      return fail(TRIFAST_EALIGN, "linear_fwd: layer %d: weight and output must be 16-byte aligned", p);
+    a.w[p] = w[p]; a.bias[p] = bias ? bias[p] : nullptr; a.y[p] = y[p]; a.n[p] = (int)n[p];
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const hipError_t e = dtype == TRIFAST_BF16 ? tri::linear_fwd_launch_t<__bf16>(a, st) : tri::linear_fwd_launch_t<_Float16>(a, st);
+  if (e != hipSuccess) return hip_fail(e, "linear_fwd launch");
+  return 0;
+}
+
 int trifast_linear_dx(void* dx, int64_t rows, int64_t k, int nlayers, const void* const* dy, const void* const* wt,
                       const int64_t* n, int dtype, void* stream) {
   g_err[0] = 0;

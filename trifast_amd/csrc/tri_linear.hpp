@@ -430,3 +430,210 @@ inline hipError_t linear_dx_launch(const LinearDxArgs& a, int dtype, hipStream_t
 }
 
 }  // namespace tri
+
+namespace tri {
+
+// ---------------------------------------------------------------------------------------
+// Several linear layers over one input in one pass,
+//   y_p[r, :] = x[r, :] W_p^T + bias_p        x [rows, K], W_p [N_p, K], y_p [rows, N_p]
+// x is read once for all layers (the BLAS library reads it once per layer).  A workgroup
+// owns 256 rows: their K / 16 operand fragments go through LDS once (coalesced loads) into
+// registers (wave w: rows 64 w .. 64 w + 63 as two 32-row tiles) and stay there; the layers'
+// weights pass through LDS 32 output columns at a time (one stage ahead in registers).  The
+// product is computed transposed (W x^T, bias as accumulator init), so a lane holds one row
+// and 4 x 4 consecutive columns of the chunk; the chunk goes back through the wave's own
+// piece of LDS and leaves as 16-byte pieces, 64 contiguous bytes per row.
+// ---------------------------------------------------------------------------------------
+struct LinearFwdArgs {
+  const void* x;                    // [rows, K]
+  const void* w[kLinearLayers];     // [n[p], K]
+  const void* bias[kLinearLayers];  // [n[p]] or null
+  void* y[kLinearLayers];           // [rows, n[p]]
+  int n[kLinearLayers];
+  int nlayers;
+  int64_t rows;
+  int K;
+};
+
+// LDS of the kernel below: the x tile, or what takes its place (two weight chunks and the
+// output chunk), whichever is larger
+constexpr int linear_fwd_lds_bytes(int kd, int es) {
+  const int xbytes = 256 * (kd + 8) * es, cbytes = 2 * 32 * (kd + 8) * es + 256 * (32 + 8) * es;
+  return xbytes > cbytes ? xbytes : cbytes;
+}
+
+template <typename T, int KD>
+__global__ __launch_bounds__(256) void linear_fwd_kernel(const LinearFwdArgs a) {
+  using E = Elem<T>;
+  using frag = typename E::frag;
+  using vec = typename E::vec;
+  constexpr int KS = KD / 16;        // MFMA steps over K
+  constexpr int RT = 2, ROWS = 256;
+  constexpr int LDX = KD + 8;        // padded row of the x tile and of a weight chunk
+  constexpr int LDO = 32 + 8;        // padded row of an output chunk
+  constexpr int XP = ROWS * KD / 8 / 256;  // 16-byte pieces of the x tile per lane
+  constexpr int WPC = 32 * KD / 8;   // ... of a weight chunk (32 rows of W)
+  constexpr int WCH = (WPC + 255) / 256;
+  // LDS: first the x tile; once its fragments are in registers, two weight chunks and the
+  // output chunk take its place
+  extern __shared__ __attribute__((aligned(16))) unsigned char lin_smem[];
+  T (*xs)[LDX] = reinterpret_cast<T (*)[LDX]>(lin_smem);
+  T (*wsm)[32][LDX] = reinterpret_cast<T (*)[32][LDX]>(lin_smem);                       // [2][32][LDX]
+  T (*os)[LDO] = reinterpret_cast<T (*)[LDO]>(lin_smem + 2 * 32 * LDX * sizeof(T));      // [ROWS][LDO]
+  static_assert(2 * 32 * LDX * sizeof(T) + ROWS * LDO * sizeof(T) <= linear_fwd_lds_bytes(KD, (int)sizeof(T)), "the launcher sizes LDS with linear_fwd_lds_bytes");
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int cl = lane & 31, g = lane >> 5;
+  const int64_t row0 = (int64_t)blockIdx.x * ROWS;
+  const T* xg = reinterpret_cast<const T*>(a.x);
+
+  // x tile -> LDS -> registers
+#pragma unroll
+  for (int x4 = 0; x4 < XP; x4 += 4) {
+    vec v[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int q = (x4 + x) * 256 + tid, r = q / (KD / 8), col = 8 * (q % (KD / 8));
+      v[x] = vec{};
+      if (row0 + r < a.rows) v[x] = *reinterpret_cast<const vec*>(xg + (row0 + r) * KD + col);
+    }
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int q = (x4 + x) * 256 + tid, r = q / (KD / 8), col = 8 * (q % (KD / 8));
+      *reinterpret_cast<vec*>(&xs[r][col]) = v[x];
+    }
+  }
+  __syncthreads();
+  frag xf[RT][KS];
+#pragma unroll
+  for (int t = 0; t < RT; ++t)
+#pragma unroll
+    for (int s = 0; s < KS; ++s) xf[t][s] = *reinterpret_cast<const frag*>(&xs[64 * wave + 32 * t + cl][16 * s + 8 * g]);
+  __syncthreads();
+
+  int total = 0;
+  for (int p = 0; p < a.nlayers; ++p) total += (a.n[p] + 31) / 32;
+  struct Cursor {
+    int p, c;
+  };
+  auto advance = [&](Cursor& cur) {
+    if (32 * (cur.c + 1) < a.n[cur.p]) ++cur.c;
+    else { ++cur.p; cur.c = 0; }
+  };
+  // rows 32 c .. 32 c + 31 of W_p (rows past N_p are zero)
+  vec wr[2][WCH];
+  auto load_chunk = [&](const Cursor& cur, vec* dst) {
+    const T* wsrc = reinterpret_cast<const T*>(a.w[cur.p]);
+    const int N = a.n[cur.p];
+#pragma unroll
+    for (int x = 0; x < WCH; ++x) {
+      const int q = x * 256 + tid, r = q / (KD / 8), col = 8 * (q % (KD / 8));
+      vec v = {};
+      if (q < WPC && 32 * cur.c + r < N) v = *reinterpret_cast<const vec*>(wsrc + (int64_t)(32 * cur.c + r) * KD + col);
+      dst[x] = v;
+    }
+  };
+  auto store_chunk = [&](int buf, const vec* src) {
+#pragma unroll
+    for (int x = 0; x < WCH; ++x) {
+      const int q = x * 256 + tid, r = q / (KD / 8), col = 8 * (q % (KD / 8));
+      if (q < WPC) *reinterpret_cast<vec*>(&wsm[buf][r][col]) = src[x];
+    }
+  };
+
+  Cursor ld{0, 0}, use{0, 0};
+  load_chunk(ld, wr[0]);
+  advance(ld);
+  if (total > 1) { load_chunk(ld, wr[1]); advance(ld); }
+  store_chunk(0, wr[0]);
+  __syncthreads();
+  auto one_chunk = [&](int q, auto which) __attribute__((always_inline)) {
+    constexpr int buf = decltype(which)::value;
+    if (q + 2 < total) { load_chunk(ld, wr[buf]); advance(ld); }
+    const int N = a.n[use.p], n0 = 32 * use.c;
+    const T* bias = reinterpret_cast<const T*>(a.bias[use.p]);
+    T* y = reinterpret_cast<T*>(a.y[use.p]);
+    // this lane's 16 columns of the chunk: n0 + 8 q4 + 4 g + e
+    f32x16 acc[RT];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int n = n0 + 8 * (v / 4) + 4 * g + (v % 4);
+      const float b = (bias && n < N) ? (float)bias[n] : 0.f;
+#pragma unroll
+      for (int t = 0; t < RT; ++t) acc[t][v] = b;
+    }
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const frag af = *reinterpret_cast<const frag*>(&wsm[buf][cl][16 * s + 8 * g]);
+#pragma unroll
+      for (int t = 0; t < RT; ++t) acc[t] = E::mfma(af, xf[t][s], acc[t]);
+    }
+    // the chunk of this wave's 64 rows -> its own rows of the output tile -> global memory
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        typename E::vec4 ov;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ov[e] = (T)acc[t][4 * q4 + e];
+        *reinterpret_cast<typename E::vec4*>(&os[64 * wave + 32 * t + cl][8 * q4 + 4 * g]) = ov;
+      }
+    // (the wave reads back only what it wrote: LDS operations of a wave complete in order)
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int idx = x * 64 + lane, r = 64 * wave + idx / 4, col = n0 + 8 * (idx % 4);
+      const int64_t row = row0 + r;
+      const vec v = *reinterpret_cast<const vec*>(&os[r][8 * (idx % 4)]);
+      if (row < a.rows && col < N) {
+        T* dst = y + row * N + col;
+        if ((N % 8) == 0) {
+          *reinterpret_cast<vec*>(dst) = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (col + e < N) dst[e] = v[e];
+        }
+      }
+    }
+    advance(use);
+    if (q + 1 < total) store_chunk(buf ^ 1, wr[buf ^ 1]);
+    __syncthreads();
+  };
+  for (int q = 0; q < total; q += 2) {
+    one_chunk(q, std::integral_constant<int, 0>{});
+    if (q + 1 < total) one_chunk(q + 1, std::integral_constant<int, 1>{});
+  }
+}
+
+inline bool linear_fwd_k_ok(int64_t k) { return k == 32 || k == 64 || k == 128; }
+
+template <typename T, int KD>
+inline hipError_t linear_fwd_launch_k(const LinearFwdArgs& a, hipStream_t st) {
+  const dim3 grid((unsigned)((a.rows + 255) / 256)), block(256);
+  constexpr int lds = linear_fwd_lds_bytes(KD, (int)sizeof(T));
+  if (lds > 64 * 1024) {
+    // (more dynamic LDS than the default limit: raised once per kernel)
+    static thread_local bool raised = false;
+    if (!raised) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(linear_fwd_kernel<T, KD>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      if (e != hipSuccess) return e;
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL((linear_fwd_kernel<T, KD>), grid, block, lds, st, a);
+  return hipGetLastError();
+}
+
+template <typename T>
+inline hipError_t linear_fwd_launch_t(const LinearFwdArgs& a, hipStream_t st) {
+  switch (a.K) {
+    case 32: return linear_fwd_launch_k<T, 32>(a, st);
+    case 64: return linear_fwd_launch_k<T, 64>(a, st);
+    case 128: return linear_fwd_launch_k<T, 128>(a, st);
+  }
+  return hipErrorInvalidConfiguration;
+}
+
+}  // namespace tri

@@ -13,8 +13,9 @@ tensor is copied to change its layout:
 * The weight gradients of the six linear layers come from ``trifast_linear_dw``: for rows in
   the millions and a few hundred channels the BLAS library runs that product (a contraction
   over all rows into a tiny matrix) on one or two workgroups, ten times slower than the
-  layer's other two products.  The input gradient of the five projections of x is one pass
-  (``trifast_linear_dx``) instead of five products and four additions.
+  layer's other two products.  The five projections of x are one pass over x
+  (``trifast_linear_fwd``) and their input gradient is one pass (``trifast_linear_dx``)
+  instead of five products and four additions.
 * The output gate ``o * sigmoid(g)`` and the layout change from the operator's
   ``[*, h, n, n, d]`` to the ``[*, n, n, h*d]`` that the output projection consumes are one
   streaming HIP kernel (``trifast_gate_fwd`` / ``trifast_gate_bwd``).
@@ -146,10 +147,28 @@ def linear_input_grad(dys, weights) -> torch.Tensor:
     return dx
 
 
+def linear_outputs(x: torch.Tensor, weights, biases) -> list[torch.Tensor]:
+    """``[x @ w.T + b for w, b in zip(weights, biases)]`` for ``x [rows, k]`` in one pass that reads
+    x once (``trifast_linear_fwd``); a bias may be None."""
+    x = x.contiguous()
+    rows, k = x.shape
+    ws = [w.contiguous() for w in weights]
+    bs = [None if b is None else b.contiguous() for b in biases]
+    ys = [torch.empty(rows, w.shape[0], dtype=x.dtype, device=x.device) for w in ws]
+    ptrs = lambda ts: (_lib.c_void_p * len(ts))(*[None if t is None else t.data_ptr() for t in ts])
+    with torch.cuda.device(x.device):
+        rc = _lib.load().trifast_linear_fwd(x.data_ptr(), rows, k, len(ws), ptrs(ws), ptrs(bs), ptrs(ys), _lib.i64_array([w.shape[0] for w in ws]),
+                                            _dtype_code(x), torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, "trifast_linear_fwd")
+    return ys
+
+
 class _Project(torch.autograd.Function):
-    """Several linear layers over one input.  Forward: the BLAS library's product per layer.
-    Backward: one pass for the input gradient of all layers (``trifast_linear_dx``), this
-    library's kernel for each weight gradient (``trifast_linear_dw``)."""
+    """Several linear layers over one input.  Forward: one pass over x for all layers
+    (``trifast_linear_fwd``).  Backward: one pass for the input gradient of all layers
+    (``trifast_linear_dx``), this library's kernel for each weight gradient
+    (``trifast_linear_dw``).  For 256 input channels the forward and the input gradient are the
+    BLAS library's products."""
 
     @staticmethod
     def forward(ctx, x, n_layers, *params):
@@ -157,6 +176,9 @@ class _Project(torch.autograd.Function):
         ctx.save_for_backward(x, *weights)
         ctx.has_bias = [b is not None for b in biases]
         ctx.set_materialize_grads(False)  # an unused output gives None, not a tensor of zeros to multiply
+        if x.shape[-1] in _DX_K:
+            ys = linear_outputs(x.reshape(-1, x.shape[-1]), weights, biases)
+            return tuple(y.view(*x.shape[:-1], y.shape[1]) for y in ys)
         return tuple(torch.nn.functional.linear(x, w, b) for w, b in zip(weights, biases))
 
     @staticmethod

@@ -163,6 +163,11 @@ def block(n: int, c_in: int) -> None:
             dx = dx + dy @ w  # (what autograd does with the layers' separate input gradients)
         return dx
 
+    nb_fwd = (sum(t.numel() for t in dys) + x2.numel()) * x2.element_size()
+    ms_fwd = _median_ms(lambda: nn.linear_outputs(x2, ws, [None] * len(ws)))
+    ms_fwd_blas = _median_ms(lambda: [torch.nn.functional.linear(x2, w) for w in ws])
+    print(f"the five projections of x              {ms_fwd * 1e3:8.1f} us  {nb_fwd / ms_fwd / 1e6:7.1f} GB/s of x and the outputs ({nb_fwd / 2**20:.0f} MiB); "
+          f"the BLAS library's five products {ms_fwd_blas * 1e3:8.1f} us")
     ms_blas = _median_ms(blas_dx)
     print(f"input gradient of the five projections {ms * 1e3:8.1f} us  {nbytes / ms / 1e6:7.1f} GB/s of the dy and dx ({nbytes / 2**20:.0f} MiB); "
           f"the BLAS library's five products and four additions {ms_blas * 1e3:8.1f} us")
