@@ -186,7 +186,9 @@ int trifast_bwd_one(int kernel,
  * Weight gradient of a linear layer over a pair representation: dw[n, k] = sum over r of
  * dy[r, n] x[r, k] for x [rows, k], dy [rows, n], dw [n, k], all dense, of one 16-bit dtype,
  * rows = b n^2 in the millions and k in {32, 64, 128, 256}: the rows are split over
- * workgroups, whose fp32 partials (the workspace) are added in a fixed order.  No counterpart
+ * workgroups, whose fp32 partials (the workspace) are added in a fixed order.  head_dim = 0:
+ * dy is [rows, n]; head_dim = d: dy is kept heads-outermost, [n / d][rows][d], the layout the
+ * attention operator takes q, k, v in (d a multiple of 8 that divides n).  No counterpart
  * in the reference, whose callers are only hinted at by the module of
  * tests/unit/test_trifast.py:152-169 (its q, k, v, bias linear layers, trained in :172-210).
  */
@@ -195,21 +197,22 @@ int64_t trifast_linear_dw_workspace_bytes(int64_t rows, int64_t k, int64_t n);
  * Up to 6 linear layers over the same pair representation in one pass that reads x once:
  * y_p = x W_p^T + bias_p for x [rows, k], W_p [n_p, k], bias_p [n_p] or null, y_p [rows, n_p]
  * (all dense, one 16-bit dtype, k in {32, 64, 128}).  w, bias, y, n are host arrays of nlayers
- * entries (bias itself may be null: no layer has one).  No counterpart in the reference (see
- * trifast_linear_dw).
+ * entries (bias itself may be null: no layer has one; head_dim may be null: every y_p is
+ * [rows, n_p]; head_dim[p] = d writes y_p heads-outermost, see trifast_linear_dw).  No counterpart
+ * in the reference (see trifast_linear_dw).
  */
 int trifast_linear_fwd(const void* x, int64_t rows, int64_t k, int nlayers, const void* const* w, const void* const* bias,
-                       void* const* y, const int64_t* n, int dtype, void* stream);
+                       void* const* y, const int64_t* n, const int64_t* head_dim, int dtype, void* stream);
 /*
  * Input gradient of up to 6 linear layers over the same pair representation in one pass:
  * dx[r, :] = sum over layers p of dy_p[r, :] W_p, with dy_p [rows, n_p] and the weights given
  * transposed, wt_p = W_p^T [k, n_p] (all dense, one 16-bit dtype, k in {32, 64, 128}); every
- * dy_p is read once and dx [rows, k] written once.  dy, wt, n are host arrays of nlayers
- * entries.  No counterpart in the reference (see trifast_linear_dw).
+ * dy_p is read once and dx [rows, k] written once.  dy, wt, n, head_dim are host arrays of
+ * nlayers entries (head_dim may be null; see trifast_linear_dw).  No counterpart in the reference (see trifast_linear_dw).
  */
 int trifast_linear_dx(void* dx, int64_t rows, int64_t k, int nlayers, const void* const* dy, const void* const* wt,
-                      const int64_t* n, int dtype, void* stream);
-int trifast_linear_dw(void* dw, const void* dy, const void* x, int64_t rows, int64_t k, int64_t n, int dtype,
+                      const int64_t* n, const int64_t* head_dim, int dtype, void* stream);
+int trifast_linear_dw(void* dw, const void* dy, const void* x, int64_t rows, int64_t k, int64_t n, int64_t head_dim, int dtype,
                       void* workspace, int64_t workspace_bytes, void* stream);
 
 /*

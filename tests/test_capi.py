@@ -127,13 +127,15 @@ def test_gate_argument_errors_come_back_as_codes():
 def test_weight_gradient_argument_errors_come_back_as_codes():
     lib = _lib.load()
     ok = 0x1000
-    call = lambda dw, dy, x, rows, k, n, dtype=_lib.BF16, ws=ok, nbytes=1 << 40: lib.trifast_linear_dw(dw, dy, x, rows, k, n, dtype, ws, nbytes, None)
+    call = lambda dw, dy, x, rows, k, n, dtype=_lib.BF16, ws=ok, nbytes=1 << 40, hd=0: lib.trifast_linear_dw(dw, dy, x, rows, k, n, hd, dtype, ws, nbytes, None)
     assert call(ok, ok, ok, 100, 48, 8) == -2 and "input channels" in _lib.last_error()
     assert call(ok, ok, ok, 100, 64, 8, _lib.F32) == -2 and "16-bit" in _lib.last_error()
     assert call(ok, ok, ok, 0, 64, 8) == -1 and "positive" in _lib.last_error()
     assert call(None, ok, ok, 100, 64, 8) == -1 and "null" in _lib.last_error()
     assert call(ok, ok + 8, ok, 100, 64, 8) == -3 and "aligned" in _lib.last_error()
     assert call(ok, ok, ok, 100, 64, 8, nbytes=16) == -4 and "workspace" in _lib.last_error()
+    assert call(ok, ok, ok, 100, 64, 48, hd=32) == -1 and "head dim" in _lib.last_error()  # 32 does not divide 48
+    assert call(ok, ok, ok, 100, 64, 48, hd=12) == -1 and "head dim" in _lib.last_error()  # not a multiple of 8
     # the partials: one [n, k] fp32 matrix per chunk of at least 1024 rows, at most 768 chunks
     assert lib.trifast_linear_dw_workspace_bytes(1024, 128, 128) == 128 * 128 * 4
     assert lib.trifast_linear_dw_workspace_bytes(3000, 128, 128) == 3 * 128 * 128 * 4
@@ -149,7 +151,7 @@ def test_linear_forward_argument_errors_come_back_as_codes():
     ok = 0x1000
     vp = lambda *v: (ctypes.c_void_p * len(v))(*v)
     n1 = _lib.i64_array([8])
-    call = lambda x, k, nl, w, y, n, dtype=_lib.BF16, rows=4: lib.trifast_linear_fwd(x, rows, k, nl, w, None, y, n, dtype, None)
+    call = lambda x, k, nl, w, y, n, dtype=_lib.BF16, rows=4, hd=None: lib.trifast_linear_fwd(x, rows, k, nl, w, None, y, n, hd, dtype, None)
     assert call(ok, 256, 1, vp(ok), vp(ok), n1) == -2 and "input channels" in _lib.last_error()
     assert call(ok, 64, 1, vp(ok), vp(ok), n1, _lib.F32) == -2 and "16-bit" in _lib.last_error()
     assert call(ok, 64, 7, vp(*[ok] * 7), vp(*[ok] * 7), _lib.i64_array([8] * 7)) == -1 and "layers per call" in _lib.last_error()
@@ -157,6 +159,7 @@ def test_linear_forward_argument_errors_come_back_as_codes():
     assert call(ok, 64, 1, vp(ok), vp(ok + 4), n1) == -3 and "layer 0" in _lib.last_error()
     assert call(ok, 64, 1, vp(None), vp(ok), n1) == -1 and "null" in _lib.last_error()
     assert call(ok, 64, 1, vp(ok), vp(ok), n1, rows=0) == -1 and "rows" in _lib.last_error()
+    assert call(ok, 64, 1, vp(ok), vp(ok), n1, hd=_lib.i64_array([16])) == -1 and "head dim" in _lib.last_error()
 
 
 def test_input_gradient_argument_errors_come_back_as_codes():
@@ -166,7 +169,7 @@ def test_input_gradient_argument_errors_come_back_as_codes():
     ok = 0x1000
     vp = lambda *v: (ctypes.c_void_p * len(v))(*v)
     n1 = _lib.i64_array([8])
-    call = lambda dx, k, nl, dy, wt, n, dtype=_lib.BF16, rows=4: lib.trifast_linear_dx(dx, rows, k, nl, dy, wt, n, dtype, None)
+    call = lambda dx, k, nl, dy, wt, n, dtype=_lib.BF16, rows=4, hd=None: lib.trifast_linear_dx(dx, rows, k, nl, dy, wt, n, hd, dtype, None)
     assert call(ok, 256, 1, vp(ok), vp(ok), n1) == -2 and "input channels" in _lib.last_error()
     assert call(ok, 64, 1, vp(ok), vp(ok), n1, _lib.F32) == -2 and "16-bit" in _lib.last_error()
     assert call(ok, 64, 7, vp(*[ok] * 7), vp(*[ok] * 7), _lib.i64_array([8] * 7)) == -1 and "layers per call" in _lib.last_error()
@@ -175,6 +178,7 @@ def test_input_gradient_argument_errors_come_back_as_codes():
     assert call(ok, 64, 1, vp(None), vp(ok), n1) == -1 and "null" in _lib.last_error()
     assert call(ok, 64, 1, vp(ok), vp(ok), _lib.i64_array([0])) == -1 and "outputs" in _lib.last_error()
     assert call(ok, 64, 1, vp(ok), vp(ok), n1, rows=0) == -1 and "rows" in _lib.last_error()
+    assert call(ok, 64, 1, vp(ok), vp(ok), n1, hd=_lib.i64_array([16])) == -1 and "head dim" in _lib.last_error()
 
 
 def test_gated_output_checks_shapes_on_the_host():
@@ -194,6 +198,10 @@ def test_gated_output_checks_shapes_on_the_host():
     # linear layers over CPU tensors are torch's own
     assert nn.linear(torch.zeros(2, 24), block.b).shape == (2, 2)
     assert [t.shape for t in nn.project(torch.zeros(2, 24), (block.q, block.b))] == [(2, 32), (2, 2)]
+    # heads-outermost outputs: [h, *, d]; on tensors the kernels do not take, a permuted copy
+    assert [t.shape for t in nn.project(torch.zeros(3, 5, 24), (block.q, block.b), (16, 0))] == [(2, 3, 5, 16), (3, 5, 2)]
+    with pytest.raises(ValueError, match="no bias"):
+        nn.project(torch.zeros(2, 24), (block.g,), (16,))
     assert {n for n, _ in block.named_parameters()} == {"q.weight", "k.weight", "v.weight", "b.weight", "g.weight", "g.bias", "out.weight", "out.bias"}
 
 

@@ -256,3 +256,52 @@ def test_projection_gradients_are_those_of_the_layers():
             assert (a is None) == (r is None)
             if a is not None:
                 assert (a - r).abs().max().item() <= 2.0**-7 * r.abs().max().item(), f"{(a - r).abs().max().item():.3e} of {r.abs().max().item():.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_heads_outermost_layers(dtype):
+    """Layers whose outputs are kept [h, rows, d]: the forward writes that layout, the input and
+    weight gradients read it; everything equals the plain-layout kernels on permuted copies, bit
+    for bit (the same products in the same order)."""
+    gen = torch.Generator().manual_seed(11)
+    rows, k, h, d = 4099, 128, 4, 32
+    x = torch.randn(rows, k, generator=gen).to(DEV, dtype)
+    ws = [(torch.randn(n, k, generator=gen) * k**-0.5).to(DEV, dtype) for n in (h * d, 4, 2 * 64)]
+    hds = (d, 0, 64)
+    ys = nn.linear_outputs(x, ws, [None] * 3, hds)
+    plain = nn.linear_outputs(x, ws, [None] * 3)
+    to_heads = lambda t, hd: t.unflatten(-1, (-1, hd)).movedim(-2, 0).contiguous() if hd else t
+    for y, p, hd in zip(ys, plain, hds):
+        assert y.shape == to_heads(p, hd).shape and torch.equal(y, to_heads(p, hd))
+    dys = [torch.randn(rows, w.shape[0], generator=gen).to(DEV, dtype) for w in ws]
+    dys_h = [to_heads(t, hd) for t, hd in zip(dys, hds)]
+    assert torch.equal(nn.linear_input_grad(dys_h, ws, hds), nn.linear_input_grad(dys, ws))
+    for t, th, hd in zip(dys, dys_h, hds):
+        assert torch.equal(nn.linear_weight_grad(th, x, hd), nn.linear_weight_grad(t, x))
+
+
+def test_projection_with_heads_outermost_outputs():
+    """project(..., head_dims) through autograd against the layers themselves."""
+    torch.manual_seed(8)
+    dtype, h, d = torch.bfloat16, 2, 32
+    x = torch.randn(2, 30, 30, 64, device=DEV, dtype=dtype)
+    layers = [torch.nn.Linear(64, h * d, bias=False).to(DEV, dtype), torch.nn.Linear(64, 32, bias=True).to(DEV, dtype)]
+    dys = [torch.randn(2, 30, 30, m.out_features, device=DEV, dtype=dtype) for m in layers]
+
+    def grads(fn):
+        xi = x.clone().requires_grad_(True)
+        for m in layers:
+            m.zero_grad()
+        outs = fn(xi)
+        torch.autograd.backward(outs, dys)
+        return [o.detach().float() for o in outs], [xi.grad.float()] + [p.grad.float().clone() for m in layers for p in m.parameters()]
+
+    def ours(xi):
+        q, g = nn.project(xi, layers, (d, 0))
+        assert q.shape == (h, 2, 30, 30, d) and q.is_contiguous()
+        return [q.movedim(0, -2).flatten(-2), g]  # back to [*, h * d] for the comparison
+
+    (o1, g1), (o2, g2) = grads(ours), grads(lambda xi: [m(xi) for m in layers])
+    for a, r in zip(o1 + g1, o2 + g2):
+        assert a.shape == r.shape
+        assert (a - r).abs().max().item() <= 2.0**-7 * r.abs().max().item(), f"{(a - r).abs().max().item():.3e} of {r.abs().max().item():.3e}"

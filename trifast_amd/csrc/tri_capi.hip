@@ -624,14 +624,22 @@ int gate_impl(bool bwd, void* y_or_dg, void* dox, const void* dy, const void* o,
 }
 }  // namespace
 
+// head dim of a layer whose output is kept heads-outermost (0: plain [rows, n])
+static int check_linear_head(const char* what, int p, int64_t n, int64_t hd) {
+  if (hd == 0) return 0;
+  if (hd < 8 || hd % 8 != 0 || n % hd != 0) return fail(TRIFAST_EINVAL, "%s: layer %d: head dim %lld must be a multiple of 8 that divides its %lld outputs", what, p, (long long)hd, (long long)n);
+  return 0;
+}
+
 int64_t trifast_linear_dw_workspace_bytes(int64_t rows, int64_t k, int64_t n) {
   if (rows < 1 || k < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
   return align256(tri::linear_dw_chunks(rows) * n * k * 4);
 }
 
-int trifast_linear_dw(void* dw, const void* dy, const void* x, int64_t rows, int64_t k, int64_t n, int dtype,
+int trifast_linear_dw(void* dw, const void* dy, const void* x, int64_t rows, int64_t k, int64_t n, int64_t head_dim, int dtype,
                       void* workspace, int64_t workspace_bytes, void* stream) {
   g_err[0] = 0;
+  if (int rc = check_linear_head("linear_dw", 0, n, head_dim)) return rc;
   if (dtype != TRIFAST_BF16 && dtype != TRIFAST_F16) return fail(TRIFAST_EUNSUPPORTED, "linear_dw: 16-bit element types only (dtype code %d)", dtype);
   if (rows < 1 || n < 1 || n > 65535 * 128) return fail(TRIFAST_EINVAL, "linear_dw: rows and n must be positive (rows=%lld n=%lld)", (long long)rows, (long long)n);
   if (!tri::linear_dw_k_ok(k)) return fail(TRIFAST_EUNSUPPORTED, "linear_dw: %lld input channels (32, 64, 128 or 256 are compiled)", (long long)k);
@@ -643,14 +651,14 @@ int trifast_linear_dw(void* dw, const void* dy, const void* x, int64_t rows, int
   tri::LinearDwArgs a{};
   a.x = x; a.dy = dy; a.dw = dw; a.part = static_cast<float*>(workspace);
   a.rows = rows; a.rows_per_chunk = tri::linear_dw_rows_per_chunk(rows); a.chunks = (int)tri::linear_dw_chunks(rows);
-  a.K = (int)k; a.N = (int)n;
+  a.K = (int)k; a.N = (int)n; a.hd = (int)head_dim;
   const hipError_t e = tri::linear_dw_launch(a, dtype, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "linear_dw launch");
   return 0;
 }
 
 int trifast_linear_fwd(const void* x, int64_t rows, int64_t k, int nlayers, const void* const* w, const void* const* bias,
-                       void* const* y, const int64_t* n, int dtype, void* stream) {
+                       void* const* y, const int64_t* n, const int64_t* head_dim, int dtype, void* stream) {
   g_err[0] = 0;
   if (dtype != TRIFAST_BF16 && dtype != TRIFAST_F16) return fail(TRIFAST_EUNSUPPORTED, "linear_fwd: 16-bit element types only (dtype code %d)", dtype);
   if (rows < 1) return fail(TRIFAST_EINVAL, "linear_fwd: rows must be positive (%lld)", (long long)rows);
@@ -665,7 +673,8 @@ int trifast_linear_fwd(const void* x, int64_t rows, int64_t k, int nlayers, cons
     if (n[p] < 1 || n[p] > (1 << 20)) return fail(TRIFAST_EINVAL, "linear_fwd: layer %d: %lld outputs", p, (long long)n[p]);
     if ((reinterpret_cast<uintptr_t>(w[p]) & 15) != 0 || (reinterpret_cast<uintptr_t>(y[p]) & 15) != 0)
       return fail(TRIFAST_EALIGN, "linear_fwd: layer %d: weight and output must be 16-byte aligned", p);
-    a.w[p] = w[p]; a.bias[p] = bias ? bias[p] : nullptr; a.y[p] = y[p]; a.n[p] = (int)n[p];
+    if (int rc = check_linear_head("linear_fwd", p, n[p], head_dim ? head_dim[p] : 0)) return rc;
+    a.w[p] = w[p]; a.bias[p] = bias ? bias[p] : nullptr; a.y[p] = y[p]; a.n[p] = (int)n[p]; a.hd[p] = head_dim ? (int)head_dim[p] : 0;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   const hipError_t e = dtype == TRIFAST_BF16 ? tri::linear_fwd_launch_t<__bf16>(a, st) : tri::linear_fwd_launch_t<_Float16>(a, st);
@@ -674,7 +683,7 @@ int trifast_linear_fwd(const void* x, int64_t rows, int64_t k, int nlayers, cons
 }
 
 int trifast_linear_dx(void* dx, int64_t rows, int64_t k, int nlayers, const void* const* dy, const void* const* wt,
-                      const int64_t* n, int dtype, void* stream) {
+                      const int64_t* n, const int64_t* head_dim, int dtype, void* stream) {
   g_err[0] = 0;
   if (dtype != TRIFAST_BF16 && dtype != TRIFAST_F16) return fail(TRIFAST_EUNSUPPORTED, "linear_dx: 16-bit element types only (dtype code %d)", dtype);
   if (rows < 1) return fail(TRIFAST_EINVAL, "linear_dx: rows must be positive (%lld)", (long long)rows);
@@ -689,7 +698,8 @@ int trifast_linear_dx(void* dx, int64_t rows, int64_t k, int nlayers, const void
     if (n[p] < 1 || n[p] > (1 << 20)) return fail(TRIFAST_EINVAL, "linear_dx: layer %d: %lld outputs", p, (long long)n[p]);
     if ((reinterpret_cast<uintptr_t>(dy[p]) & 15) != 0 || (reinterpret_cast<uintptr_t>(wt[p]) & 15) != 0)
       return fail(TRIFAST_EALIGN, "linear_dx: layer %d: dy and the transposed weight must be 16-byte aligned", p);
-    a.dy[p] = dy[p]; a.wt[p] = wt[p]; a.n[p] = (int)n[p];
+    if (int rc = check_linear_head("linear_dx", p, n[p], head_dim ? head_dim[p] : 0)) return rc;
+    a.dy[p] = dy[p]; a.wt[p] = wt[p]; a.n[p] = (int)n[p]; a.hd[p] = head_dim ? (int)head_dim[p] : 0;
   }
   const hipError_t e = tri::linear_dx_launch(a, dtype, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "linear_dx launch");

@@ -20,9 +20,18 @@
 
 namespace tri {
 
+// A layer's output (or output gradient) is [rows, N] or, "heads outermost", [N / hd][rows][hd]:
+// the layout the attention operator reads q, k, v in (and writes dq, dk, dv in) without the
+// two heads of a 128-byte line belonging to different workgroups.  hd = 0: plain.
+// (hd is a multiple of 8 and divides N, so a 16-byte piece never straddles two heads.)
+TRI_DEV int64_t linear_offset(int64_t row, int col, int N, int hd, int64_t rows) {
+  return hd ? ((int64_t)(col / hd) * rows + row) * hd + col % hd : row * N + col;
+}
+
 struct LinearDwArgs {
   const void* x;    // [rows, K]
-  const void* dy;   // [rows, N]
+  const void* dy;   // [rows, N] (see linear_offset)
+  int hd;
   float* part;      // [chunks, N, K] partial sums
   void* dw;         // [N, K]
   int64_t rows;
@@ -91,7 +100,7 @@ __global__ __launch_bounds__(256) void linear_dw_kernel(const LinearDwArgs a) {
       const int p = c * 256 + tid, r = p / (ND / 8), col = n_grp + 8 * (p % (ND / 8));
       vec v = {};
       if (p < YCH && r0 + r < r_end && col < N) {
-        const T* src = yg + (r0 + r) * N + col;
+        const T* src = yg + linear_offset(r0 + r, col, N, a.hd, a.rows);
         if (y_vec) {
           v = *reinterpret_cast<const vec*>(src);
         } else {
@@ -253,9 +262,10 @@ namespace tri {
 constexpr int kLinearLayers = 6;
 
 struct LinearDxArgs {
-  const void* dy[kLinearLayers];   // [rows, n[p]]
+  const void* dy[kLinearLayers];   // [rows, n[p]] (see linear_offset)
   const void* wt[kLinearLayers];   // [K, n[p]]: W_p transposed
   int n[kLinearLayers];
+  int hd[kLinearLayers];
   int nlayers;
   void* dx;                        // [rows, K]
   int64_t rows;
@@ -323,7 +333,7 @@ __global__ __launch_bounds__(256) void linear_dx_kernel(const LinearDxArgs a) {
       const int q = x * 256 + tid, r = q / 4, col = 32 * cur.c + 8 * (q % 4);
       vec v = {};
       if (row0 + r < a.rows && col < N) {
-        const T* s = src + (row0 + r) * N + col;
+        const T* s = src + linear_offset(row0 + r, col, N, a.hd[cur.p], a.rows);
         if (vec_ok) {
           v = *reinterpret_cast<const vec*>(s);
         } else {
@@ -448,8 +458,9 @@ struct LinearFwdArgs {
   const void* x;                    // [rows, K]
   const void* w[kLinearLayers];     // [n[p], K]
   const void* bias[kLinearLayers];  // [n[p]] or null
-  void* y[kLinearLayers];           // [rows, n[p]]
+  void* y[kLinearLayers];           // [rows, n[p]] (see linear_offset)
   int n[kLinearLayers];
+  int hd[kLinearLayers];
   int nlayers;
   int64_t rows;
   int K;
@@ -587,7 +598,7 @@ __global__ __launch_bounds__(256) void linear_fwd_kernel(const LinearFwdArgs a) 
       const int64_t row = row0 + r;
       const vec v = *reinterpret_cast<const vec*>(&os[r][8 * (idx % 4)]);
       if (row < a.rows && col < N) {
-        T* dst = y + row * N + col;
+        T* dst = y + linear_offset(row, col, N, a.hd[use.p], a.rows);
         if ((N % 8) == 0) {
           *reinterpret_cast<vec*>(dst) = v;
         } else {

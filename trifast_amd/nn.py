@@ -90,17 +90,24 @@ def _dw_ready(x: torch.Tensor, weight: torch.Tensor) -> bool:
     return x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and weight.dtype == x.dtype and x.shape[-1] in _DW_K and x.numel() > 0
 
 
-def linear_weight_grad(dy: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+def _rows_n(dy: torch.Tensor, head_dim: int) -> tuple[int, int]:
+    """rows and outputs of a layer's output gradient: ``[rows, n]``, or ``[n / head_dim, rows,
+    head_dim]`` for a layer kept heads-outermost."""
+    return (dy.shape[1], dy.shape[0] * dy.shape[2]) if head_dim else (dy.shape[0], dy.shape[1])
+
+
+def linear_weight_grad(dy: torch.Tensor, x: torch.Tensor, head_dim: int = 0) -> torch.Tensor:
     """``dy^T x`` for ``dy [rows, n]``, ``x [rows, k]``: the weight gradient of a linear layer, with
-    the long contraction over the rows split over the whole GPU (``trifast_linear_dw``)."""
+    the long contraction over the rows split over the whole GPU (``trifast_linear_dw``).  With
+    ``head_dim = d``, dy is ``[n / d, rows, d]`` (heads outermost)."""
     dy, x = dy.contiguous(), x.contiguous()
-    rows, n = dy.shape
+    rows, n = _rows_n(dy, head_dim)
     k = x.shape[1]
     lib = _lib.load()
     dw = torch.empty(n, k, dtype=x.dtype, device=x.device)
     ws = torch.empty(lib.trifast_linear_dw_workspace_bytes(rows, k, n), dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
-        rc = lib.trifast_linear_dw(dw.data_ptr(), dy.data_ptr(), x.data_ptr(), rows, k, n, _dtype_code(x), ws.data_ptr(), ws.numel(),
+        rc = lib.trifast_linear_dw(dw.data_ptr(), dy.data_ptr(), x.data_ptr(), rows, k, n, head_dim, _dtype_code(x), ws.data_ptr(), ws.numel(),
                                    torch.cuda.current_stream(x.device).cuda_stream)
     _lib.check(rc, "trifast_linear_dw")
     return dw
@@ -131,34 +138,37 @@ _DX_K = (32, 64, 128)
 _DX_LAYERS = 6
 
 
-def linear_input_grad(dys, weights) -> torch.Tensor:
+def linear_input_grad(dys, weights, head_dims=None) -> torch.Tensor:
     """``sum_p dys[p] @ weights[p]`` for ``dys[p] [rows, n_p]``, ``weights[p] [n_p, k]``: the input
     gradient of several linear layers over one input, every ``dys[p]`` read once and the sum
-    written once (``trifast_linear_dx``)."""
+    written once (``trifast_linear_dx``).  ``head_dims[p] = d``: ``dys[p]`` is ``[n_p / d, rows, d]``."""
+    head_dims = list(head_dims) if head_dims is not None else [0] * len(dys)
     dys = [dy.contiguous() for dy in dys]
     wts = [w.t().contiguous() for w in weights]  # [k, n_p]: a few tens of KiB each
-    rows, k = dys[0].shape[0], weights[0].shape[1]
+    rows, k = _rows_n(dys[0], head_dims[0])[0], weights[0].shape[1]
     dx = torch.empty(rows, k, dtype=dys[0].dtype, device=dys[0].device)
     ptrs = lambda ts: (_lib.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
     with torch.cuda.device(dx.device):
-        rc = _lib.load().trifast_linear_dx(dx.data_ptr(), rows, k, len(dys), ptrs(dys), ptrs(wts), _lib.i64_array([dy.shape[1] for dy in dys]),
-                                           _dtype_code(dx), torch.cuda.current_stream(dx.device).cuda_stream)
+        rc = _lib.load().trifast_linear_dx(dx.data_ptr(), rows, k, len(dys), ptrs(dys), ptrs(wts), _lib.i64_array([w.shape[0] for w in weights]),
+                                           _lib.i64_array(head_dims), _dtype_code(dx), torch.cuda.current_stream(dx.device).cuda_stream)
     _lib.check(rc, "trifast_linear_dx")
     return dx
 
 
-def linear_outputs(x: torch.Tensor, weights, biases) -> list[torch.Tensor]:
+def linear_outputs(x: torch.Tensor, weights, biases, head_dims=None) -> list[torch.Tensor]:
     """``[x @ w.T + b for w, b in zip(weights, biases)]`` for ``x [rows, k]`` in one pass that reads
-    x once (``trifast_linear_fwd``); a bias may be None."""
+    x once (``trifast_linear_fwd``); a bias may be None.  ``head_dims[p] = d``: output p comes
+    heads-outermost, ``[n_p / d, rows, d]``."""
+    head_dims = list(head_dims) if head_dims is not None else [0] * len(weights)
     x = x.contiguous()
     rows, k = x.shape
     ws = [w.contiguous() for w in weights]
     bs = [None if b is None else b.contiguous() for b in biases]
-    ys = [torch.empty(rows, w.shape[0], dtype=x.dtype, device=x.device) for w in ws]
+    ys = [torch.empty((w.shape[0] // d, rows, d) if d else (rows, w.shape[0]), dtype=x.dtype, device=x.device) for w, d in zip(ws, head_dims)]
     ptrs = lambda ts: (_lib.c_void_p * len(ts))(*[None if t is None else t.data_ptr() for t in ts])
     with torch.cuda.device(x.device):
         rc = _lib.load().trifast_linear_fwd(x.data_ptr(), rows, k, len(ws), ptrs(ws), ptrs(bs), ptrs(ys), _lib.i64_array([w.shape[0] for w in ws]),
-                                            _dtype_code(x), torch.cuda.current_stream(x.device).cuda_stream)
+                                            _lib.i64_array(head_dims), _dtype_code(x), torch.cuda.current_stream(x.device).cuda_stream)
     _lib.check(rc, "trifast_linear_fwd")
     return ys
 
@@ -167,46 +177,62 @@ class _Project(torch.autograd.Function):
     """Several linear layers over one input.  Forward: one pass over x for all layers
     (``trifast_linear_fwd``).  Backward: one pass for the input gradient of all layers
     (``trifast_linear_dx``), this library's kernel for each weight gradient
-    (``trifast_linear_dw``).  For 256 input channels the forward and the input gradient are the
-    BLAS library's products."""
+    (``trifast_linear_dw``).  Layers with a head dim give their output heads-outermost,
+    ``[n / d, *x.shape[:-1], d]``.  For 256 input channels the forward and the input gradient
+    are the BLAS library's products (and every output is plain)."""
 
     @staticmethod
-    def forward(ctx, x, n_layers, *params):
+    def forward(ctx, x, head_dims, *params):
+        n_layers = len(head_dims)
         weights, biases = params[:n_layers], params[n_layers:]
         ctx.save_for_backward(x, *weights)
         ctx.has_bias = [b is not None for b in biases]
+        ctx.head_dims = head_dims
         ctx.set_materialize_grads(False)  # an unused output gives None, not a tensor of zeros to multiply
+        lead = x.shape[:-1]
         if x.shape[-1] in _DX_K:
-            ys = linear_outputs(x.reshape(-1, x.shape[-1]), weights, biases)
-            return tuple(y.view(*x.shape[:-1], y.shape[1]) for y in ys)
+            ys = linear_outputs(x.reshape(-1, x.shape[-1]), weights, biases, head_dims)
+            return tuple(y.view(y.shape[0], *lead, d) if d else y.view(*lead, y.shape[1]) for y, d in zip(ys, head_dims))
         return tuple(torch.nn.functional.linear(x, w, b) for w, b in zip(weights, biases))
 
     @staticmethod
     def backward(ctx, *dys):
         x, *weights = ctx.saved_tensors
         x2 = x.reshape(-1, x.shape[-1])
-        # (a layer whose output took no part in the loss has no gradient to give)
-        live = [(dy.reshape(-1, dy.shape[-1]), w) for dy, w in zip(dys, weights) if dy is not None]
+        # two dims per layer ([rows, n], or [n / d, rows, d] for a heads-outermost layer); a layer
+        # whose output took no part in the loss has no gradient to give
+        flat = [None if dy is None else (dy.reshape(dy.shape[0], -1, d) if d else dy.reshape(-1, dy.shape[-1])) for dy, d in zip(dys, ctx.head_dims)]
+        live = [(dy, w, d) for dy, w, d in zip(flat, weights, ctx.head_dims) if dy is not None]
         dx = None
         if ctx.needs_input_grad[0] and live:
             if x.shape[-1] in _DX_K:
-                dx = linear_input_grad([dy for dy, _ in live], [w for _, w in live]).view(x.shape)
+                dx = linear_input_grad([t[0] for t in live], [t[1] for t in live], [t[2] for t in live]).view(x.shape)
             else:
-                dx = sum(dy @ w for dy, w in live).view(x.shape)
-        dws = [None if dy is None else linear_weight_grad(dy.reshape(-1, dy.shape[-1]), x2) for dy in dys]
-        dbs = [dy.reshape(-1, dy.shape[-1]).sum(0) if (dy is not None and has) else None for dy, has in zip(dys, ctx.has_bias)]
+                dx = sum(dy @ w for dy, w, _ in live).view(x.shape)
+        dws = [None if dy is None else linear_weight_grad(dy, x2, d) for dy, d in zip(flat, ctx.head_dims)]
+        dbs = [dy.sum(0) if (dy is not None and has) else None for dy, has in zip(flat, ctx.has_bias)]  # (a layer with a bias is plain)
         return (dx, None, *dws, *dbs)
 
 
-def project(x: torch.Tensor, layers) -> tuple[torch.Tensor, ...]:
+def project(x: torch.Tensor, layers, head_dims=None) -> tuple[torch.Tensor, ...]:
     """``tuple(layer(x) for layer in layers)`` for up to 6 ``torch.nn.Linear`` layers over the
-    same pair representation ``x [*, k]``, with a backward that reads every output gradient
-    once for the input gradient and computes the weight gradients with this library's kernel
-    (GPU, 16-bit, k in (32, 64, 128, 256)); anything else is the layers themselves."""
+    same pair representation ``x [*, k]``: one pass over x, and a backward that reads every
+    output gradient once for the input gradient and computes the weight gradients with this
+    library's kernel (GPU, 16-bit, k in (32, 64, 128); k = 256: the weight gradients only);
+    anything else is the layers themselves.
+
+    ``head_dims[p] = d`` (a bias-free layer of ``h * d`` outputs) returns output p as
+    ``[h, *x.shape[:-1], d]``, heads outermost, which is how the attention operator reads q, k, v
+    fastest; the kernels write and read that layout directly (elsewhere it is a copy)."""
     layers = list(layers)
-    if not layers or len(layers) > _DX_LAYERS or not all(_dw_ready(x, m.weight) for m in layers):
-        return tuple(m(x) for m in layers)
-    return _Project.apply(x, len(layers), *[m.weight for m in layers], *[m.bias for m in layers])
+    head_dims = tuple(head_dims) if head_dims is not None else (0,) * len(layers)
+    if any(d and m.bias is not None for m, d in zip(layers, head_dims)):
+        raise ValueError("a heads-outermost layer takes no bias")
+    fused = bool(layers) and len(layers) <= _DX_LAYERS and all(_dw_ready(x, m.weight) for m in layers)
+    if not fused or x.shape[-1] not in _DX_K:
+        ys = _Project.apply(x, (0,) * len(layers), *[m.weight for m in layers], *[m.bias for m in layers]) if fused else tuple(m(x) for m in layers)
+        return tuple(y.unflatten(-1, (-1, d)).movedim(-2, 0).contiguous() if d else y for y, d in zip(ys, head_dims))
+    return _Project.apply(x, head_dims, *[m.weight for m in layers], *[m.bias for m in layers])
 
 
 def linear(x: torch.Tensor, layer: torch.nn.Linear) -> torch.Tensor:
@@ -239,7 +265,8 @@ class TriangleAttention(torch.nn.Module):
         return t.unflatten(-1, (self.h, self.d)).movedim(-2, -4)
 
     def forward(self, x: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
-        q, k, v, bias, g = project(x, (self.q, self.k, self.v, self.b, self.g))
+        # q, k, v come heads-outermost, [h, *, n, n, d]: the operator's fastest input layout
+        q, k, v, bias, g = project(x, (self.q, self.k, self.v, self.b, self.g), (self.d, self.d, self.d, 0, 0))
         attend = triangle_attention_ending_node if self.ending_node else triangle_attention
-        o = attend(self.heads(q), self.heads(k), self.heads(v), bias.movedim(-1, -3), mask)
+        o = attend(q.movedim(0, -4), k.movedim(0, -4), v.movedim(0, -4), bias.movedim(-1, -3), mask)
         return linear(gated_output(o, g), self.out)
