@@ -5,11 +5,13 @@ The reference ships the operator only; its tests hint at the surrounding module
 a pair representation ``x [*, n, n, c]``).  This module is that block written so that no
 tensor is copied to change its layout:
 
-* q, k, v leave their linear layers as ``[*, n, n, h*d]`` and go to the operator as
-  ``[*, h, n, n, d]`` *views* (heads interleaved, 64-byte rows for d = 32 bf16); the bias
-  as a ``[*, h, n, n]`` view of ``[*, n, n, h]``.  The operator reads them through their
-  strides and writes dq, dk, dv, db with the same strides, so autograd needs no re-layout
-  copy on the way back either.
+* q, k, v are written by their projection heads-outermost, ``[h, *, n, n, d]``, and go to the
+  operator as ``[*, h, n, n, d]`` views: its fastest layout (interleaved heads, which is what
+  separate linear layers produce, share every 128-byte line between two heads); the bias as a
+  ``[*, h, n, n]`` view of ``[*, n, n, h]``.  The operator reads them through their strides
+  and writes dq, dk, dv, db with the same strides, so autograd needs no re-layout copy on the
+  way back either, and the projections' backward reads the heads-outermost gradients as
+  they are.
 * The weight gradients of the six linear layers come from ``trifast_linear_dw``: for rows in
   the millions and a few hundred channels the BLAS library runs that product (a contraction
   over all rows into a tiny matrix) on one or two workgroups, ten times slower than the
