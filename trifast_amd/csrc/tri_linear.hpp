@@ -449,7 +449,7 @@ namespace tri {
 // x is read once for all layers (the BLAS library reads it once per layer).  A workgroup
 // owns 256 rows: their K / 16 operand fragments go through LDS once (coalesced loads) into
 // registers (wave w: rows 64 w .. 64 w + 63 as two 32-row tiles) and stay there; the layers'
-// weights pass through LDS 32 output columns at a time (one stage ahead in registers).  The
+// weights pass through LDS 128 output columns at a time (the next group ahead in registers).  The
 // product is computed transposed (W x^T, bias as accumulator init), so a lane holds one row
 // and 4 x 4 consecutive columns of the chunk; the chunk goes back through the wave's own
 // piece of LDS and leaves as 16-byte pieces, 64 contiguous bytes per row.
@@ -466,10 +466,10 @@ struct LinearFwdArgs {
   int K;
 };
 
-// LDS of the kernel below: the x tile, or what takes its place (two weight chunks and the
+// LDS of the kernel below: the x tile, or what takes its place (128 weight rows and the
 // output chunk), whichever is larger
 constexpr int linear_fwd_lds_bytes(int kd, int es) {
-  const int xbytes = 256 * (kd + 8) * es, cbytes = 2 * 32 * (kd + 8) * es + 256 * (32 + 8) * es;
+  const int xbytes = 256 * (kd + 8) * es, cbytes = 128 * (kd + 8) * es + 256 * (32 + 8) * es;
   return xbytes > cbytes ? xbytes : cbytes;
 }
 
@@ -483,15 +483,10 @@ __global__ __launch_bounds__(256) void linear_fwd_kernel(const LinearFwdArgs a) 
   constexpr int LDX = KD + 8;        // padded row of the x tile and of a weight chunk
   constexpr int LDO = 32 + 8;        // padded row of an output chunk
   constexpr int XP = ROWS * KD / 8 / 256;  // 16-byte pieces of the x tile per lane
-  constexpr int WPC = 32 * KD / 8;   // ... of a weight chunk (32 rows of W)
-  constexpr int WCH = (WPC + 255) / 256;
-  // LDS: first the x tile; once its fragments are in registers, two weight chunks and the
-  // output chunk take its place
+  // LDS: first the x tile; once its fragments are in registers, a group of weight rows and
+  // the output chunk take its place
   extern __shared__ __attribute__((aligned(16))) unsigned char lin_smem[];
   T (*xs)[LDX] = reinterpret_cast<T (*)[LDX]>(lin_smem);
-  T (*wsm)[32][LDX] = reinterpret_cast<T (*)[32][LDX]>(lin_smem);                       // [2][32][LDX]
-  T (*os)[LDO] = reinterpret_cast<T (*)[LDO]>(lin_smem + 2 * 32 * LDX * sizeof(T));      // [ROWS][LDO]
-  static_assert(2 * 32 * LDX * sizeof(T) + ROWS * LDO * sizeof(T) <= linear_fwd_lds_bytes(KD, (int)sizeof(T)), "the launcher sizes LDS with linear_fwd_lds_bytes");
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -523,98 +518,107 @@ __global__ __launch_bounds__(256) void linear_fwd_kernel(const LinearFwdArgs a) 
     for (int s = 0; s < KS; ++s) xf[t][s] = *reinterpret_cast<const frag*>(&xs[64 * wave + 32 * t + cl][16 * s + 8 * g]);
   __syncthreads();
 
+  // The weights pass through LDS in groups of up to 128 output columns (four chunks of 32): the
+  // next group waits in registers while this one is used, and takes its place between two
+  // barriers.  (Loads and stores share one counter of operations in flight, and a wait for a
+  // load is in effect a wait for the stores issued before it: staging every chunk of 32
+  // columns separately made each chunk wait for the output stores of the one before.)
+  constexpr int GROUP = 128;
+  constexpr int GP = GROUP * KD / 8 / 256;  // 16-byte pieces of a group per lane
   int total = 0;
-  for (int p = 0; p < a.nlayers; ++p) total += (a.n[p] + 31) / 32;
+  for (int p = 0; p < a.nlayers; ++p) total += (a.n[p] + GROUP - 1) / GROUP;
   struct Cursor {
-    int p, c;
+    int p, c;  // layer, group of 128 columns inside it
   };
   auto advance = [&](Cursor& cur) {
-    if (32 * (cur.c + 1) < a.n[cur.p]) ++cur.c;
+    if (GROUP * (cur.c + 1) < a.n[cur.p]) ++cur.c;
     else { ++cur.p; cur.c = 0; }
   };
-  // rows 32 c .. 32 c + 31 of W_p (rows past N_p are zero)
-  vec wr[2][WCH];
-  auto load_chunk = [&](const Cursor& cur, vec* dst) {
+  T (*wg)[LDX] = reinterpret_cast<T (*)[LDX]>(lin_smem);                              // [GROUP][LDX]
+  T (*os)[LDO] = reinterpret_cast<T (*)[LDO]>(lin_smem + GROUP * LDX * sizeof(T));      // [ROWS][LDO]
+  static_assert(GROUP * LDX * sizeof(T) + ROWS * LDO * sizeof(T) <= linear_fwd_lds_bytes(KD, (int)sizeof(T)), "the launcher sizes LDS with linear_fwd_lds_bytes");
+  // rows GROUP c .. GROUP c + 127 of W_p (rows past N_p are zero)
+  vec wr[GP];
+  auto load_group = [&](const Cursor& cur) {
     const T* wsrc = reinterpret_cast<const T*>(a.w[cur.p]);
     const int N = a.n[cur.p];
 #pragma unroll
-    for (int x = 0; x < WCH; ++x) {
+    for (int x = 0; x < GP; ++x) {
       const int q = x * 256 + tid, r = q / (KD / 8), col = 8 * (q % (KD / 8));
       vec v = {};
-      if (q < WPC && 32 * cur.c + r < N) v = *reinterpret_cast<const vec*>(wsrc + (int64_t)(32 * cur.c + r) * KD + col);
-      dst[x] = v;
+      if (GROUP * cur.c + r < N) v = *reinterpret_cast<const vec*>(wsrc + (int64_t)(GROUP * cur.c + r) * KD + col);
+      wr[x] = v;
     }
   };
-  auto store_chunk = [&](int buf, const vec* src) {
+  auto store_group = [&] {
 #pragma unroll
-    for (int x = 0; x < WCH; ++x) {
+    for (int x = 0; x < GP; ++x) {
       const int q = x * 256 + tid, r = q / (KD / 8), col = 8 * (q % (KD / 8));
-      if (q < WPC) *reinterpret_cast<vec*>(&wsm[buf][r][col]) = src[x];
+      *reinterpret_cast<vec*>(&wg[r][col]) = wr[x];
     }
   };
 
   Cursor ld{0, 0}, use{0, 0};
-  load_chunk(ld, wr[0]);
+  load_group(ld);
   advance(ld);
-  if (total > 1) { load_chunk(ld, wr[1]); advance(ld); }
-  store_chunk(0, wr[0]);
-  __syncthreads();
-  auto one_chunk = [&](int q, auto which) __attribute__((always_inline)) {
-    constexpr int buf = decltype(which)::value;
-    if (q + 2 < total) { load_chunk(ld, wr[buf]); advance(ld); }
-    const int N = a.n[use.p], n0 = 32 * use.c;
+  for (int gq = 0; gq < total; ++gq) {
+    store_group();
+    __syncthreads();
+    if (gq + 1 < total) { load_group(ld); advance(ld); }
+    const int N = a.n[use.p];
     const T* bias = reinterpret_cast<const T*>(a.bias[use.p]);
     T* y = reinterpret_cast<T*>(a.y[use.p]);
-    // this lane's 16 columns of the chunk: n0 + 8 q4 + 4 g + e
-    f32x16 acc[RT];
+    const int hd = a.hd[use.p];
+    const int chunks = min(GROUP, N - GROUP * use.c + 31) / 32;  // chunks of 32 columns in this group
+    for (int c = 0; c < chunks; ++c) {
+      const int n0 = GROUP * use.c + 32 * c;
+      // this lane's 16 columns of the chunk: n0 + 8 q4 + 4 g + e
+      f32x16 acc[RT];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int n = n0 + 8 * (v / 4) + 4 * g + (v % 4);
-      const float b = (bias && n < N) ? (float)bias[n] : 0.f;
+      for (int v = 0; v < 16; ++v) {
+        const int n = n0 + 8 * (v / 4) + 4 * g + (v % 4);
+        const float bv = (bias && n < N) ? (float)bias[n] : 0.f;
 #pragma unroll
-      for (int t = 0; t < RT; ++t) acc[t][v] = b;
-    }
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const frag af = *reinterpret_cast<const frag*>(&wsm[buf][cl][16 * s + 8 * g]);
-#pragma unroll
-      for (int t = 0; t < RT; ++t) acc[t] = E::mfma(af, xf[t][s], acc[t]);
-    }
-    // the chunk of this wave's 64 rows -> its own rows of the output tile -> global memory
-#pragma unroll
-    for (int t = 0; t < RT; ++t)
-#pragma unroll
-      for (int q4 = 0; q4 < 4; ++q4) {
-        typename E::vec4 ov;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) ov[e] = (T)acc[t][4 * q4 + e];
-        *reinterpret_cast<typename E::vec4*>(&os[64 * wave + 32 * t + cl][8 * q4 + 4 * g]) = ov;
+        for (int t = 0; t < RT; ++t) acc[t][v] = bv;
       }
-    // (the wave reads back only what it wrote: LDS operations of a wave complete in order)
-    __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      const int idx = x * 64 + lane, r = 64 * wave + idx / 4, col = n0 + 8 * (idx % 4);
-      const int64_t row = row0 + r;
-      const vec v = *reinterpret_cast<const vec*>(&os[r][8 * (idx % 4)]);
-      if (row < a.rows && col < N) {
-        T* dst = y + linear_offset(row, col, N, a.hd[use.p], a.rows);
-        if ((N % 8) == 0) {
-          *reinterpret_cast<vec*>(dst) = v;
-        } else {
+      for (int s = 0; s < KS; ++s) {
+        const frag af = *reinterpret_cast<const frag*>(&wg[32 * c + cl][16 * s + 8 * g]);
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (col + e < N) dst[e] = v[e];
+        for (int t = 0; t < RT; ++t) acc[t] = E::mfma(af, xf[t][s], acc[t]);
+      }
+      // the chunk of this wave's 64 rows -> its own rows of the output tile -> global memory
+#pragma unroll
+      for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          typename E::vec4 ov;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) ov[e] = (T)acc[t][4 * q4 + e];
+          *reinterpret_cast<typename E::vec4*>(&os[64 * wave + 32 * t + cl][8 * q4 + 4 * g]) = ov;
+        }
+      // (the wave reads back only what it wrote: LDS operations of a wave complete in order)
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int idx = x * 64 + lane, r = 64 * wave + idx / 4, col = n0 + 8 * (idx % 4);
+        const int64_t row = row0 + r;
+        const vec v = *reinterpret_cast<const vec*>(&os[r][8 * (idx % 4)]);
+        if (row < a.rows && col < N) {
+          T* dst = y + linear_offset(row, col, N, hd, a.rows);
+          if ((N % 8) == 0) {
+            *reinterpret_cast<vec*>(dst) = v;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (col + e < N) dst[e] = v[e];
+          }
         }
       }
+      __builtin_amdgcn_wave_barrier();
     }
     advance(use);
-    if (q + 1 < total) store_chunk(buf ^ 1, wr[buf ^ 1]);
-    __syncthreads();
-  };
-  for (int q = 0; q < total; q += 2) {
-    one_chunk(q, std::integral_constant<int, 0>{});
-    if (q + 1 < total) one_chunk(q + 1, std::integral_constant<int, 1>{});
+    __syncthreads();  // every wave is done with this group's weights
   }
 }
 
