@@ -186,7 +186,8 @@ int trifast_bwd_one(int kernel,
  * Weight gradient of a linear layer over a pair representation: dw[n, k] = sum over r of
  * dy[r, n] x[r, k] for x [rows, k], dy [rows, n], dw [n, k], all dense, of one 16-bit dtype,
  * rows = b n^2 in the millions and k in {32, 64, 128, 256}: the rows are split over
- * workgroups, whose fp32 partials (the workspace) are added in a fixed order.  head_dim = 0:
+ * workgroups, whose fp32 partials (the workspace) are added in a fixed order.  db, if not null,
+ * receives the layer's bias gradient db[n] = sum over r of dy[r, n] from the same pass.  head_dim = 0:
  * dy is [rows, n]; head_dim = d: dy is kept heads-outermost, [n / d][rows][d], the layout the
  * attention operator takes q, k, v in (d a multiple of 8 that divides n).  No counterpart
  * in the reference, whose callers are only hinted at by the module of
@@ -212,7 +213,7 @@ int trifast_linear_fwd(const void* x, int64_t rows, int64_t k, int nlayers, cons
  */
 int trifast_linear_dx(void* dx, int64_t rows, int64_t k, int nlayers, const void* const* dy, const void* const* wt,
                       const int64_t* n, const int64_t* head_dim, int dtype, void* stream);
-int trifast_linear_dw(void* dw, const void* dy, const void* x, int64_t rows, int64_t k, int64_t n, int64_t head_dim, int dtype,
+int trifast_linear_dw(void* dw, void* db, const void* dy, const void* x, int64_t rows, int64_t k, int64_t n, int64_t head_dim, int dtype,
                       void* workspace, int64_t workspace_bytes, void* stream);
 
 /*

@@ -127,7 +127,7 @@ def test_gate_argument_errors_come_back_as_codes():
 def test_weight_gradient_argument_errors_come_back_as_codes():
     lib = _lib.load()
     ok = 0x1000
-    call = lambda dw, dy, x, rows, k, n, dtype=_lib.BF16, ws=ok, nbytes=1 << 40, hd=0: lib.trifast_linear_dw(dw, dy, x, rows, k, n, hd, dtype, ws, nbytes, None)
+    call = lambda dw, dy, x, rows, k, n, dtype=_lib.BF16, ws=ok, nbytes=1 << 40, hd=0: lib.trifast_linear_dw(dw, None, dy, x, rows, k, n, hd, dtype, ws, nbytes, None)
     assert call(ok, ok, ok, 100, 48, 8) == -2 and "input channels" in _lib.last_error()
     assert call(ok, ok, ok, 100, 64, 8, _lib.F32) == -2 and "16-bit" in _lib.last_error()
     assert call(ok, ok, ok, 0, 64, 8) == -1 and "positive" in _lib.last_error()
@@ -137,10 +137,11 @@ def test_weight_gradient_argument_errors_come_back_as_codes():
     assert call(ok, ok, ok, 100, 64, 48, hd=32) == -1 and "head dim" in _lib.last_error()  # 32 does not divide 48
     assert call(ok, ok, ok, 100, 64, 48, hd=12) == -1 and "head dim" in _lib.last_error()  # not a multiple of 8
     # the partials: one [n, k] fp32 matrix per chunk of at least 1024 rows, at most 768 chunks
-    assert lib.trifast_linear_dw_workspace_bytes(1024, 128, 128) == 128 * 128 * 4
-    assert lib.trifast_linear_dw_workspace_bytes(3000, 128, 128) == 3 * 128 * 128 * 4
-    assert 700 * 128 * 128 * 4 <= lib.trifast_linear_dw_workspace_bytes(1 << 20, 128, 128) <= 768 * 128 * 128 * 4
-    assert lib.trifast_linear_dw_workspace_bytes(1 << 24, 128, 4) <= 768 * 128 * 4 * 4
+    # (plus one [n] fp32 vector per chunk for the bias gradient)
+    assert lib.trifast_linear_dw_workspace_bytes(1024, 128, 128) == 128 * 128 * 4 + 128 * 4
+    assert lib.trifast_linear_dw_workspace_bytes(3000, 128, 128) == 3 * 128 * 128 * 4 + 3 * 128 * 4
+    assert 700 * 128 * 129 * 4 <= lib.trifast_linear_dw_workspace_bytes(1 << 20, 128, 128) <= 768 * 128 * 129 * 4
+    assert lib.trifast_linear_dw_workspace_bytes(1 << 24, 128, 4) <= 768 * 129 * 4 * 4 + 512
     assert lib.trifast_linear_dw_workspace_bytes(0, 128, 4) < 0
 
 

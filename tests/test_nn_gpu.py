@@ -152,6 +152,12 @@ def test_weight_gradient_against_float64(dtype, rows, k, n):
     err = (got.double() - want).abs()
     assert bool((err <= bound).all()), f"max excess {(err - bound).max().item():.3e}"
     assert torch.equal(got, nn.linear_weight_grad(dy, x)), "two runs differ"
+    # the bias gradient from the same pass
+    dw2, db = nn.linear_weight_grad(dy, x, 0, True)
+    assert torch.equal(dw2, got) and db.shape == (n,) and db.dtype == dtype
+    want_b, size_b = dy.double().sum(0), dy.double().abs().sum(0)
+    bound_b = 0.5 * torch.finfo(dtype).eps * want_b.abs() + max(rows, 64) ** 0.5 * 2.0**-22 * size_b + torch.finfo(dtype).smallest_normal
+    assert bool(((db.double() - want_b).abs() <= bound_b).all())
 
 
 def test_linear_gradients_are_those_of_the_layer():

@@ -68,7 +68,7 @@ SIGNATURES = {
     "trifast_linear_dw_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64]),
     "trifast_linear_fwd": (c_int, [c_void_p, c_int64, c_int64, c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64), POINTER(c_int64), c_int, c_void_p]),
     "trifast_linear_dx": (c_int, [c_void_p, c_int64, c_int64, c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64), POINTER(c_int64), c_int, c_void_p]),
-    "trifast_linear_dw": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p]),
+    "trifast_linear_dw": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p, c_int64, c_void_p]),
     "trifast_gate_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "trifast_gate_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
 }

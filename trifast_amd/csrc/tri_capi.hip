@@ -633,10 +633,10 @@ static int check_linear_head(const char* what, int p, int64_t n, int64_t hd) {
 
 int64_t trifast_linear_dw_workspace_bytes(int64_t rows, int64_t k, int64_t n) {
   if (rows < 1 || k < 1 || n < 1) return fail(TRIFAST_EINVAL, "sizes must be positive");
-  return align256(tri::linear_dw_chunks(rows) * n * k * 4);
+  return align256(tri::linear_dw_chunks(rows) * n * k * 4) + align256(tri::linear_dw_chunks(rows) * n * 4);
 }
 
-int trifast_linear_dw(void* dw, const void* dy, const void* x, int64_t rows, int64_t k, int64_t n, int64_t head_dim, int dtype,
+int trifast_linear_dw(void* dw, void* db, const void* dy, const void* x, int64_t rows, int64_t k, int64_t n, int64_t head_dim, int dtype,
                       void* workspace, int64_t workspace_bytes, void* stream) {
   g_err[0] = 0;
   if (int rc = check_linear_head("linear_dw", 0, n, head_dim)) return rc;
@@ -650,6 +650,8 @@ int trifast_linear_dw(void* dw, const void* dy, const void* x, int64_t rows, int
     return fail(TRIFAST_EWORKSPACE, "linear_dw: workspace missing, misaligned or smaller than trifast_linear_dw_workspace_bytes");
   tri::LinearDwArgs a{};
   a.x = x; a.dy = dy; a.dw = dw; a.part = static_cast<float*>(workspace);
+  a.db = db;
+  a.part_b = db ? reinterpret_cast<float*>(static_cast<char*>(workspace) + align256(tri::linear_dw_chunks(rows) * n * k * 4)) : nullptr;
   a.rows = rows; a.rows_per_chunk = tri::linear_dw_rows_per_chunk(rows); a.chunks = (int)tri::linear_dw_chunks(rows);
   a.K = (int)k; a.N = (int)n; a.hd = (int)head_dim;
   const hipError_t e = tri::linear_dw_launch(a, dtype, static_cast<hipStream_t>(stream));

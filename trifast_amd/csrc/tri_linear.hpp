@@ -10,7 +10,8 @@
 // their memory row, so both are read back transposed, ds_read_tr), keeps its part of dW in
 // fp32 accumulators (wave w: rows n of its 32-block, all K columns), and writes it as an fp32
 // partial; a second kernel adds the partials in a fixed order (deterministic, no atomics)
-// and rounds once.  Bound by HBM: every element of dY and x is read once per group of n.
+// and rounds once.  The layer's bias gradient, the column sums of dY, comes out of the same
+// pass on request (dY^T times a vector of ones: one more MFMA per 16 rows).  Bound by HBM: every element of dY and x is read once per group of n.
 // No counterpart in the reference: the linear layers around its operator are only hinted
 // at by the module of reference tests/unit/test_trifast.py:152-169.
 #pragma once
@@ -34,6 +35,8 @@ struct LinearDwArgs {
   int hd;
   float* part;      // [chunks, N, K] partial sums
   void* dw;         // [N, K]
+  float* part_b;    // [chunks, N] partial column sums of dy (the layer's bias gradient), or null
+  void* db;         // [N], or null
   int64_t rows;
   int64_t rows_per_chunk;  // multiple of 32
   int chunks;
@@ -57,7 +60,7 @@ inline int64_t linear_dw_chunks(int64_t rows) {
 // KD: columns of x (K, one of 32, 64, 128, 256); ND: output rows n per workgroup, 128 (wave w
 // owns rows 32 w .. 32 w + 31 and every column block of x) or, for layers of up to 32 outputs,
 // 32 (the four waves share the column blocks of x)
-template <typename T, int KD, int ND>
+template <typename T, int KD, int ND, bool BIAS>
 __global__ __launch_bounds__(256) void linear_dw_kernel(const LinearDwArgs a) {
   using E = Elem<T>;
   using frag = typename E::frag;
@@ -132,6 +135,11 @@ __global__ __launch_bounds__(256) void linear_dw_kernel(const LinearDwArgs a) {
   auto col_block = [&](int i) { return SPLIT_K ? wave + 4 * i : i; };  // ... and its column blocks of x
   // (a wave whose output rows lie past N, or that has no column block, only stages)
   const bool wave_live = __builtin_amdgcn_readfirstlane((int)(n_grp + 32 * n_blk < N && col_block(0) < KB)) != 0;
+  // the bias gradient, the column sums of dy, rides along as one more product: dy^T times ones
+  // (one wave per 32 output rows does it)
+  const bool sums = BIAS && (!SPLIT_K || wave == 0);
+  const frag ones = E::splat(1.0f);
+  f32x16 bacc = zero16();
 
   load_step(0, xr2[0], yr2[0]);
   if (steps > 1) load_step(1, xr2[1], yr2[1]);
@@ -145,6 +153,7 @@ __global__ __launch_bounds__(256) void linear_dw_kernel(const LinearDwArgs a) {
       for (int s2 = 0; s2 < 2; ++s2) {
         // A: dY^T (output row n in the lane, 8 memory rows as contraction slots); B: x^T
         const frag af = lds_tr_frag<T, LDY>(ys[buf], 16 * s2 + 8 * g, 32 * n_blk, lane);
+        if (sums) bacc = E::mfma(af, ones, bacc);
 #pragma unroll
         for (int i = 0; i < KBW; ++i) {
           if (col_block(i) < KB) {
@@ -166,6 +175,15 @@ __global__ __launch_bounds__(256) void linear_dw_kernel(const LinearDwArgs a) {
   if (!wave_live) return;
   // partial [chunk][n][k]: the lane holds column k = 32 kb + lane % 32 and rows
   // n = 32 wave + 8 q + 4 g + e of the group
+  if (sums && (lane & 31) == 0) {
+    // (every column of the product holds the same sums: lanes 0 and 32 store theirs)
+    float* pb = a.part_b + (int64_t)blockIdx.x * N;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int n = n_grp + 32 * n_blk + 8 * (v / 4) + 4 * g + (v % 4);
+      if (n < N) pb[n] = bacc[v];
+    }
+  }
   float* part = a.part + (int64_t)blockIdx.x * N * K;
 #pragma unroll
   for (int i = 0; i < KBW; ++i) {
@@ -182,15 +200,14 @@ __global__ __launch_bounds__(256) void linear_dw_kernel(const LinearDwArgs a) {
 // adds the chunks c, c + 8, ... in increasing order, then the 8 sums are added in order of c
 // (one fixed association, whatever the timing).
 template <typename T>
-__global__ __launch_bounds__(256) void linear_dw_reduce_kernel(const LinearDwArgs a) {
+__global__ __launch_bounds__(256) void linear_dw_reduce_kernel(const float* part, T* out, int64_t count, int chunks) {
   __shared__ float sums[8][32];
-  const int64_t count = (int64_t)a.N * a.K;
   const int e = threadIdx.x & 31, c0 = threadIdx.x >> 5;
   const int64_t idx = (int64_t)blockIdx.x * 32 + e;
   float sum = 0.f;
   if (idx < count) {
 #pragma unroll 4
-    for (int c = c0; c < a.chunks; c += 8) sum += a.part[(int64_t)c * count + idx];
+    for (int c = c0; c < chunks; c += 8) sum += part[(int64_t)c * count + idx];
   }
   sums[c0][e] = sum;
   __syncthreads();
@@ -198,7 +215,7 @@ __global__ __launch_bounds__(256) void linear_dw_reduce_kernel(const LinearDwArg
     float total = sums[0][e];
 #pragma unroll
     for (int c = 1; c < 8; ++c) total += sums[c][e];
-    reinterpret_cast<T*>(a.dw)[idx] = (T)total;
+    out[idx] = (T)total;
   }
 }
 
@@ -207,29 +224,30 @@ inline bool linear_dw_k_ok(int64_t k) { return k == 32 || k == 64 || k == 128 ||
 template <typename T>
 inline hipError_t linear_dw_launch_t(const LinearDwArgs& a, hipStream_t st) {
   const dim3 block(256);
-  if (a.N <= 32) {
-    const dim3 grid((unsigned)a.chunks, 1);
-    switch (a.K) {
-      case 32: hipLaunchKernelGGL((linear_dw_kernel<T, 32, 32>), grid, block, 0, st, a); break;
-      case 64: hipLaunchKernelGGL((linear_dw_kernel<T, 64, 32>), grid, block, 0, st, a); break;
-      case 128: hipLaunchKernelGGL((linear_dw_kernel<T, 128, 32>), grid, block, 0, st, a); break;
-      case 256: hipLaunchKernelGGL((linear_dw_kernel<T, 256, 32>), grid, block, 0, st, a); break;
-      default: return hipErrorInvalidConfiguration;
-    }
-  } else {
-    const dim3 grid((unsigned)a.chunks, (unsigned)((a.N + 127) / 128));
-    switch (a.K) {
-      case 32: hipLaunchKernelGGL((linear_dw_kernel<T, 32, 128>), grid, block, 0, st, a); break;
-      case 64: hipLaunchKernelGGL((linear_dw_kernel<T, 64, 128>), grid, block, 0, st, a); break;
-      case 128: hipLaunchKernelGGL((linear_dw_kernel<T, 128, 128>), grid, block, 0, st, a); break;
-      case 256: hipLaunchKernelGGL((linear_dw_kernel<T, 256, 128>), grid, block, 0, st, a); break;
-      default: return hipErrorInvalidConfiguration;
-    }
+  const bool split_k = a.N <= 32;
+  const dim3 grid((unsigned)a.chunks, split_k ? 1u : (unsigned)((a.N + 127) / 128));
+#define TRI_DW_CASE(KD)                                                                                          \
+  case KD:                                                                                                       \
+    if (split_k && a.part_b) hipLaunchKernelGGL((linear_dw_kernel<T, KD, 32, true>), grid, block, 0, st, a);     \
+    else if (split_k) hipLaunchKernelGGL((linear_dw_kernel<T, KD, 32, false>), grid, block, 0, st, a);           \
+    else if (a.part_b) hipLaunchKernelGGL((linear_dw_kernel<T, KD, 128, true>), grid, block, 0, st, a);          \
+    else hipLaunchKernelGGL((linear_dw_kernel<T, KD, 128, false>), grid, block, 0, st, a);                       \
+    break;
+  switch (a.K) {
+    TRI_DW_CASE(32)
+    TRI_DW_CASE(64)
+    TRI_DW_CASE(128)
+    TRI_DW_CASE(256)
+    default: return hipErrorInvalidConfiguration;
   }
+#undef TRI_DW_CASE
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   const int64_t count = (int64_t)a.N * a.K;
-  hipLaunchKernelGGL((linear_dw_reduce_kernel<T>), dim3((unsigned)((count + 31) / 32)), block, 0, st, a);
+  hipLaunchKernelGGL((linear_dw_reduce_kernel<T>), dim3((unsigned)((count + 31) / 32)), block, 0, st, (const float*)a.part, reinterpret_cast<T*>(a.dw), count, a.chunks);
+  e = hipGetLastError();
+  if (e != hipSuccess || !a.part_b) return e;
+  hipLaunchKernelGGL((linear_dw_reduce_kernel<T>), dim3((unsigned)((a.N + 31) / 32)), block, 0, st, (const float*)a.part_b, reinterpret_cast<T*>(a.db), (int64_t)a.N, a.chunks);
   return hipGetLastError();
 }
 

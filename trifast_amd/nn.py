@@ -98,21 +98,23 @@ def _rows_n(dy: torch.Tensor, head_dim: int) -> tuple[int, int]:
     return (dy.shape[1], dy.shape[0] * dy.shape[2]) if head_dim else (dy.shape[0], dy.shape[1])
 
 
-def linear_weight_grad(dy: torch.Tensor, x: torch.Tensor, head_dim: int = 0) -> torch.Tensor:
+def linear_weight_grad(dy: torch.Tensor, x: torch.Tensor, head_dim: int = 0, with_bias: bool = False):
     """``dy^T x`` for ``dy [rows, n]``, ``x [rows, k]``: the weight gradient of a linear layer, with
     the long contraction over the rows split over the whole GPU (``trifast_linear_dw``).  With
-    ``head_dim = d``, dy is ``[n / d, rows, d]`` (heads outermost)."""
+    ``head_dim = d``, dy is ``[n / d, rows, d]`` (heads outermost).  ``with_bias``: also the bias
+    gradient ``dy.sum(0)`` from the same pass; the result is then the pair (dw, db)."""
     dy, x = dy.contiguous(), x.contiguous()
     rows, n = _rows_n(dy, head_dim)
     k = x.shape[1]
     lib = _lib.load()
     dw = torch.empty(n, k, dtype=x.dtype, device=x.device)
+    db = torch.empty(n, dtype=x.dtype, device=x.device) if with_bias else None
     ws = torch.empty(lib.trifast_linear_dw_workspace_bytes(rows, k, n), dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
-        rc = lib.trifast_linear_dw(dw.data_ptr(), dy.data_ptr(), x.data_ptr(), rows, k, n, head_dim, _dtype_code(x), ws.data_ptr(), ws.numel(),
-                                   torch.cuda.current_stream(x.device).cuda_stream)
+        rc = lib.trifast_linear_dw(dw.data_ptr(), None if db is None else db.data_ptr(), dy.data_ptr(), x.data_ptr(), rows, k, n, head_dim,
+                                   _dtype_code(x), ws.data_ptr(), ws.numel(), torch.cuda.current_stream(x.device).cuda_stream)
     _lib.check(rc, "trifast_linear_dw")
-    return dw
+    return (dw, db) if with_bias else dw
 
 
 class _Linear(torch.autograd.Function):
@@ -131,8 +133,7 @@ class _Linear(torch.autograd.Function):
         x, weight = ctx.saved_tensors
         dy2 = dy.reshape(-1, dy.shape[-1])
         dx = (dy2 @ weight).view(x.shape) if ctx.needs_input_grad[0] else None
-        dw = linear_weight_grad(dy2, x.reshape(-1, x.shape[-1])) if ctx.needs_input_grad[1] else None
-        db = dy2.sum(0) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        dw, db = linear_weight_grad(dy2, x.reshape(-1, x.shape[-1]), 0, True) if ctx.has_bias else (linear_weight_grad(dy2, x.reshape(-1, x.shape[-1])), None)
         return dx, dw, db
 
 
@@ -211,8 +212,16 @@ class _Project(torch.autograd.Function):
                 dx = linear_input_grad([t[0] for t in live], [t[1] for t in live], [t[2] for t in live]).view(x.shape)
             else:
                 dx = sum(dy @ w for dy, w, _ in live).view(x.shape)
-        dws = [None if dy is None else linear_weight_grad(dy, x2, d) for dy, d in zip(flat, ctx.head_dims)]
-        dbs = [dy.sum(0) if (dy is not None and has) else None for dy, has in zip(flat, ctx.has_bias)]  # (a layer with a bias is plain)
+        dws, dbs = [], []
+        for dy, d, has in zip(flat, ctx.head_dims, ctx.has_bias):
+            if dy is None:
+                dw, db = None, None
+            elif has:  # (a layer with a bias is plain)
+                dw, db = linear_weight_grad(dy, x2, 0, True)
+            else:
+                dw, db = linear_weight_grad(dy, x2, d), None
+            dws.append(dw)
+            dbs.append(db)
         return (dx, None, *dws, *dbs)
 
 
