@@ -29,6 +29,13 @@ struct BiasPrepArgs {
   int H, N, NP;
 };
 
+// Split of the pre-pass grid: workgroups [0, bias_blocks) re-tile the bias
+// (bias_blocks_per_head per batch*head), the rest take four mask rows each.
+struct PrepGrid {
+  unsigned bias_blocks, bias_blocks_per_head;
+  int64_t mask_rows;         // b * n
+};
+
 struct FwdArgs {
   const void *q, *k, *v;
   const void* packq;

@@ -18,17 +18,19 @@
 namespace tri {
 
 // ---------------------------------------------------------------------------
-// Mask pre-pass: bytes -> "keep" bit words + fully-masked-row flags.
-// One wave per (batch, row).  A row whose valid keys are all masked follows the
-// additive-mask semantics of reference src/trifast/equiv.py:49,59-62: all logits
-// saturate to the same value, so the row attends uniformly to every key; its
-// keep words are set to "all valid keys" and rowflag tells the kernels to
-// drop the q.k and bias terms.
+// The pre-passes: one launch of workgroups of four waves; the first `bias_blocks`
+// workgroups re-tile the bias, the rest turn mask rows into bit words, one wave per row.
+//
+// Mask: bytes -> "keep" bit words + fully-masked-row flags.  A row whose valid keys are
+// all masked follows the additive-mask semantics of reference
+// src/trifast/equiv.py:49,59-62: all logits saturate to the same value, so the row
+// attends uniformly to every key; its keep words are set to "all valid keys" and
+// rowflag tells the kernels to drop the q.k and bias terms.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void mask_prep_kernel(const MaskPrepArgs a) {
-  const int i = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
+__device__ __forceinline__ void mask_prep_row(const MaskPrepArgs& a, int64_t bi, int lane) {
+  const int b = (int)(bi / a.n), i = (int)(bi % a.n);
   const uint8_t* row = a.mask + b * a.sb + i * a.si;
-  uint32_t* out = a.keep + ((int64_t)b * a.n + i) * a.nwords;
+  uint32_t* out = a.keep + bi * a.nwords;
   bool any_kept = false;
   // (contiguous, 16-byte aligned rows: the 32 bytes of a word are two vector loads)
   const bool vec_rows = a.sk == 1 && (reinterpret_cast<uintptr_t>(row) & 15) == 0;
@@ -59,25 +61,16 @@ __global__ __launch_bounds__(64) void mask_prep_kernel(const MaskPrepArgs a) {
       out[w] = rem >= 32 ? 0xffffffffu : ((1u << rem) - 1u);
     }
   }
-  if (lane == 0) a.rowflag[(int64_t)b * a.n + i] = row_kept ? 0 : 1;
+  if (lane == 0) a.rowflag[bi] = row_kept ? 0 : 1;
 }
 
-hipError_t mask_prep_launch(const MaskPrepArgs& a, int b, hipStream_t st) {
-  hipLaunchKernelGGL(mask_prep_kernel, dim3(a.n, b), dim3(64), 0, st, a);
-  return hipGetLastError();
-}
-
-// ---------------------------------------------------------------------------
-// Bias pre-pass: re-tile bias[b, h, j, k] (any strides) into the register layouts
-// of the kernels (see BiasPrepArgs), zero-padded to whole tiles.  One thread
-// writes the 8 elements of one (tile, r, lane) slot of each requested layout.
-// ---------------------------------------------------------------------------
+// Bias: re-tile bias[b, h, j, k] (any strides) into the register layouts of the kernels
+// (see BiasPrepArgs), zero-padded to whole tiles.  One thread writes the 8 elements of
+// one (tile, r, lane) slot of each requested layout.
 template <typename T>
-__global__ __launch_bounds__(256) void bias_prep_kernel(const BiasPrepArgs a) {
-  const int bh = blockIdx.y;
+__device__ __forceinline__ void bias_prep_slot(const BiasPrepArgs& a, int bh, int64_t slot) {
   const int b = bh / a.H, h = bh % a.H;
-  const int64_t slot = (int64_t)blockIdx.x * 256 + threadIdx.x;  // ((jt*NP + kt)*2 + r)*64 + lane
-  if (slot >= (int64_t)a.NP * a.NP * 128) return;
+  if (slot >= (int64_t)a.NP * a.NP * 128) return;  // ((jt*NP + kt)*2 + r)*64 + lane
   const int lane = slot & 63, r = (slot >> 6) & 1;
   const int tile = (int)(slot >> 7);
   const int jt = tile / a.NP, kt = tile % a.NP;
@@ -109,13 +102,30 @@ __global__ __launch_bounds__(256) void bias_prep_kernel(const BiasPrepArgs a) {
   }
 }
 
-hipError_t bias_prep_launch(const BiasPrepArgs& a, int bh, int dtype, hipStream_t st) {
+template <typename T>
+__global__ __launch_bounds__(256) void prep_kernel(const MaskPrepArgs m, const BiasPrepArgs a, const PrepGrid g) {
+  if (blockIdx.x < g.bias_blocks) {
+    const unsigned bh = blockIdx.x / g.bias_blocks_per_head, bx = blockIdx.x % g.bias_blocks_per_head;
+    bias_prep_slot<T>(a, (int)bh, (int64_t)bx * 256 + threadIdx.x);
+  } else {
+    const int64_t row = (int64_t)(blockIdx.x - g.bias_blocks) * 4 + (threadIdx.x >> 6);
+    if (row < g.mask_rows) mask_prep_row(m, row, threadIdx.x & 63);
+  }
+}
+
+hipError_t prep_launch(const MaskPrepArgs& m, int b, const BiasPrepArgs& a, int bh, int dtype, hipStream_t st) {
   const int64_t slots = (int64_t)a.NP * a.NP * 128;
-  dim3 grid((unsigned)((slots + 255) / 256), bh);
+  PrepGrid g;
+  g.bias_blocks_per_head = (unsigned)((slots + 255) / 256);
+  g.mask_rows = (int64_t)b * m.n;
+  const int64_t bias_blocks = (int64_t)g.bias_blocks_per_head * bh, blocks = bias_blocks + (g.mask_rows + 3) / 4;
+  if (blocks > 0x7fffffff) return hipErrorInvalidConfiguration;
+  g.bias_blocks = (unsigned)bias_blocks;
+  const dim3 grid((unsigned)blocks);
   switch (dtype) {
-    case kF32: hipLaunchKernelGGL(bias_prep_kernel<float>, grid, dim3(256), 0, st, a); break;
-    case kBF16: hipLaunchKernelGGL(bias_prep_kernel<__bf16>, grid, dim3(256), 0, st, a); break;
-    default: hipLaunchKernelGGL(bias_prep_kernel<_Float16>, grid, dim3(256), 0, st, a); break;
+    case kF32: hipLaunchKernelGGL(prep_kernel<float>, grid, dim3(256), 0, st, m, a, g); break;
+    case kBF16: hipLaunchKernelGGL(prep_kernel<__bf16>, grid, dim3(256), 0, st, m, a, g); break;
+    default: hipLaunchKernelGGL(prep_kernel<_Float16>, grid, dim3(256), 0, st, m, a, g); break;
   }
   return hipGetLastError();
 }
@@ -256,20 +266,9 @@ void contiguous4(int64_t* s, int64_t h, int64_t n) {
   s[3] = 1; s[2] = n; s[1] = n * n; s[0] = h * n * n;
 }
 
-int run_bias_prep(const void* bias, const int64_t* bs, const Workspace& w, bool want_k, int64_t b, int64_t h,
-                  int64_t n, int dtype, hipStream_t st) {
-  tri::BiasPrepArgs p;
-  p.bias = bias;
-  p.sb = bs[0]; p.sh = bs[1]; p.sj = bs[2]; p.sk = bs[3];
-  p.packq = w.packq;
-  p.packk = want_k ? w.packk : nullptr;
-  p.H = (int)h; p.N = (int)n; p.NP = w.np;
-  hipError_t e = tri::bias_prep_launch(p, (int)(b * h), dtype, st);
-  if (e != hipSuccess) return hip_fail(e, "bias pre-pass launch");
-  return 0;
-}
-
-int run_mask_prep(const uint8_t* mask, const int64_t* ms, const Workspace& w, int64_t b, int64_t n, hipStream_t st) {
+// Both pre-passes in one launch: keep words and row flags of the mask, the packed bias.
+int run_prep(const uint8_t* mask, const int64_t* ms, const void* bias, const int64_t* bs, const Workspace& w, bool want_k,
+             int64_t b, int64_t h, int64_t n, int dtype, hipStream_t st) {
   tri::MaskPrepArgs m;
   m.mask = mask;
   m.sb = ms[0]; m.si = ms[1]; m.sk = ms[2];
@@ -277,8 +276,14 @@ int run_mask_prep(const uint8_t* mask, const int64_t* ms, const Workspace& w, in
   m.rowflag = w.rowflag;
   m.n = (int)n;
   m.nwords = w.nwords;
-  hipError_t e = tri::mask_prep_launch(m, (int)b, st);
-  if (e != hipSuccess) return hip_fail(e, "mask pre-pass launch");
+  tri::BiasPrepArgs p;
+  p.bias = bias;
+  p.sb = bs[0]; p.sh = bs[1]; p.sj = bs[2]; p.sk = bs[3];
+  p.packq = w.packq;
+  p.packk = want_k ? w.packk : nullptr;
+  p.H = (int)h; p.N = (int)n; p.NP = w.np;
+  hipError_t e = tri::prep_launch(m, (int)b, p, (int)(b * h), dtype, st);
+  if (e != hipSuccess) return hip_fail(e, "mask and bias pre-pass launch");
   return 0;
 }
 
@@ -439,8 +444,7 @@ static int fwd_impl(bool use_static, void* o, float* lse, const void* q, const v
 
   hipStream_t st = static_cast<hipStream_t>(stream);
   const Workspace w = carve(workspace, b, h, n, dtype);
-  if ((rc = run_mask_prep(mask, mask_strides, w, b, n, st))) return rc;
-  if ((rc = run_bias_prep(bias, bias_strides, w, false, b, h, n, dtype, st))) return rc;
+  if ((rc = run_prep(mask, mask_strides, bias, bias_strides, w, false, b, h, n, dtype, st))) return rc;
 
   tri::FwdArgs a;
   a.q = q; a.k = k; a.v = v; a.packq = w.packq;
@@ -533,10 +537,9 @@ static int bwd_impl(int which, void* dq, void* dk, void* dv, void* db, const voi
   const Workspace w = carve(workspace, b, h, n, dtype);
   // The pre-passes are cheap (n^2 elements) and make every single-kernel call
   // self-contained, so they run on every call.
-  if ((rc = run_mask_prep(mask, mask_strides, w, b, n, st))) return rc;
   // (only the dk/dv tiles that do not also produce dq read the key-major packed bias)
   const bool want_k = do_kv && !tri::bwd_kv_tile_writes_dq(tkv);
-  if ((rc = run_bias_prep(bias, bias_strides, w, want_k, b, h, n, dtype, st))) return rc;
+  if ((rc = run_prep(mask, mask_strides, bias, bias_strides, w, want_k, b, h, n, dtype, st))) return rc;
 
   tri::BwdArgs a;
   a.q = q; a.k = k; a.v = v; a.o = o; a.dout = dout;

@@ -40,8 +40,7 @@ bool bwd_b_supports(int tile, int64_t n, int d, int dtype);
 hipError_t bwd_b_launch(const BwdArgs& a, int bh, int d, int dtype, int tile, hipStream_t st);
 int bwd_b_chunks(int64_t n, int64_t bh, int row_bytes);
 
-hipError_t mask_prep_launch(const MaskPrepArgs& a, int b, hipStream_t st);
-hipError_t bias_prep_launch(const BiasPrepArgs& a, int bh, int dtype, hipStream_t st);
+hipError_t prep_launch(const MaskPrepArgs& m, int b, const BiasPrepArgs& a, int bh, int dtype, hipStream_t st);
 
 inline bool head_dim_ok(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }
 
