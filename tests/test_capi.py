@@ -201,8 +201,8 @@ def test_gated_output_checks_shapes_on_the_host():
     assert [t.shape for t in nn.project(torch.zeros(2, 24), (block.q, block.b))] == [(2, 32), (2, 2)]
     # heads-outermost outputs: [h, *, d]; on tensors the kernels do not take, a permuted copy
     assert [t.shape for t in nn.project(torch.zeros(3, 5, 24), (block.q, block.b), (16, 0))] == [(2, 3, 5, 16), (3, 5, 2)]
-    with pytest.raises(ValueError, match="no bias"):
-        nn.project(torch.zeros(2, 24), (block.g,), (16,))
+    # (a layer with a bias too)
+    assert nn.project(torch.zeros(2, 24), (block.g,), (16,))[0].shape == (2, 2, 16)
     assert {n for n, _ in block.named_parameters()} == {"q.weight", "k.weight", "v.weight", "b.weight", "g.weight", "g.bias", "out.weight", "out.bias"}
 
 

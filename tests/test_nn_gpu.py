@@ -274,8 +274,9 @@ def test_heads_outermost_layers(dtype):
     x = torch.randn(rows, k, generator=gen).to(DEV, dtype)
     ws = [(torch.randn(n, k, generator=gen) * k**-0.5).to(DEV, dtype) for n in (h * d, 4, 2 * 64)]
     hds = (d, 0, 64)
-    ys = nn.linear_outputs(x, ws, [None] * 3, hds)
-    plain = nn.linear_outputs(x, ws, [None] * 3)
+    bs = [torch.randn(h * d, generator=gen).to(DEV, dtype), None, torch.randn(2 * 64, generator=gen).to(DEV, dtype)]
+    ys = nn.linear_outputs(x, ws, bs, hds)
+    plain = nn.linear_outputs(x, ws, bs)
     to_heads = lambda t, hd: t.unflatten(-1, (-1, hd)).movedim(-2, 0).contiguous() if hd else t
     for y, p, hd in zip(ys, plain, hds):
         assert y.shape == to_heads(p, hd).shape and torch.equal(y, to_heads(p, hd))
@@ -284,6 +285,8 @@ def test_heads_outermost_layers(dtype):
     assert torch.equal(nn.linear_input_grad(dys_h, ws, hds), nn.linear_input_grad(dys, ws))
     for t, th, hd in zip(dys, dys_h, hds):
         assert torch.equal(nn.linear_weight_grad(th, x, hd), nn.linear_weight_grad(t, x))
+        (dw_h, db_h), (dw_p, db_p) = nn.linear_weight_grad(th, x, hd, True), nn.linear_weight_grad(t, x, 0, True)
+        assert torch.equal(dw_h, dw_p) and torch.equal(db_h, db_p)
 
 
 def test_projection_with_heads_outermost_outputs():
@@ -291,7 +294,10 @@ def test_projection_with_heads_outermost_outputs():
     torch.manual_seed(8)
     dtype, h, d = torch.bfloat16, 2, 32
     x = torch.randn(2, 30, 30, 64, device=DEV, dtype=dtype)
-    layers = [torch.nn.Linear(64, h * d, bias=False).to(DEV, dtype), torch.nn.Linear(64, 32, bias=True).to(DEV, dtype)]
+    # (the second heads-outermost layer has a bias, like the layers of the module in reference
+    # tests/unit/test_trifast.py:152-169)
+    layers = [torch.nn.Linear(64, h * d, bias=False).to(DEV, dtype), torch.nn.Linear(64, 32, bias=True).to(DEV, dtype),
+              torch.nn.Linear(64, h * d, bias=True).to(DEV, dtype)]
     dys = [torch.randn(2, 30, 30, m.out_features, device=DEV, dtype=dtype) for m in layers]
 
     def grads(fn):
@@ -303,9 +309,9 @@ def test_projection_with_heads_outermost_outputs():
         return [o.detach().float() for o in outs], [xi.grad.float()] + [p.grad.float().clone() for m in layers for p in m.parameters()]
 
     def ours(xi):
-        q, g = nn.project(xi, layers, (d, 0))
-        assert q.shape == (h, 2, 30, 30, d) and q.is_contiguous()
-        return [q.movedim(0, -2).flatten(-2), g]  # back to [*, h * d] for the comparison
+        q, g, k = nn.project(xi, layers, (d, 0, d))
+        assert q.shape == (h, 2, 30, 30, d) and q.is_contiguous() and k.shape == q.shape and k.is_contiguous()
+        return [q.movedim(0, -2).flatten(-2), g, k.movedim(0, -2).flatten(-2)]  # back to [*, h * d] for the comparison
 
     (o1, g1), (o2, g2) = grads(ours), grads(lambda xi: [m(xi) for m in layers])
     for a, r in zip(o1 + g1, o2 + g2):

@@ -216,8 +216,8 @@ class _Project(torch.autograd.Function):
         for dy, d, has in zip(flat, ctx.head_dims, ctx.has_bias):
             if dy is None:
                 dw, db = None, None
-            elif has:  # (a layer with a bias is plain)
-                dw, db = linear_weight_grad(dy, x2, 0, True)
+            elif has:
+                dw, db = linear_weight_grad(dy, x2, d, True)
             else:
                 dw, db = linear_weight_grad(dy, x2, d), None
             dws.append(dw)
@@ -232,13 +232,11 @@ def project(x: torch.Tensor, layers, head_dims=None) -> tuple[torch.Tensor, ...]
     library's kernel (GPU, 16-bit, k in (32, 64, 128); k = 256: the weight gradients only);
     anything else is the layers themselves.
 
-    ``head_dims[p] = d`` (a bias-free layer of ``h * d`` outputs) returns output p as
+    ``head_dims[p] = d`` (a layer of ``h * d`` outputs) returns output p as
     ``[h, *x.shape[:-1], d]``, heads outermost, which is how the attention operator reads q, k, v
     fastest; the kernels write and read that layout directly (elsewhere it is a copy)."""
     layers = list(layers)
     head_dims = tuple(head_dims) if head_dims is not None else (0,) * len(layers)
-    if any(d and m.bias is not None for m, d in zip(layers, head_dims)):
-        raise ValueError("a heads-outermost layer takes no bias")
     fused = bool(layers) and len(layers) <= _DX_LAYERS and all(_dw_ready(x, m.weight) for m in layers)
     if not fused or x.shape[-1] not in _DX_K:
         ys = _Project.apply(x, (0,) * len(layers), *[m.weight for m in layers], *[m.bias for m in layers]) if fused else tuple(m(x) for m in layers)
