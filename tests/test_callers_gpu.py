@@ -226,3 +226,18 @@ def _ws_bytes(b, h, n, d):
     from trifast_amd import _lib
 
     return _lib.load().trifast_bwd_workspace_bytes(b, h, n, d, _lib.BF16)
+
+
+@pytest.mark.parametrize("shape", [(0, 2, 16, 32), (2, 0, 16, 32), (1, 2, 0, 32)], ids=["no_batch", "no_heads", "no_tokens"])
+def test_empty_inputs_give_empty_outputs(shape):
+    """An empty batch (a data loader's last, empty shard) passes through: empty output, empty
+    gradients, no launch."""
+    b, h, n, d = shape
+    q, k, v = (torch.zeros(b, h, n, n, d, device=DEV, dtype=torch.bfloat16, requires_grad=True) for _ in range(3))
+    bias = torch.zeros(b, h, n, n, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    mask = torch.zeros(b, n, n, device=DEV, dtype=torch.bool)
+    o = trifast_amd.triangle_attention(q, k, v, bias, mask)
+    assert o.shape == q.shape and o.dtype == q.dtype
+    o.sum().backward()
+    for t in (q, k, v, bias):
+        assert t.grad is not None and t.grad.shape == t.shape

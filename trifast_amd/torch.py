@@ -116,12 +116,14 @@ def _triangle_attention(
     lib = _lib.load()
     bs, h, n, d = _check_inputs(q, k, v, b, mask)
     code = _dtype_code(q)
+    o = torch.empty((bs, h, n, n, d), dtype=q.dtype, device=q.device)
+    lse = torch.empty((bs, h, n, n), dtype=torch.float32, device=q.device)
+    if o.numel() == 0 and d > 0:  # an empty batch (or no heads, or no tokens): nothing to launch
+        return o, lse
     # bias and mask are re-tiled by the library's pre-passes, so any strides go
     q, k, v = _vector_ready(q), _vector_ready(k), _vector_ready(v)
     mask_u8 = mask.view(torch.uint8)
 
-    o = torch.empty((bs, h, n, n, d), dtype=q.dtype, device=q.device)
-    lse = torch.empty((bs, h, n, n), dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
         ws_bytes = lib.trifast_fwd_workspace_bytes(bs, h, n, d, code)
         ws = _workspace(ws_bytes, q.device)
@@ -164,6 +166,8 @@ def triangle_attention_bwd(
     lib = _lib.load()
     bs, h, n, d = _check_inputs(q, k, v, b, mask)
     code = _dtype_code(q)
+    if q.numel() == 0 and d > 0:  # an empty batch: empty gradients
+        return _grad_like(q), _grad_like(k), _grad_like(v), _grad_like(b), torch.zeros_like(mask)
     if do.dtype != q.dtype:
         do = do.to(q.dtype)
     # the upstream gradient is often an expanded (stride-0) tensor, e.g. from
