@@ -39,7 +39,7 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC_MIB = {
     ("M", "_fwd", 3): 1518.1,
     ("M", "_bwd_q", 1): 2337.3,
-    ("M", "_bwd_kv", 7): 2673.9,
+    ("M", "_bwd_kv", 10): 2673.9,
     ("M", "_bwd_b", 4): 1586.0,
 }
 

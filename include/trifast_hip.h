@@ -40,7 +40,7 @@
 extern "C" {
 #endif
 
-#define TRIFAST_ABI_VERSION 2
+#define TRIFAST_ABI_VERSION 3
 
 /* dtype codes */
 #define TRIFAST_F32 0

@@ -40,7 +40,7 @@ def test_tile_tables():
     lib = _lib.load()
     for kernel in range(4):
         nt = lib.trifast_num_tiles(kernel)
-        assert 1 <= nt <= 9
+        assert 1 <= nt <= 12
         for t in range(nt):
             info = _lib.tile_info(kernel, t)
             assert info["BLOCK_J"] % 32 == 0 and info["BLOCK_K"] % 32 == 0 and info["num_waves"] in (1, 2, 4, 8, 16)

@@ -173,15 +173,15 @@ def test_pick_charges_a_tile_what_it_leaves_to_other_kernels(tmp_path, monkeypat
 
 
 def test_row_resident_tiles_in_the_library_tables():
-    """The row-resident kernel appears as the last five tiles of the dk/dv family: four for rows
-    of up to 256, 512, 768, 1024 keys, for 16-bit inputs, and one that runs longer rows (up to
+    """The row-resident kernel appears as the last eight tiles of the dk/dv family: seven for rows
+    of up to 256, 384, ..., 1024 keys, for 16-bit inputs, and one that runs longer rows (up to
     8192 keys at head dim 32) in passes of 1024 keys; they are the default where they are fastest."""
     lib = _lib.load()
     nt = lib.trifast_num_tiles(_lib.KERNEL_BWD_KV)
     fused = [t for t in range(nt) if lib.trifast_bwd_kv_tile_writes_dq(t)]
-    assert fused == list(range(nt - 5, nt))
+    assert fused == list(range(nt - 8, nt))
     assert not lib.trifast_bwd_kv_tile_writes_dq(-1) and not lib.trifast_bwd_kv_tile_writes_dq(nt)
-    passes = fused[4]
+    passes = fused[7]
     sup = lambda n, d, code: bool(lib.trifast_supports(_lib.KERNEL_BWD_KV, passes, n, 4, d, code))
     assert sup(1025, 32, _lib.BF16) and sup(8192, 32, _lib.F16) and sup(2047, 32, _lib.BF16)
     assert not sup(1024, 32, _lib.BF16) and not sup(8193, 32, _lib.BF16)
@@ -189,7 +189,7 @@ def test_row_resident_tiles_in_the_library_tables():
     # its low parts of dq live in the workspace tail, which is at least one more 16-bit tensor
     ws = lambda n, d: lib.trifast_bwd_workspace_bytes(1, 4, n, d, _lib.BF16)
     assert ws(2048, 32) - ws(2048, 64) >= 4 * 2048 * 2048 * 32 * 2 - 4 * 4 * 2048 * 2048 * 4
-    for t, keys in zip(fused[:4], (256, 512, 768, 1024)):
+    for t, keys in zip(fused[:7], (256, 384, 512, 640, 768, 896, 1024)):
         assert _lib.tile_info(_lib.KERNEL_BWD_KV, t)["BLOCK_K"] == keys
         assert lib.trifast_supports(_lib.KERNEL_BWD_KV, t, keys, 4, 32, _lib.BF16)
         assert lib.trifast_supports(_lib.KERNEL_BWD_KV, t, keys - 37, 2, 32, _lib.F16)
@@ -197,7 +197,8 @@ def test_row_resident_tiles_in_the_library_tables():
         assert not lib.trifast_supports(_lib.KERNEL_BWD_KV, t, keys, 4, 32, _lib.F32)
         assert not lib.trifast_supports(_lib.KERNEL_BWD_KV, t, keys, 4, 128, _lib.BF16)
     default = lambda n, d, code: lib.trifast_default_tile(_lib.KERNEL_BWD_KV, n, 4, d, code)
-    assert default(1024, 32, _lib.BF16) == fused[3] and default(300, 32, _lib.F16) == fused[1]
+    assert default(1024, 32, _lib.BF16) == fused[6] and default(300, 32, _lib.F16) == fused[1] and default(385, 32, _lib.F16) == fused[2]
+    assert default(640, 32, _lib.BF16) == fused[3] and default(641, 32, _lib.BF16) == fused[4] and default(896, 32, _lib.BF16) == fused[5]
     assert default(129, 32, _lib.BF16) == fused[0] and default(1025, 32, _lib.BF16) == passes and default(8193, 32, _lib.BF16) not in fused
     assert default(128, 32, _lib.BF16) not in fused and default(512, 64, _lib.BF16) not in fused
     assert default(512, 32, _lib.F32) not in fused

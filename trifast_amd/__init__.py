@@ -7,6 +7,6 @@ that calls the operator in AlphaFold-style models.
 
 from trifast_amd.torch import triangle_attention, triangle_attention_ending_node
 
-__version__ = "0.1.12"
+__version__ = "0.1.13"
 
 __all__ = ["triangle_attention", "triangle_attention_ending_node"]

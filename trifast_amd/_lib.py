@@ -12,7 +12,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libtrifast_hip.so"
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 F32, BF16, F16 = 0, 1, 2
 KERNEL_FWD, KERNEL_BWD_Q, KERNEL_BWD_KV, KERNEL_BWD_B = 0, 1, 2, 3

@@ -35,7 +35,7 @@ struct BwdKVFamily {
 };
 
 // tile ids: the streaming tiles above, then the row-resident ones (tri_bwd_row.hpp)
-constexpr int kRowKeyTiles[kBwdRowTiles] = {2, 4, 6, 8, 64};  // (the last one: up to eight passes of 8)
+constexpr int kRowKeyTiles[kBwdRowTiles] = {2, 3, 4, 5, 6, 7, 8, 64};  // (the last one: up to eight passes of 8)
 
 hipError_t row_launch(const BwdArgs& a, int bh, int d, int dtype, int tile, hipStream_t st, bool dry) {
   switch (dtype) {

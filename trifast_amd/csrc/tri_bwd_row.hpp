@@ -485,18 +485,19 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
         E::mfma_acc_zero(dkacc[t][mt]);
         E::mfma_acc_zero(dvacc[t][mt]);
       }
-    static_assert(KT % 2 == 0, "the two-slot bias ring assumes an even number of key tiles per wave");
     // The wave is alone on its SIMD, so nothing but its own instruction order hides a
     // latency: the code below is laid out as the schedule it should run in, and scheduling
     // barriers between the pieces keep the compiler from re-ordering it.
     auto SB = [] { __builtin_amdgcn_sched_barrier(0); };
     constexpr int NACC = 2 * PS * DM;  // dv, dk MFMAs of a tile
     constexpr int NDQ = PS * DM;       // dq MFMAs of a tile
-    // packed bias of key tile t (t >= KT: tile t - KT of the next query tile) -> ring slot t % 2,
-    // fetched two steps before its use (global memory, through L2)
+    // packed bias of key tile t (t >= KT: tile t - KT of the next query tile) -> the ring slot
+    // of that tile's parity, fetched two steps before its use (global memory, through L2).
+    // (With an odd KT, tile 0 of the next query tile goes to the slot that tile KT-1 is read
+    // from in the same step: its fetch follows the last MFMA that reads bias words.)
     u32x4v bias_ring[2][2] = {};
     auto fetch_bias = [&](int jt, int t) {
-      if constexpr (!FLAGGED) bias_load(jt + t / KT, t % KT, bias_ring[t % 2]);
+      if constexpr (!FLAGGED) bias_load(jt + t / KT, t % KT, bias_ring[(t % KT) % 2]);
     };
     fetch_bias(0, 0);
     fetch_bias(0, 1);

@@ -7,7 +7,7 @@
 namespace tri {
 
 // tile index -> key tiles per wave; a workgroup holds rows of up to 128 * KT keys
-constexpr int kRowKT[kBwdRowTiles] = {2, 4, 6, 8, 8};  // (the last one: several passes of 8)
+constexpr int kRowKT[kBwdRowTiles] = {2, 3, 4, 5, 6, 7, 8, 8};  // (the last one: several passes of 8)
 
 template <typename T, int D, int KT>
 hipError_t bwd_row_run(const BwdArgs& a, int bh, hipStream_t st, bool dry) {
@@ -51,10 +51,15 @@ hipError_t bwd_row_run_multi(const BwdArgs& a, int bh, hipStream_t st, bool dry)
       ap.pass_flags = (p > 0 ? 1 : 0) | (p + 1 < passes ? 2 : 0);
       const int left = a.nwords - p * per_pass;  // key tiles from this pass on
       hipError_t e;
-      if (left <= 2 * kRowWaves) e = bwd_row_pass<T, D, 2>(ap, bh, st);
-      else if (left <= 4 * kRowWaves) e = bwd_row_pass<T, D, 4>(ap, bh, st);
-      else if (left <= 6 * kRowWaves) e = bwd_row_pass<T, D, 6>(ap, bh, st);
-      else e = bwd_row_pass<T, D, 8>(ap, bh, st);
+      switch ((left + kRowWaves - 1) / kRowWaves) {
+        case 1:
+        case 2: e = bwd_row_pass<T, D, 2>(ap, bh, st); break;
+        case 3: e = bwd_row_pass<T, D, 3>(ap, bh, st); break;
+        case 4: e = bwd_row_pass<T, D, 4>(ap, bh, st); break;
+        case 5: e = bwd_row_pass<T, D, 5>(ap, bh, st); break;
+        case 6: e = bwd_row_pass<T, D, 6>(ap, bh, st); break;
+        default: e = bwd_row_pass<T, D, 8>(ap, bh, st); break;  // (7 key tiles per wave spill in this variant)
+      }
       if (e != hipSuccess) return e;
     }
     return hipSuccess;
@@ -70,7 +75,10 @@ hipError_t bwd_row_dispatch_kt(const BwdArgs& a, int bh, int tile, hipStream_t s
     case 1: return bwd_row_run<T, D, kRowKT[1]>(a, bh, st, dry);
     case 2: return bwd_row_run<T, D, kRowKT[2]>(a, bh, st, dry);
     case 3: return bwd_row_run<T, D, kRowKT[3]>(a, bh, st, dry);
-    case 4: return bwd_row_run_multi<T, D>(a, bh, st, dry);
+    case 4: return bwd_row_run<T, D, kRowKT[4]>(a, bh, st, dry);
+    case 5: return bwd_row_run<T, D, kRowKT[5]>(a, bh, st, dry);
+    case 6: return bwd_row_run<T, D, kRowKT[6]>(a, bh, st, dry);
+    case 7: return bwd_row_run_multi<T, D>(a, bh, st, dry);
   }
   return hipErrorInvalidValue;
 }

@@ -367,9 +367,9 @@ int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype)
       pick = (n <= 64 || row_bytes >= 256 || (row_bytes == 128 && dtype != TRIFAST_F32)) ? 0 : 1;
       // 64-byte rows of 129..1024 keys: the row-resident tile that also produces dq, with as
       // few key tiles per wave as hold the row (ids follow the four streaming tiles)
-      if (row_bytes == 64 && dtype != TRIFAST_F32 && n > 128 && n <= 1024) pick = 4 + (int)((n - 1) / 256);
+      if (row_bytes == 64 && dtype != TRIFAST_F32 && n > 128 && n <= 1024) pick = 4 + (int)((n - 1) / 128) - 1;
       // longer rows of head dim 32: the same kernel in passes of 1024 keys
-      if (d == 32 && dtype != TRIFAST_F32 && n > 1024 && n <= 8192) pick = 8;
+      if (d == 32 && dtype != TRIFAST_F32 && n > 1024 && n <= 8192) pick = tri::bwd_kv_num_tiles() - 1;
       break;
     case TRIFAST_KERNEL_BWD_B:  // 128 x 128 block of 16 waves; 8 waves, then 64 x 64 of 4 waves, as rows widen or n shrinks
       pick = (n <= 128 || row_bytes >= 256) ? 2 : (row_bytes == 128 ? 3 : 4);

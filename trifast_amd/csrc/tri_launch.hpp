@@ -29,7 +29,7 @@ hipError_t bwd_kv_launch(const BwdArgs& a, int bh, int d, int dtype, int tile, h
 // Row-resident tiles of the dk/dv family: they also produce dq (and the per-query
 // planes the db kernel reads), so the dq kernel is not launched with them.  Their tile
 // ids follow the streaming dk/dv tiles.
-constexpr int kBwdRowTiles = 5;
+constexpr int kBwdRowTiles = 8;
 bool bwd_kv_tile_writes_dq(int tile);
 hipError_t bwd_row_launch_bf16(const BwdArgs& a, int bh, int d, int tile, hipStream_t st, bool dry);
 hipError_t bwd_row_launch_f16(const BwdArgs& a, int bh, int d, int tile, hipStream_t st, bool dry);
