@@ -317,3 +317,51 @@ def test_projection_with_heads_outermost_outputs():
     for a, r in zip(o1 + g1, o2 + g2):
         assert a.shape == r.shape
         assert (a - r).abs().max().item() <= 2.0**-7 * r.abs().max().item(), f"{(a - r).abs().max().item():.3e} of {r.abs().max().item():.3e}"
+
+
+def test_block_kernels_are_well_formed_custom_ops():
+    """The block's kernels are torch.library ops like the operator: schema, shape-only
+    implementation and autograd registration agree with the real kernels."""
+    from torch.library import opcheck
+
+    gen = torch.Generator().manual_seed(21)
+    dtype, h, n, d, k = torch.bfloat16, 2, 24, 16, 64
+    o = torch.randn(1, h, n, n, d, generator=gen).to(DEV, dtype).requires_grad_(True)
+    g = torch.randn(1, n, n, h * d, generator=gen).to(DEV, dtype).requires_grad_(True)
+    opcheck(nn._gated_output, (o, g), raise_exception=True)
+    opcheck(nn._gated_output_bwd, (torch.randn_like(g), o.detach(), g.detach()), raise_exception=True)
+    rows = n * n
+    x = torch.randn(rows, k, generator=gen).to(DEV, dtype)
+    ws = [(torch.randn(m, k, generator=gen) * k**-0.5).to(DEV, dtype) for m in (h * d, 4)]
+    bs = [None, torch.randn(4, generator=gen).to(DEV, dtype)]
+    opcheck(nn._linear_outputs, (x, ws, bs, [d, 0]), raise_exception=True)
+    dys = [torch.randn(h, rows, d, generator=gen).to(DEV, dtype), torch.randn(rows, 4, generator=gen).to(DEV, dtype)]
+    opcheck(nn._linear_input_grad, (dys, ws, [d, 0]), raise_exception=True)
+    opcheck(nn._linear_weight_grad, (dys[0], x, d, False), raise_exception=True)
+    opcheck(nn._linear_weight_grad, (dys[1], x, 0, True), raise_exception=True)
+
+
+@pytest.mark.parametrize("ending_node", [False, True], ids=["starting", "ending"])
+def test_block_compiles_as_one_graph(ending_node):
+    """torch.compile traces the whole block, forward and backward, without a graph break, and the
+    compiled block gives the bits of the eager one (aot_eager: the traced graphs run as they are)."""
+    torch.manual_seed(5)
+    dtype = torch.bfloat16
+    block = nn.TriangleAttention(64, 2, 32, ending_node=ending_node).to(DEV, dtype)
+    x = torch.randn(2, 40, 40, 64, device=DEV, dtype=dtype)
+    mask = torch.rand(2, 40, 40, device=DEV) < 0.3
+    dy = torch.randn(2, 40, 40, 64, device=DEV, dtype=dtype)
+    explanation = torch._dynamo.explain(block)(x, mask)
+    assert explanation.graph_break_count == 0, explanation
+
+    def run(fn):
+        xi = x.clone().requires_grad_(True)
+        block.zero_grad(set_to_none=True)
+        y = fn(xi, mask)
+        y.backward(dy)
+        return [y.detach(), xi.grad] + [p.grad.clone() for p in block.parameters()]
+
+    eager = run(block)
+    compiled = run(torch.compile(block, fullgraph=True, backend="aot_eager"))
+    for a, b in zip(compiled, eager):
+        assert torch.equal(a, b)

@@ -25,6 +25,8 @@ tensor is copied to change its layout:
 
 from __future__ import annotations
 
+from typing import Optional, Sequence
+
 import torch
 
 from trifast_amd import _lib
@@ -49,39 +51,69 @@ def _gate_shapes(o: torch.Tensor, g: torch.Tensor) -> tuple[int, int, int, int]:
     return b, h, n, d
 
 
-class _GatedOutput(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
-        b, h, n, d = _gate_shapes(o, g)
-        o, g = o.contiguous(), g.contiguous()
-        y = torch.empty_like(g)
-        if y.numel():
-            with torch.cuda.device(o.device):
-                rc = _lib.load().trifast_gate_fwd(y.data_ptr(), o.data_ptr(), g.data_ptr(), b, h, n, d, _dtype_code(o),
-                                                  torch.cuda.current_stream(o.device).cuda_stream)
-            _lib.check(rc, "trifast_gate_fwd")
-        ctx.save_for_backward(o, g)
-        ctx.dims = (b, h, n, d)
-        return y
+def _dims4(o: torch.Tensor) -> tuple[int, int, int, int]:
+    *lead, h, n, _, d = o.shape
+    b = 1
+    for s in lead:
+        b *= s
+    return b, h, n, d
 
-    @staticmethod
-    def backward(ctx, dy: torch.Tensor):
-        o, g = ctx.saved_tensors
-        b, h, n, d = ctx.dims
-        dy = dy.contiguous()
-        do, dg = torch.empty_like(o), torch.empty_like(g)
-        if dy.numel():
-            with torch.cuda.device(o.device):
-                rc = _lib.load().trifast_gate_bwd(do.data_ptr(), dg.data_ptr(), dy.data_ptr(), o.data_ptr(), g.data_ptr(),
-                                                  b, h, n, d, _dtype_code(o), torch.cuda.current_stream(o.device).cuda_stream)
-            _lib.check(rc, "trifast_gate_bwd")
-        return do, dg
+
+# The kernels are torch.library custom ops, like the operator itself: opaque to a tracing
+# compiler (torch.compile sees one node each), with shape-only implementations for it.
+@torch.library.custom_op("trifast::gated_output", mutates_args=())
+def _gated_output(o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+    b, h, n, d = _dims4(o)
+    o, g = o.contiguous(), g.contiguous()
+    y = torch.empty_like(g)
+    if y.numel():
+        with torch.cuda.device(o.device):
+            rc = _lib.load().trifast_gate_fwd(y.data_ptr(), o.data_ptr(), g.data_ptr(), b, h, n, d, _dtype_code(o),
+                                              torch.cuda.current_stream(o.device).cuda_stream)
+        _lib.check(rc, "trifast_gate_fwd")
+    return y
+
+
+@_gated_output.register_fake
+def _(o, g):
+    return g.new_empty(g.shape)
+
+
+@torch.library.custom_op("trifast::gated_output_backward", mutates_args=())
+def _gated_output_bwd(dy: torch.Tensor, o: torch.Tensor, g: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    b, h, n, d = _dims4(o)
+    dy, o, g = dy.contiguous(), o.contiguous(), g.contiguous()
+    do, dg = torch.empty_like(o), torch.empty_like(g)
+    if dy.numel():
+        with torch.cuda.device(o.device):
+            rc = _lib.load().trifast_gate_bwd(do.data_ptr(), dg.data_ptr(), dy.data_ptr(), o.data_ptr(), g.data_ptr(),
+                                              b, h, n, d, _dtype_code(o), torch.cuda.current_stream(o.device).cuda_stream)
+        _lib.check(rc, "trifast_gate_bwd")
+    return do, dg
+
+
+@_gated_output_bwd.register_fake
+def _(dy, o, g):
+    return o.new_empty(o.shape), g.new_empty(g.shape)
+
+
+def _gate_setup(ctx, inputs, output) -> None:
+    ctx.save_for_backward(*inputs)
+
+
+def _gate_backward(ctx, dy):
+    o, g = ctx.saved_tensors
+    return _gated_output_bwd(dy, o, g)
+
+
+_gated_output.register_autograd(_gate_backward, setup_context=_gate_setup)
 
 
 def gated_output(o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
     """``y[*, i, j, h*d] = o[*, h, i, j, d] * sigmoid(g[*, i, j, h*d])``: the operator's output
     gated and handed to the output projection in one pass."""
-    return _GatedOutput.apply(o, g)
+    _gate_shapes(o, g)
+    return _gated_output(o, g)
 
 
 _DW_K = (32, 64, 128, 256)
@@ -98,22 +130,34 @@ def _rows_n(dy: torch.Tensor, head_dim: int) -> tuple[int, int]:
     return (dy.shape[1], dy.shape[0] * dy.shape[2]) if head_dim else (dy.shape[0], dy.shape[1])
 
 
-def linear_weight_grad(dy: torch.Tensor, x: torch.Tensor, head_dim: int = 0, with_bias: bool = False):
-    """``dy^T x`` for ``dy [rows, n]``, ``x [rows, k]``: the weight gradient of a linear layer, with
-    the long contraction over the rows split over the whole GPU (``trifast_linear_dw``).  With
-    ``head_dim = d``, dy is ``[n / d, rows, d]`` (heads outermost).  ``with_bias``: also the bias
-    gradient ``dy.sum(0)`` from the same pass; the result is then the pair (dw, db)."""
+@torch.library.custom_op("trifast::linear_weight_grad", mutates_args=())
+def _linear_weight_grad(dy: torch.Tensor, x: torch.Tensor, head_dim: int, with_bias: bool) -> tuple[torch.Tensor, torch.Tensor]:
     dy, x = dy.contiguous(), x.contiguous()
     rows, n = _rows_n(dy, head_dim)
     k = x.shape[1]
     lib = _lib.load()
     dw = torch.empty(n, k, dtype=x.dtype, device=x.device)
-    db = torch.empty(n, dtype=x.dtype, device=x.device) if with_bias else None
+    db = torch.empty(n if with_bias else 0, dtype=x.dtype, device=x.device)
     ws = torch.empty(lib.trifast_linear_dw_workspace_bytes(rows, k, n), dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
-        rc = lib.trifast_linear_dw(dw.data_ptr(), None if db is None else db.data_ptr(), dy.data_ptr(), x.data_ptr(), rows, k, n, head_dim,
+        rc = lib.trifast_linear_dw(dw.data_ptr(), db.data_ptr() if with_bias else None, dy.data_ptr(), x.data_ptr(), rows, k, n, head_dim,
                                    _dtype_code(x), ws.data_ptr(), ws.numel(), torch.cuda.current_stream(x.device).cuda_stream)
     _lib.check(rc, "trifast_linear_dw")
+    return dw, db
+
+
+@_linear_weight_grad.register_fake
+def _(dy, x, head_dim, with_bias):
+    n = _rows_n(dy, head_dim)[1]
+    return x.new_empty((n, x.shape[1])), x.new_empty((n if with_bias else 0,))
+
+
+def linear_weight_grad(dy: torch.Tensor, x: torch.Tensor, head_dim: int = 0, with_bias: bool = False):
+    """``dy^T x`` for ``dy [rows, n]``, ``x [rows, k]``: the weight gradient of a linear layer, with
+    the long contraction over the rows split over the whole GPU (``trifast_linear_dw``).  With
+    ``head_dim = d``, dy is ``[n / d, rows, d]`` (heads outermost).  ``with_bias``: also the bias
+    gradient ``dy.sum(0)`` from the same pass; the result is then the pair (dw, db)."""
+    dw, db = _linear_weight_grad(dy, x, head_dim, with_bias)
     return (dw, db) if with_bias else dw
 
 
@@ -141,11 +185,8 @@ _DX_K = (32, 64, 128)
 _DX_LAYERS = 6
 
 
-def linear_input_grad(dys, weights, head_dims=None) -> torch.Tensor:
-    """``sum_p dys[p] @ weights[p]`` for ``dys[p] [rows, n_p]``, ``weights[p] [n_p, k]``: the input
-    gradient of several linear layers over one input, every ``dys[p]`` read once and the sum
-    written once (``trifast_linear_dx``).  ``head_dims[p] = d``: ``dys[p]`` is ``[n_p / d, rows, d]``."""
-    head_dims = list(head_dims) if head_dims is not None else [0] * len(dys)
+@torch.library.custom_op("trifast::linear_input_grad", mutates_args=())
+def _linear_input_grad(dys: Sequence[torch.Tensor], weights: Sequence[torch.Tensor], head_dims: Sequence[int]) -> torch.Tensor:
     dys = [dy.contiguous() for dy in dys]
     wts = [w.t().contiguous() for w in weights]  # [k, n_p]: a few tens of KiB each
     rows, k = _rows_n(dys[0], head_dims[0])[0], weights[0].shape[1]
@@ -153,27 +194,53 @@ def linear_input_grad(dys, weights, head_dims=None) -> torch.Tensor:
     ptrs = lambda ts: (_lib.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
     with torch.cuda.device(dx.device):
         rc = _lib.load().trifast_linear_dx(dx.data_ptr(), rows, k, len(dys), ptrs(dys), ptrs(wts), _lib.i64_array([w.shape[0] for w in weights]),
-                                           _lib.i64_array(head_dims), _dtype_code(dx), torch.cuda.current_stream(dx.device).cuda_stream)
+                                           _lib.i64_array(list(head_dims)), _dtype_code(dx), torch.cuda.current_stream(dx.device).cuda_stream)
     _lib.check(rc, "trifast_linear_dx")
     return dx
+
+
+@_linear_input_grad.register_fake
+def _(dys, weights, head_dims):
+    return dys[0].new_empty((_rows_n(dys[0], head_dims[0])[0], weights[0].shape[1]))
+
+
+def linear_input_grad(dys, weights, head_dims=None) -> torch.Tensor:
+    """``sum_p dys[p] @ weights[p]`` for ``dys[p] [rows, n_p]``, ``weights[p] [n_p, k]``: the input
+    gradient of several linear layers over one input, every ``dys[p]`` read once and the sum
+    written once (``trifast_linear_dx``).  ``head_dims[p] = d``: ``dys[p]`` is ``[n_p / d, rows, d]``."""
+    return _linear_input_grad(list(dys), list(weights), list(head_dims) if head_dims is not None else [0] * len(dys))
+
+
+def _output_shape(rows: int, n: int, d: int) -> tuple[int, ...]:
+    return (n // d, rows, d) if d else (rows, n)
+
+
+@torch.library.custom_op("trifast::linear_outputs", mutates_args=())
+def _linear_outputs(x: torch.Tensor, weights: Sequence[torch.Tensor], biases: Sequence[Optional[torch.Tensor]],
+                    head_dims: Sequence[int]) -> list[torch.Tensor]:
+    x = x.contiguous()
+    rows, k = x.shape
+    ws = [w.contiguous() for w in weights]
+    bs = [None if b is None else b.contiguous() for b in biases]
+    ys = [torch.empty(_output_shape(rows, w.shape[0], d), dtype=x.dtype, device=x.device) for w, d in zip(ws, head_dims)]
+    ptrs = lambda ts: (_lib.c_void_p * len(ts))(*[None if t is None else t.data_ptr() for t in ts])
+    with torch.cuda.device(x.device):
+        rc = _lib.load().trifast_linear_fwd(x.data_ptr(), rows, k, len(ws), ptrs(ws), ptrs(bs), ptrs(ys), _lib.i64_array([w.shape[0] for w in ws]),
+                                            _lib.i64_array(list(head_dims)), _dtype_code(x), torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, "trifast_linear_fwd")
+    return ys
+
+
+@_linear_outputs.register_fake
+def _(x, weights, biases, head_dims):
+    return [x.new_empty(_output_shape(x.shape[0], w.shape[0], d)) for w, d in zip(weights, head_dims)]
 
 
 def linear_outputs(x: torch.Tensor, weights, biases, head_dims=None) -> list[torch.Tensor]:
     """``[x @ w.T + b for w, b in zip(weights, biases)]`` for ``x [rows, k]`` in one pass that reads
     x once (``trifast_linear_fwd``); a bias may be None.  ``head_dims[p] = d``: output p comes
     heads-outermost, ``[n_p / d, rows, d]``."""
-    head_dims = list(head_dims) if head_dims is not None else [0] * len(weights)
-    x = x.contiguous()
-    rows, k = x.shape
-    ws = [w.contiguous() for w in weights]
-    bs = [None if b is None else b.contiguous() for b in biases]
-    ys = [torch.empty((w.shape[0] // d, rows, d) if d else (rows, w.shape[0]), dtype=x.dtype, device=x.device) for w, d in zip(ws, head_dims)]
-    ptrs = lambda ts: (_lib.c_void_p * len(ts))(*[None if t is None else t.data_ptr() for t in ts])
-    with torch.cuda.device(x.device):
-        rc = _lib.load().trifast_linear_fwd(x.data_ptr(), rows, k, len(ws), ptrs(ws), ptrs(bs), ptrs(ys), _lib.i64_array([w.shape[0] for w in ws]),
-                                            _lib.i64_array(head_dims), _dtype_code(x), torch.cuda.current_stream(x.device).cuda_stream)
-    _lib.check(rc, "trifast_linear_fwd")
-    return ys
+    return _linear_outputs(x, list(weights), list(biases), list(head_dims) if head_dims is not None else [0] * len(weights))
 
 
 class _Project(torch.autograd.Function):
@@ -237,7 +304,7 @@ def project(x: torch.Tensor, layers, head_dims=None) -> tuple[torch.Tensor, ...]
     fastest; the kernels write and read that layout directly (elsewhere it is a copy)."""
     layers = list(layers)
     head_dims = tuple(head_dims) if head_dims is not None else (0,) * len(layers)
-    fused = bool(layers) and len(layers) <= _DX_LAYERS and all(_dw_ready(x, m.weight) for m in layers)
+    fused = 0 < len(layers) <= _DX_LAYERS and all(_dw_ready(x, m.weight) for m in layers)
     if not fused or x.shape[-1] not in _DX_K:
         ys = _Project.apply(x, (0,) * len(layers), *[m.weight for m in layers], *[m.bias for m in layers]) if fused else tuple(m(x) for m in layers)
         return tuple(y.unflatten(-1, (-1, d)).movedim(-2, 0).contiguous() if d else y for y, d in zip(ys, head_dims))

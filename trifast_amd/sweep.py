@@ -142,7 +142,7 @@ def block(n: int, c_in: int) -> None:
     g = torch.randn(1, n, n, H * D, device=dev, dtype=DTYPE)
     gy = torch.randn_like(g)
     size = o.numel() * o.element_size()
-    ms = _median_ms(lambda: nn._GatedOutput.apply(o, g))
+    ms = _median_ms(lambda: nn.gated_output(o, g))
     print(f"gate forward  {ms * 1e3:8.1f} us  {3 * size / ms / 1e6:7.1f} GB/s of 3 tensors x {size / 2**20:.0f} MiB")
     oo, gg = o.clone().requires_grad_(True), g.clone().requires_grad_(True)
     y = nn.gated_output(oo, gg)
