@@ -51,17 +51,38 @@ hipError_t dispatch(const Args& a, int bh, int d, int dtype, int tile, hipStream
 constexpr int kMaxStaticLds = 64 * 1024;
 constexpr int kMaxLds = 160 * 1024;  // LDS per workgroup on gfx950
 
-// Launch with `lds` bytes of dynamic LDS; above the default 64 KiB limit the
-// kernel's attribute has to be raised first (once per instantiation).
+// More dynamic LDS than the default 64 KiB limit: the kernel's attribute has to be raised
+// first, once per kernel and device (each device holds its own copy of the code object).
+// Every thread keeps its own note of the (kernel, device) pairs it has done.
+inline hipError_t raise_lds_limit(const void* kernel, int lds) {
+  struct Note { const void* kernel; uint64_t devices; };
+  constexpr int kNotes = 256;
+  static thread_local Note notes[kNotes];
+  static thread_local int count = 0;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = dev < 64 ? (uint64_t)1 << dev : 0;  // (devices past 63: raised on every call)
+  Note* note = nullptr;
+  for (int i = 0; i < count && !note; ++i)
+    if (notes[i].kernel == kernel) note = &notes[i];
+  if (note && (note->devices & bit)) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  if (e != hipSuccess) return e;
+  if (!note && count < kNotes) {  // (a full table: raised on every call, which is only slower)
+    note = &notes[count++];
+    *note = Note{kernel, 0};
+  }
+  if (note) note->devices |= bit;
+  return hipSuccess;
+}
+
+// Launch with `lds` bytes of dynamic LDS.
 template <typename Kernel, typename Args>
 hipError_t launch_dyn(Kernel kernel, dim3 grid, dim3 block, int lds, hipStream_t st, const Args& a) {
   if (lds > kMaxStaticLds) {
-    static thread_local const void* raised = nullptr;
-    if (raised != reinterpret_cast<const void*>(kernel)) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-      if (e != hipSuccess) return e;
-      raised = reinterpret_cast<const void*>(kernel);
-    }
+    const hipError_t e = raise_lds_limit(reinterpret_cast<const void*>(kernel), lds);
+    if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
   return hipGetLastError();

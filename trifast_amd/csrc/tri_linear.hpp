@@ -18,6 +18,7 @@
 #include <type_traits>
 
 #include "tri_common.hpp"
+#include "tri_dispatch.hpp"
 
 namespace tri {
 
@@ -647,13 +648,9 @@ inline hipError_t linear_fwd_launch_k(const LinearFwdArgs& a, hipStream_t st) {
   const dim3 grid((unsigned)((a.rows + 255) / 256)), block(256);
   constexpr int lds = linear_fwd_lds_bytes(KD, (int)sizeof(T));
   if (lds > 64 * 1024) {
-    // (more dynamic LDS than the default limit: raised once per kernel)
-    static thread_local bool raised = false;
-    if (!raised) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(linear_fwd_kernel<T, KD>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-      if (e != hipSuccess) return e;
-      raised = true;
-    }
+    // (more dynamic LDS than the default limit: raised once per kernel and device)
+    const hipError_t e = raise_lds_limit(reinterpret_cast<const void*>(linear_fwd_kernel<T, KD>), lds);
+    if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL((linear_fwd_kernel<T, KD>), grid, block, lds, st, a);
   return hipGetLastError();
