@@ -104,3 +104,20 @@ def test_hip_graph_capture_and_replay():
         torch.cuda.synchronize()
         for name, x, e in zip(("o", "dq", "dk", "dv", "db"), got, (eo, eq.grad, ek.grad, ev.grad, eb.grad)):
             assert torch.equal(x, e.detach()), f"replay {trial}: {name} differs from the eager result"
+
+
+def test_compile_with_dynamic_shapes():
+    """One compiled graph with symbolic sizes serves several n (the shape-only implementations
+    work on symbolic ints) and gives the eager bits, forward and backward."""
+    compiled = torch.compile(trifast_amd.triangle_attention, fullgraph=True, backend="aot_eager", dynamic=True)
+    for n in (48, 64, 80):
+        q, k, v, b, m = gen_tensors(n, 32, 2, True, "cuda", dtype=torch.bfloat16)
+        qc, kc, vc, bc = (t.detach().clone().requires_grad_(True) for t in (q, k, v, b))
+        qe, ke, ve, be = (t.detach().clone().requires_grad_(True) for t in (q, k, v, b))
+        oc = compiled(qc, kc, vc, bc, m)
+        oe = trifast_amd.triangle_attention(qe, ke, ve, be, m)
+        assert torch.equal(oc, oe)
+        oc.sum().backward()
+        oe.sum().backward()
+        for name, x, y in zip(("dq", "dk", "dv", "db"), (qc.grad, kc.grad, vc.grad, bc.grad), (qe.grad, ke.grad, ve.grad, be.grad)):
+            assert torch.equal(x, y), f"n={n}: {name} differs between compiled and eager"
