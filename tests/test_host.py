@@ -200,8 +200,11 @@ def test_row_resident_tiles_in_the_library_tables():
     assert default(1024, 32, _lib.BF16) == fused[6] and default(300, 32, _lib.F16) == fused[1] and default(385, 32, _lib.F16) == fused[2]
     assert default(640, 32, _lib.BF16) == fused[3] and default(641, 32, _lib.BF16) == fused[4] and default(896, 32, _lib.BF16) == fused[5]
     assert default(129, 32, _lib.BF16) == fused[0] and default(1025, 32, _lib.BF16) == passes and default(8193, 32, _lib.BF16) not in fused
-    assert default(128, 32, _lib.BF16) not in fused and default(512, 64, _lib.BF16) not in fused
-    assert default(512, 32, _lib.F32) not in fused
+    # (from the smallest rows on: one launch instead of two; head dim 16 like 32, head dim 64 up to 384 keys)
+    assert default(128, 32, _lib.BF16) == fused[0] and default(16, 32, _lib.F16) == fused[0]
+    assert default(700, 16, _lib.BF16) == fused[4] and default(1025, 16, _lib.BF16) not in fused
+    assert default(300, 64, _lib.F16) == fused[1] and default(385, 64, _lib.F16) not in fused and default(512, 64, _lib.BF16) not in fused
+    assert default(512, 32, _lib.F32) not in fused and default(64, 128, _lib.BF16) not in fused
 
 
 def test_tune_cli_flags_and_sweep():

@@ -365,9 +365,11 @@ int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype)
       break;
     case TRIFAST_KERNEL_BWD_KV:  // 2 pair rows, 32 queries per stage; one row, 64 queries for wide 16-bit rows
       pick = (n <= 64 || row_bytes >= 256 || (row_bytes == 128 && dtype != TRIFAST_F32)) ? 0 : 1;
-      // 64-byte rows of 129..1024 keys: the row-resident tile that also produces dq, with as
-      // few key tiles per wave as hold the row (ids follow the four streaming tiles)
-      if (row_bytes == 64 && dtype != TRIFAST_F32 && n > 128 && n <= 1024) pick = 4 + (int)((n - 1) / 128) - 1;
+      // 16-bit rows of up to 1024 keys at head dim 16 or 32, up to 384 keys at head dim 64 (more
+      // of them spill): the row-resident tile that also produces dq, with as few key tiles per
+      // wave as hold the row (ids follow the four streaming tiles).  It wins from the smallest
+      // rows on, where it is one launch instead of two.
+      if (dtype != TRIFAST_F32 && n <= 1024 && (d == 16 || d == 32 || (d == 64 && n <= 384))) pick = 4 + (n <= 256 ? 0 : (int)((n - 1) / 128) - 1);
       // longer rows of head dim 32: the same kernel in passes of 1024 keys
       if (d == 32 && dtype != TRIFAST_F32 && n > 1024 && n <= 8192) pick = tri::bwd_kv_num_tiles() - 1;
       break;
