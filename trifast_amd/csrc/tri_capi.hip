@@ -357,8 +357,14 @@ int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype)
   const int64_t row_bytes = d * elem_size(dtype);
   int pick = 0;
   switch (kernel) {
-    case TRIFAST_KERNEL_FWD:  // 4 pair rows share a bias tile; 2 rows for 128-byte rows, one for wider ones
-      pick = (n <= 64 || row_bytes >= 256) ? 0 : (row_bytes == 128 ? 4 : 3);
+    case TRIFAST_KERNEL_FWD:
+      // pair rows that share a bias tile: one for the smallest and the widest rows; two for
+      // 128-byte rows (one in fp32) and for 64-byte 16-bit rows of fewer than 1024 keys; four
+      // above that; 32-byte rows: four, or two with 64 keys per stage from 256 keys on
+      if (n <= 64 || row_bytes >= 256) pick = 0;
+      else if (row_bytes == 128) pick = dtype == TRIFAST_F32 ? 0 : 4;
+      else if (row_bytes == 64) pick = (dtype != TRIFAST_F32 && n < 1024) ? 4 : 3;
+      else pick = n >= 256 ? 1 : 3;
       break;
     case TRIFAST_KERNEL_BWD_Q:  // 2 pair rows, 64 keys per stage; one row from 128-byte rows on
       pick = (n <= 64 || row_bytes >= 128) ? 0 : 1;
@@ -373,8 +379,11 @@ int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype)
       // longer rows of head dim 32: the same kernel in passes of 1024 keys
       if (d == 32 && dtype != TRIFAST_F32 && n > 1024 && n <= 8192) pick = tri::bwd_kv_num_tiles() - 1;
       break;
-    case TRIFAST_KERNEL_BWD_B:  // 128 x 128 block of 16 waves; 8 waves, then 64 x 64 of 4 waves, as rows widen or n shrinks
-      pick = (n <= 128 || row_bytes >= 256) ? 2 : (row_bytes == 128 ? 3 : 4);
+    case TRIFAST_KERNEL_BWD_B:
+      // 64 x 64 block of 4 waves up to 256 keys (more workgroups than a larger block gives
+      // there), for 32-byte rows and for the widest ones; else 128 x 128 of 16 waves, of 8 waves
+      // for 128-byte rows
+      pick = (n <= 256 || row_bytes <= 32 || row_bytes >= 256) ? 2 : (row_bytes == 128 ? 3 : 4);
       break;
 
     default: return fail(TRIFAST_EINVAL, "unknown kernel id %d", kernel);
