@@ -60,33 +60,34 @@ bool bwd_b_supports(int tile, int64_t n, int d, int dtype) {
   return dispatch<BwdBFamily>(a, 1, d, dtype, tile, nullptr, true) == hipSuccess;
 }
 
-// The pair rows are split into chunks when one chunk would leave most of the
-// GPU idle (few query/key blocks at small n); every tile uses the same split so
-// that the workspace does not depend on the tile.
-// (`row_bytes`: bytes of a row of q.  The default tile for 64-byte rows is one workgroup of
-// 16 waves per CU, so 256 workgroups fill the GPU; the tiles of wider rows run two to four
-// per CU.  Measured at n = 1024, h = 4, d = 32: one chunk instead of two, which needs no
-// partials and no reduce pass, is 6 % faster.)
+// The pair rows are split into chunks when one chunk would leave part of the GPU idle;
+// every tile uses the same split so that the workspace does not depend on the tile.
+// The split follows a model of how the kernel occupies the GPU: the (batch*head, chunk)
+// groups go to the 8 XCDs in turn (fewer than 8 groups share the XCDs between them, a whole
+// number each), an XCD runs 32 workgroups of the large tiles at a time (one per CU), and a
+// workgroup takes one unit per pair row plus a start-up of about 8: the time is
+//   rounds of 32 workgroups on the fullest XCD  x  (rows per chunk + 8).
+// Measured against it (h = 4, d = 32, 128 x 128 blocks, microseconds against units): n = 320,
+// 5 chunks 73 / 72; 384, 6 chunks 79 / 72 and 8 chunks 115 / 112; 448, 4 chunks 120 / 120;
+// 768, 2 chunks 776 / 784; 1024, 1 chunk 1040 / 1032.  Up to 8 chunks of at least 16 rows;
+// with equal times the fewer chunks win (one chunk needs no partials and no reduce pass).
 int bwd_b_chunks(int64_t n, int64_t bh, int row_bytes) {
-  const int64_t blocks = ((n + 127) / 128) * ((n + 127) / 128) * bh;
-  const int64_t target = row_bytes <= 64 ? 256 : 512;
-  int64_t chunks = (target + blocks - 1) / blocks;
-  const int64_t max_chunks = (n + 63) / 64;  // at least 64 rows per chunk
-  if (chunks > max_chunks) chunks = max_chunks;
-  if (chunks > 8) chunks = 8;
-  if (chunks < 1) chunks = 1;
-  // The kernel runs each (batch*head, chunk) group on one XCD: when the rows are split
-  // anyway, make the number of groups a multiple of the 8 XCDs if the row count allows
-  // it.  (One chunk stays one chunk: it needs no partials and no reduce pass.)
-  if (chunks > 1) {
-    int64_t g = bh % 8 == 0 ? 8 : (bh % 4 == 0 ? 4 : (bh % 2 == 0 ? 2 : 1));
-    const int64_t m = 8 / g;  // chunks must be a multiple of m
-    const int64_t rounded = (chunks + m - 1) / m * m;
-    if (rounded <= max_chunks && rounded <= 8) chunks = rounded;
+  (void)row_bytes;
+  const int64_t blocks = ((n + 127) / 128) * ((n + 127) / 128);  // per group
+  const int64_t max_chunks = n / 16 < 1 ? 1 : (n / 16 > 8 ? 8 : n / 16);
+  int64_t best = 1, best_cost = -1;
+  for (int64_t c = 1; c <= max_chunks; ++c) {
+    const int64_t groups = bh * c;
+    // the groups are the grid's z extent (padded to a multiple of 8), at most 65535
+    if (c > 1 && (groups + 7) / 8 * 8 > 65535) break;
+    const int64_t on_xcd = groups >= 8 ? (groups + 7) / 8 * blocks : (blocks + 8 / groups - 1) / (8 / groups);
+    const int64_t cost = (on_xcd + 31) / 32 * ((n + c - 1) / c + 8);
+    if (best_cost < 0 || cost < best_cost) {
+      best = c;
+      best_cost = cost;
+    }
   }
-  // the groups are the grid's z extent (padded to a multiple of 8), at most 65535
-  while (chunks > 1 && (bh * chunks + 7) / 8 * 8 > 65535) --chunks;
-  return (int)chunks;
+  return (int)best;
 }
 
 hipError_t bwd_b_launch(const BwdArgs& a, int bh, int d, int dtype, int tile, hipStream_t st) {
