@@ -246,6 +246,15 @@ def test_db_chunks_do_not_inflate_the_workspace():
     assert per_head(5, 2048) <= 1.01 * per_head(8, 2048)
     assert per_head(5, 4096) <= 1.01 * per_head(8, 4096)
     assert per_head(1, 4096) <= 1.01 * per_head(8, 4096)
+    # The split follows where the (batch*head, chunk) groups land on the 8 XCDs: at n = 1024,
+    # h = 4 one chunk fills the GPU (no partials); at n = 768 two chunks would leave 36 workgroups
+    # on 32 CUs, and eight run; tiny rows split down to 16 rows per chunk.  The partials are
+    # fp32 [chunks, b*h, n, n] in the workspace tail (d = 64 has no other use for the tail).
+    # (before the tail: the lse and delta planes and two packed copies of the bias, three such units)
+    chunks = lambda h, n: lib.trifast_bwd_workspace_bytes(1, h, n, 64, _lib.BF16) // (h * n * n * 4) - 3
+    assert chunks(4, 1024) == chunks(4, 2048) == 0
+    assert chunks(4, 768) == 8 and chunks(4, 64) == 4 and chunks(4, 256) == 8
+    assert chunks(64, 256) == 0  # many heads fill the GPU with one chunk
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
