@@ -132,16 +132,6 @@ struct RowSchedOf {
   static constexpr RowSched value = make_row_sched(HAS_PREV, HAS_NEXT, FLAGGED, NSB, DS, NACC, NDQ);
 };
 
-template <typename F, int... I>
-TRI_DEV void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in order
-template <int N, typename F>
-TRI_DEV void static_for(F&& f) {
-  static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
 // Key tiles per wave whose V operands live in LDS instead of registers: the longest rows
 // leave the vector registers no room for all of them (the accumulators fill the other file).
 constexpr int bwd_row_v_lds_tiles(int D, int KT) { return KT * (D / 16) < 16 ? 0 : D <= 32 ? KT - 2 : 1; }

@@ -359,11 +359,12 @@ int trifast_default_tile(int kernel, int64_t n, int64_t h, int64_t d, int dtype)
   switch (kernel) {
     case TRIFAST_KERNEL_FWD:
       // pair rows that share a bias tile: one for the smallest and the widest rows; two for
-      // 128-byte rows (one in fp32) and for 64-byte 16-bit rows of fewer than 1024 keys; four
-      // above that; 32-byte rows: four, or two with 64 keys per stage from 256 keys on
+      // 128-byte rows (one in fp32) and for 64-byte 16-bit rows of fewer than 768 keys; four
+      // above that, with the scheduled loop for workgroups without masked keys; 32-byte rows:
+      // four, or two with 64 keys per stage from 256 keys on
       if (n <= 64 || row_bytes >= 256) pick = 0;
       else if (row_bytes == 128) pick = dtype == TRIFAST_F32 ? 0 : 4;
-      else if (row_bytes == 64) pick = (dtype != TRIFAST_F32 && n < 1024) ? 4 : 3;
+      else if (row_bytes == 64) pick = dtype == TRIFAST_F32 ? 3 : (n < 768 ? 4 : 7);  // (7: four rows, scheduled loop)
       else pick = n >= 256 ? 1 : 3;
       break;
     case TRIFAST_KERNEL_BWD_Q:  // 2 pair rows, 64 keys per stage; one row from 128-byte rows on

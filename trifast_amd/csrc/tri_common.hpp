@@ -17,6 +17,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
+#include <utility>
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -368,6 +370,20 @@ TRI_DEV typename Elem<T>::frag resident_ones() {
   }
   return f;
 }
+
+template <typename F, int... I>
+TRI_DEV void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in order
+template <int N, typename F>
+TRI_DEV void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// acc + the two values of a packed pair (what an MFMA that consumes the pair sees)
+TRI_DEV float pair_sum(bf16x2 w, bf16x2 ones, float acc) { return __builtin_amdgcn_fdot2_f32_bf16(w, ones, acc, false); }
+TRI_DEV float pair_sum(f16x2 w, f16x2 ones, float acc) { return __builtin_amdgcn_fdot2(w, ones, acc, false); }
 
 TRI_DEV f32x16 zero16() {
   f32x16 z;

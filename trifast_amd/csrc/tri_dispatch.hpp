@@ -30,10 +30,12 @@ hipError_t dispatch_tile(const Args& a, int bh, int tile, hipStream_t st, bool d
 template <class F, typename T, class Args>
 hipError_t dispatch_d(const Args& a, int bh, int d, int tile, hipStream_t st, bool dry) {
   switch (d) {
+#ifndef TRI_DEV_ONLY_BF16_D32  // (development builds: one instantiation family compiles in seconds)
     case 16: return dispatch_tile<F, T, 16>(a, bh, tile, st, dry);
-    case 32: return dispatch_tile<F, T, 32>(a, bh, tile, st, dry);
     case 64: return dispatch_tile<F, T, 64>(a, bh, tile, st, dry);
     case 128: return dispatch_tile<F, T, 128>(a, bh, tile, st, dry);
+#endif
+    case 32: return dispatch_tile<F, T, 32>(a, bh, tile, st, dry);
   }
   return hipErrorInvalidValue;
 }
@@ -41,9 +43,11 @@ hipError_t dispatch_d(const Args& a, int bh, int d, int tile, hipStream_t st, bo
 template <class F, class Args>
 hipError_t dispatch(const Args& a, int bh, int d, int dtype, int tile, hipStream_t st, bool dry) {
   switch (dtype) {
+#ifndef TRI_DEV_ONLY_BF16_D32
     case kF32: return dispatch_d<F, float>(a, bh, d, tile, st, dry);
-    case kBF16: return dispatch_d<F, __bf16>(a, bh, d, tile, st, dry);
     case kF16: return dispatch_d<F, _Float16>(a, bh, d, tile, st, dry);
+#endif
+    case kBF16: return dispatch_d<F, __bf16>(a, bh, d, tile, st, dry);
   }
   return hipErrorInvalidValue;
 }

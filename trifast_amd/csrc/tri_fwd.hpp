@@ -42,8 +42,26 @@ namespace tri {
 constexpr float kLazy = 8.0f;
 constexpr float kLazyLimit = 256.0f;  // 2^kLazy
 
-template <typename T, int D, int NW, int R, int BK>
-__global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd_kernel(const FwdArgs a) {
+// BKF: keys per stage of the general stage loop, plus kFwdFast when the workgroup may take
+// the scheduled loop below for rows without masked keys.
+constexpr int kFwdFast = 256;
+// LDS bytes of the two loops (without the key-tile bitmaps that follow them)
+constexpr int fwd_stage_bytes(int D, int es, int NW, int R, int BK) { return (2 * R * BK * D + NW * (BK / 32) * 1024) * es + 256; }
+// stages of the scheduled loop's ring: what is in use, what the next barrier publishes, and
+// the rest in flight (four pair rows per stage leave room for three stages at two workgroups
+// per compute unit; their loads are then issued three tiles before the barrier that needs them)
+constexpr int fwd_fast_stages(int R) { return R >= 4 ? 3 : 4; }
+constexpr int fwd_fast_stage_bytes(int D, int es, int NW, int R) { return 2 * R * 32 * D * es + NW * 2048; }
+constexpr int fwd_main_lds_bytes(int D, int es, int NW, int R, int BKF) {
+  const int gen = 2 * fwd_stage_bytes(D, es, NW, R, BKF % kFwdFast);
+  const int fast = BKF >= kFwdFast ? fwd_fast_stages(R) * fwd_fast_stage_bytes(D, es, NW, R) : 0;
+  return gen > fast ? gen : fast;
+}
+
+template <typename T, int D, int NW, int R, int BKF>
+__global__ __launch_bounds__(NW * 64, (R * ((BKF % kFwdFast) / 32) >= 8) ? 1 : 2) void tri_fwd_kernel(const FwdArgs a) {
+  constexpr int BK = BKF % kFwdFast;
+  constexpr bool FAST = BKF >= kFwdFast;
   using E = Elem<T>;
   using frag = typename E::frag;
   constexpr int KP = E::KP;
@@ -60,6 +78,8 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
   constexpr int BIAS_B = 2 * 64 * 8 * (int)sizeof(T);  // one packed 32 x 32 bias tile
   constexpr int OFF_KW = OFF_B + NW * KU * BIAS_B;  // keep words of the stage's tiles, [R][KU] (64 slots)
   constexpr int STAGE = OFF_KW + 256;
+  static_assert(STAGE == fwd_stage_bytes(D, (int)sizeof(T), NW, R, BK), "the launcher sizes LDS with fwd_stage_bytes");
+  constexpr int LDS_MAIN = fwd_main_lds_bytes(D, (int)sizeof(T), NW, R, BKF);  // the key-tile bitmaps follow
   static_assert(R * KU <= 64, "the keep words of a stage are one 64-lane load");
   extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
 
@@ -117,16 +137,10 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
   // element of this lane's key (patched in place per tile) against a constant queries
   // operand (see OffsetMask; its per-query offset is not used here: the word is zero)
   typename OffsetMask<T>::Keys kop;
-  kop.init(perm32(jl), g);
   frag qzero;
-  {
-    typename OffsetMask<T>::Queries qz;
-    qz.init(split_word<T>(0.f), g);
-    qzero = qz.get();
-  }
 
   KeyTileMasks masks;
-  masks.build<R, NW>(reinterpret_cast<uint64_t*>(tri_smem + 2 * STAGE), [&](int r) { return keep_row[r]; }, a.nwords, any_flagged, wave, lane);
+  masks.build<R, NW>(reinterpret_cast<uint64_t*>(tri_smem + LDS_MAIN), [&](int r) { return keep_row[r]; }, a.nwords, any_flagged, wave, lane);
 
   // lane-constant LDS offsets of the operand reads: K rows as natural operands
   // (tile row m stands for key perm32(m)), V rows through transposing reads
@@ -134,9 +148,17 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
   ofs.init(perm32(jl), lane);
 
   // per-lane source pointers of the K and V stage tiles for keys 0..BK-1
+  // (set up by the general stage loop only: the scheduled loop below has no use for them, and
+  // what is live across the choice between the two loops takes registers from both)
   TileStream<T, D, R * BK, NW> kstream, vstream;
-  kstream.init([&](int x) { return kbh + min(i0 + x / BK, N - 1) * a.sk.i + (int64_t)(x % BK) * a.sk.j; }, wave, lane);
-  vstream.init([&](int x) { return vbh + min(i0 + x / BK, N - 1) * a.sv.i + (int64_t)(x % BK) * a.sv.j; }, wave, lane);
+  auto setup_general = [&] {
+    kop.init(perm32(jl), g);
+    typename OffsetMask<T>::Queries qz;
+    qz.init(split_word<T>(0.f), g);
+    qzero = qz.get();
+    kstream.init([&](int x) { return kbh + min(i0 + x / BK, N - 1) * a.sk.i + (int64_t)(x % BK) * a.sk.j; }, wave, lane);
+    vstream.init([&](int x) { return vbh + min(i0 + x / BK, N - 1) * a.sv.i + (int64_t)(x % BK) * a.sv.j; }, wave, lane);
+  };
 
   // Stage loads: direct global->LDS.  A stage that lies inside the key range adds
   // one uniform offset to the precomputed pointers; the last, ragged one clamps
@@ -337,6 +359,315 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
       if (t + 1 < TS) sc = sn;
     }
   };
+  // ---- the scheduled loop: workgroups whose rows attend to every key ------------------------
+  // Same work as the plain stage loop above, laid out as the schedule it should run in.  A
+  // wave issues in order, so everything a tile needs is asked for a whole tile ahead:
+  //   * a ring of three or four 32-key stages (K rows, V rows and the waves' packed bias
+  //     tiles), filled by global->LDS loads that are issued two or three stages ahead; one barrier per stage, before
+  //     its last tile, publishes the next stage.  Every load in the loop is an asm statement
+  //     and every wait for them is a counted one written here: a load the compiler knows of
+  //     (or a register it reloads from scratch) would make it wait for everything in flight;
+  //   * in the slot of tile t the wave reads the K operand of tile t+1 and the V operand of
+  //     tile t from LDS, issues the P.V MFMAs of tile t-1 and the score MFMAs of tile t+1,
+  //     and spreads the softmax arithmetic of tile t (in units of two scores: two fma, two
+  //     exp2, a packed conversion and a row-sum step) between them;
+  //   * the bias tile of the next stage enters through the matrix pipe in the last slot of a
+  //     stage: its packed words are the B operand against a constant A operand that holds
+  //     sqrt(d) where the contraction slot is the row's key (sqrt(32) as hi + lo parts), and
+  //     the product is the accumulator init of the score MFMAs of the R rows.
+  auto fast_loop = [&]() __attribute__((always_inline)) {
+    static_assert(!FAST || (sizeof(T) == 2 && BK == 32 && R >= 2), "16-bit types, 32-key stages, two or more pair rows");
+    if constexpr (FAST) {
+    typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
+    typedef T pair_t __attribute__((ext_vector_type(2)));
+    constexpr int NS = fwd_fast_stages(R);
+    constexpr int FSTAGE = fwd_fast_stage_bytes(D, (int)sizeof(T), NW, R);
+    constexpr int FOFF_V = R * 32 * ROWB, FOFF_B = 2 * R * 32 * ROWB;
+    constexpr int G = 2 * R * 32 * Tile::CPR / 64;  // 1 KiB wave loads per stage: K rows, then V rows
+    static_assert(G % NW == 0, "every wave issues the same number of loads");
+    constexpr int XN = G / NW;
+    constexpr int NLD = XN + 2;  // loads per wave and stage: its share of K and V, its bias tile
+    auto SB = [] { __builtin_amdgcn_sched_barrier(0); };
+    const int ns = N >> 5;
+
+    // this wave's loads of a stage: a 32-bit byte offset per lane from the stage's first K / V row
+    uint32_t lofs[XN];
+#pragma unroll
+    for (int x = 0; x < XN; ++x) {
+      const int gi = x * NW + wave;
+      const bool is_k = gi < G / 2;
+      const int p = (gi % (G / 2)) * 64 + lane;
+      const int r_ = p / Tile::CPR, cc = (p % Tile::CPR) ^ Tile::swz(r_);
+      const int64_t rr = min(i0 + r_ / 32, N - 1) - i0;
+      const Str5& st = is_k ? a.sk : a.sv;
+      lofs[x] = (uint32_t)((rr * st.i + (int64_t)(r_ % 32) * st.j + cc * Tile::VEC) * (int64_t)sizeof(T));
+    }
+    const uint32_t lane16 = (uint32_t)lane * 16u;
+    const T* krow0 = kbh + (int64_t)i0 * a.sk.i;
+    const T* vrow0 = vbh + (int64_t)i0 * a.sv.i;
+    const T* bias_wave = pack_bh + (int64_t)jt_ld * a.NP * 1024;  // packed bias tiles of this wave's queries
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(TRI_L3 unsigned char*)tri_smem;
+    // (the sources move along the keys by a constant step per stage: three scalar pointers)
+    const int64_t kstep = 32 * a.sk.j, vstep = 32 * a.sv.j;
+    const T* kfill = krow0;
+    const T* vfill = vrow0;
+    const T* bfill = bias_wave;
+    int filled = 0;  // the stage the pointers stand at
+    auto issue_fast = [&](int boff) {
+#pragma unroll
+      for (int x = 0; x < XN; ++x) {
+        const int gi = x * NW + wave;
+        const T* base = gi < G / 2 ? kfill : vfill;  // wave-uniform
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)(boff + gi * 1024));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(lofs[x]), "s"(base) : "memory", "m0");
+      }
+      const uint32_t dstb = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)(boff + FOFF_B + wave * 2048));
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %1, %2 offset:1024" : : "s"(dstb), "v"(lane16), "s"(bfill) : "memory", "m0");
+      // (the second load lands 1 KiB further: the instruction offset applies to both addresses)
+      // past the last stage the pointers stay: a valid stage is fetched again, which nobody uses
+      const bool more = filled + 1 < ns;
+      kfill += more ? kstep : 0;
+      vfill += more ? vstep : 0;
+      bfill += more ? 1024 : 0;
+      filled += 1;
+    };
+    // A operand of the bias products: row m of the score tile stands for key perm32(m); half r2
+    // of the packed words gives the contraction slots 8 g + e the keys 16 r2 + 8 g + e
+    constexpr int NPART = D == 32 ? 2 : 1;
+    constexpr int NB = 2 * NPART;
+    frag bsel[2][NPART];
+    {
+      const T hi = (T)a.sqrt_d;
+      const T part[2] = {hi, (T)(a.sqrt_d - (float)hi)};
+#pragma unroll
+      for (int r2 = 0; r2 < 2; ++r2)
+#pragma unroll
+        for (int pp = 0; pp < NPART; ++pp) {
+          const int e = perm32(jl) - 16 * r2 - 8 * g;
+          const uint32_t bits = (uint32_t)__builtin_bit_cast(uint16_t, part[pp]) << (16 * (e & 1));
+          u32x4v w;
+#pragma unroll
+          for (int x = 0; x < 4; ++x) w[x] = (e >= 0 && e < 8 && (e >> 1) == x) ? bits : 0u;
+          asm volatile("" : "+v"(w));  // resident: not rebuilt from the lane id at every use
+          bsel[r2][pp] = __builtin_bit_cast(frag, w);
+        }
+    }
+    const pair_t ones = {(T)1.0f, (T)1.0f};
+
+    // absolute LDS addresses of this lane's operand reads in the stage in use (K rows as natural
+    // operands, V rows through transposing reads, the wave's bias words); they move with the ring
+    uint32_t ak[DS], avl[DM], avh[DM], ab;
+#pragma unroll
+    for (int sd = 0; sd < DS; ++sd) ak[sd] = lds0 + (uint32_t)ofs.nat[sd];
+#pragma unroll
+    for (int mt = 0; mt < DM; ++mt) {
+      avl[mt] = lds0 + (uint32_t)(FOFF_V + ofs.tlo[mt]);
+      avh[mt] = lds0 + (uint32_t)(FOFF_V + ofs.thi[mt]);
+    }
+    ab = lds0 + (uint32_t)(FOFF_B + wave * 2048) + lane16;
+    auto lds_frag = [](uint32_t addr) { return *reinterpret_cast<TRI_L3 const frag*>((uintptr_t)addr); };
+    auto lds_tr = [](uint32_t lo, uint32_t hi) {
+      const auto x = lds_tr4(reinterpret_cast<TRI_L3 const T*>((uintptr_t)lo));
+      const auto y = lds_tr4(reinterpret_cast<TRI_L3 const T*>((uintptr_t)hi));
+      frag f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { f[e] = x[e]; f[4 + e] = y[e]; }
+      return f;
+    };
+
+    // ---- the state that moves from slot to slot ----
+    f32x16 sc_cur = zero16(), bias_s = zero16();
+    frag vf_prev[DM][PS], pf_prev[PS];
+#pragma unroll
+    for (int s2 = 0; s2 < PS; ++s2) {
+      pf_prev[s2] = E::zero();
+#pragma unroll
+      for (int mt = 0; mt < DM; ++mt) vf_prev[mt][s2] = E::zero();
+    }
+
+    // ---- prologue: the first stages on their way, bias tile and scores of the first tile ----
+#pragma unroll
+    for (int st = 0; st < NS - 1; ++st) issue_fast(st * FSTAGE);
+    // (a wait the compiler knows: the loads made before the loop, the Q operands among them, no
+    // longer count as in flight, or it would wait for everything again where the loop first
+    // uses them, in every trip)
+    wait_dma_known();
+    ring_sync<0>();
+    if (wave_active) {
+#pragma unroll
+      for (int x = 0; x < NB; ++x)
+        bias_s = E::mfma(bsel[x / NPART][x % NPART], lds_frag(ab + (x / NPART) * 1024), bias_s);
+      sc_cur = bias_s;
+#pragma unroll
+      for (int sd = 0; sd < DS; ++sd) sc_cur = E::mfma(lds_frag(ak[sd]), qf[0][sd], sc_cur);
+    }
+
+    enum { F_B, F_PV, F_S };
+    // (the loop exists twice: for waves with queries, and for the waves past the end of the pair
+    // row, which only take part in the loads and barriers; one loop with the test inside would
+    // make the compiler copy the state where the two cases meet)
+    auto stage_loop_fast = [&](auto active_c) __attribute__((always_inline)) {
+    constexpr bool ACTIVE = decltype(active_c)::value;
+    // offsets of the ring: the stage in use, the one after it, the one the next loads go to
+    int boff = 0;
+    for (int stage = 0; stage < ns; ++stage) {
+      const int boff_next = boff == (NS - 1) * FSTAGE ? 0 : boff + FSTAGE;
+      const int boff_fill = boff == 0 ? (NS - 1) * FSTAGE : boff - FSTAGE;  // stage + NS - 1
+      const int step_next = boff_next - boff;
+      static_for<R>([&](auto r_c) __attribute__((always_inline)) {
+        constexpr int r = decltype(r_c)::value;
+        constexpr bool last_r = r == R - 1;
+        constexpr int rn = (r + 1) % R, rp = (r + R - 1) % R;
+        constexpr int NPV = PS * DM;
+        constexpr int NM = DS + NPV + (last_r ? NB : 0);
+        constexpr int NU = 8;
+        // MFMA order: the P.V products of the last tile, (the bias products,) the score products
+        struct Order { int kind[NM], idx[NM]; };
+        constexpr Order ord = [] {
+          Order o{};
+          int n = 0;
+          for (int i = 0; i < NPV; ++i) { o.kind[n] = F_PV; o.idx[n++] = i; }
+          if (last_r) for (int i = 0; i < NB; ++i) { o.kind[n] = F_B; o.idx[n++] = i; }
+          for (int i = 0; i < DS; ++i) { o.kind[n] = F_S; o.idx[n++] = i; }
+          return o;
+        }();
+        if constexpr (ACTIVE) {
+          SB();
+          // operand reads: K rows of the next tile, V rows of this one, (the next stage's bias words)
+          const uint32_t knext = last_r ? (uint32_t)step_next : (uint32_t)(rn * 32 * ROWB);
+          frag kf[DS], vf[DM][PS], bwf[2];
+#pragma unroll
+          for (int sd = 0; sd < DS; ++sd) kf[sd] = lds_frag(ak[sd] + knext);
+#pragma unroll
+          for (int mt = 0; mt < DM; ++mt)
+#pragma unroll
+            for (int s2 = 0; s2 < PS; ++s2)
+              vf[mt][s2] = lds_tr(avl[mt] + (uint32_t)(r * 32 * ROWB + 16 * s2 * ROWB), avh[mt] + (uint32_t)(r * 32 * ROWB + 16 * s2 * ROWB));
+          if constexpr (last_r) {
+            bwf[0] = lds_frag(ab + (uint32_t)step_next);
+            bwf[1] = lds_frag(ab + (uint32_t)step_next + 1024u);
+          }
+          SB();
+          f32x16 sc_next, bias_next = zero16();
+          uint32_t pw[NU];
+          const float mcr = mc[r], l_old = lrun[r];
+          float l_new = l_old;  // the running row sum with this tile's probabilities on top
+          // The arithmetic of a unit is a chain (fma -> exp2 -> conversion -> row sum), and a wave
+          // that issues a dependent instruction right behind its producer waits for it: the
+          // chain is cut into three steps that run one piece apart, so that between two MFMAs
+          // the wave converts the units of the piece before, exponentiates its own and scales
+          // those of the next.
+          float xs[2 * NU], ps[2 * NU];
+          auto scale_unit = [&](int u) __attribute__((always_inline)) {
+            xs[2 * u] = __builtin_fmaf(sc_cur[2 * u], c, -mcr);
+            xs[2 * u + 1] = __builtin_fmaf(sc_cur[2 * u + 1], c, -mcr);
+          };
+          auto exp_unit = [&](int u) __attribute__((always_inline)) {
+            ps[2 * u] = fast_exp2(xs[2 * u]);
+            ps[2 * u + 1] = fast_exp2(xs[2 * u + 1]);
+          };
+          auto pack_unit = [&](int u) __attribute__((always_inline)) {
+            const pair_t w = {(T)ps[2 * u], (T)ps[2 * u + 1]};
+            pw[u] = __builtin_bit_cast(uint32_t, w);
+            l_new = pair_sum(w, ones, l_new);
+          };
+#pragma unroll
+          for (int u = 0; u < NU / NM; ++u) scale_unit(u);
+          SB();
+          static_for<NM>([&](auto xc) __attribute__((always_inline)) {
+            constexpr int x = decltype(xc)::value;
+            constexpr int kind = ord.kind[x], idx = ord.idx[x];
+            if constexpr (kind == F_B) {
+              bias_next = E::mfma(bsel[idx / NPART][idx % NPART], bwf[idx / NPART], bias_next);
+            } else if constexpr (kind == F_PV) {
+              constexpr int s2 = idx / DM, mt = idx % DM;
+              oacc[rp][mt] = E::mfma(vf_prev[mt][s2], pf_prev[s2], oacc[rp][mt]);
+            } else {
+              if constexpr (idx == 0) sc_next = E::mfma(kf[0], qf[rn][0], last_r ? bias_next : bias_s);
+              else sc_next = E::mfma(kf[idx], qf[rn][idx], sc_next);
+            }
+            SB();
+            if constexpr (x > 0) {
+#pragma unroll
+              for (int u = (x - 1) * NU / NM; u < x * NU / NM; ++u) pack_unit(u);
+            }
+#pragma unroll
+            for (int u = x * NU / NM; u < (x + 1) * NU / NM; ++u) exp_unit(u);
+            if constexpr (x + 1 < NM) {
+#pragma unroll
+              for (int u = (x + 1) * NU / NM; u < (x + 2) * NU / NM; ++u) scale_unit(u);
+            } else {
+#pragma unroll
+              for (int u = x * NU / NM; u < (x + 1) * NU / NM; ++u) pack_unit(u);
+            }
+            SB();
+          });
+          if (__any(!(l_new - l_old <= kLazyLimit))) {
+            // some query outgrew the reference: raise it to the running maximum and redo the tile
+            // (the reference lives in the log2 domain only: mc = c * max)
+            asm volatile("" ::);
+            float mx = fmaxf(sc_cur[0], sc_cur[1]);
+#pragma unroll
+            for (int v = 2; v < 16; ++v) mx = fmaxf(mx, sc_cur[v]);
+            mx = half_max(mx);
+            const float mcn = fmaxf(mc[r], mx * c);
+            const float alpha = fast_exp2(mc[r] - mcn);
+#pragma unroll
+            for (int mt = 0; mt < DM; ++mt)
+#pragma unroll
+              for (int v = 0; v < 16; ++v) oacc[r][mt][v] *= alpha;
+            mc[r] = mcn;
+            l_new = l_old * alpha;
+#pragma unroll
+            for (int u = 0; u < NU; ++u) {
+              const float p0 = fast_exp2(__builtin_fmaf(sc_cur[2 * u], c, -mcn));
+              const float p1 = fast_exp2(__builtin_fmaf(sc_cur[2 * u + 1], c, -mcn));
+              const pair_t w = {(T)p0, (T)p1};
+              pw[u] = __builtin_bit_cast(uint32_t, w);
+              l_new = pair_sum(w, ones, l_new);
+            }
+          }
+          lrun[r] = l_new;
+#pragma unroll
+          for (int s2 = 0; s2 < PS; ++s2) {
+            pf_prev[s2] = __builtin_bit_cast(frag, (u32x4v){pw[4 * s2], pw[4 * s2 + 1], pw[4 * s2 + 2], pw[4 * s2 + 3]});
+#pragma unroll
+            for (int mt = 0; mt < DM; ++mt) vf_prev[mt][s2] = vf[mt][s2];
+          }
+          sc_cur = sc_next;
+          if constexpr (last_r) bias_s = bias_next;
+        }
+        // The next slot reads stage s+1: every wave's loads of it have landed (a ring of four
+        // leaves one younger stage in flight), and nobody reads stage s-1 any more: the buffer
+        // that the loads issued in the next slot overwrite.
+        if constexpr (r == R - 2) ring_sync<(NS - 3) * NLD>();
+        if constexpr (last_r) issue_fast(boff_fill);
+      });
+      // the ring moves on
+#pragma unroll
+      for (int sd = 0; sd < DS; ++sd) ak[sd] += (uint32_t)step_next;
+#pragma unroll
+      for (int mt = 0; mt < DM; ++mt) {
+        avl[mt] += (uint32_t)step_next;
+        avh[mt] += (uint32_t)step_next;
+      }
+      ab += (uint32_t)step_next;
+      boff = boff_next;
+    }
+    };
+    if (wave_active) stage_loop_fast(std::true_type{});
+    else stage_loop_fast(std::false_type{});
+    // P.V of the last tile
+    if (wave_active) {
+#pragma unroll
+      for (int s2 = 0; s2 < PS; ++s2)
+#pragma unroll
+        for (int mt = 0; mt < DM; ++mt) oacc[R - 1][mt] = E::mfma(vf_prev[mt][s2], pf_prev[s2], oacc[R - 1][mt]);
+    }
+    wait_dma();  // (the last prefetches are still on their way into LDS)
+    }
+  };
+
   // Stage loop over the live stages, unrolled by two for the two LDS buffers.  A
   // workgroup whose rows attend to every key runs the loop specialised for plain
   // stages; any other one runs the general loop for all of its stages (mixing the
@@ -367,9 +698,22 @@ __global__ __launch_bounds__(NW * 64, (R * (BK / 32) >= 8) ? 1 : 2) void tri_fwd
     }
   };
   // (a last stage with fewer than KU key tiles is not plain: its missing tiles are masked)
-  if (masks.all_plain() && ntiles % KU == 0) stage_loop(std::integral_constant<int, kPlain>{});
-  else if (!any_flagged) stage_loop(std::integral_constant<int, kMasked>{});
-  else stage_loop(std::integral_constant<int, kGeneral>{});
+  bool fast = false;
+  if constexpr (FAST) {
+    // (the per-lane offsets of the stage loads are 32-bit: rows and keys of a stage must lie within 4 GiB)
+    const auto fits = [&](const Str5& st) {
+      return st.i >= 0 && st.j >= 0 && (uint64_t)(R - 1) * st.i + 31ull * st.j + D < (1ull << 31) / sizeof(T);
+    };
+    fast = masks.all_plain() && (N & 31) == 0 && fits(a.sk) && fits(a.sv);
+  }
+  if (fast) {
+    if constexpr (FAST) fast_loop();
+  } else {
+    setup_general();
+    if (masks.all_plain() && ntiles % KU == 0) stage_loop(std::integral_constant<int, kPlain>{});
+    else if (!any_flagged) stage_loop(std::integral_constant<int, kMasked>{});
+    else stage_loop(std::integral_constant<int, kGeneral>{});
+  }
 
   if (!wave_active) return;
 #pragma unroll
