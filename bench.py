@@ -184,6 +184,54 @@ def kernel_breakdown(q, k, v, bias, mask, do, reps):
     return out
 
 
+def other_workloads(names, warmup: int = 5, steps: int = 10):
+    """fwd+bwd step and forward of the other configurations, in the same run as the headline
+    one: ``warmup`` untimed steps, then ``steps`` timed ones between synchronisations, with the
+    library's default tiles (nothing is tuned here, so the figures do not depend on a cache)."""
+    import trifast_amd
+
+    out = {}
+    saved = os.environ.get("TRIFAST_AUTOTUNE")
+    os.environ["TRIFAST_AUTOTUNE"] = "0"
+    try:
+        for name in names:
+            dtype, b, n, h, d, _ = WORKLOADS[name]
+            q, k, v, bias, mask, do = make_workload(name, "cuda:0")
+            q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True), bias.requires_grad_(True)
+
+            def step():
+                trifast_amd.triangle_attention(q, k, v, bias, mask).backward(do)
+                q.grad = k.grad = v.grad = bias.grad = None
+
+            def fwd_only():
+                with torch.no_grad():
+                    trifast_amd.triangle_attention(q, k, v, bias, mask)
+
+            for _ in range(warmup):
+                step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                step()
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) * 1e3 / steps
+            fwd_only()
+            torch.cuda.synchronize()
+            ms_fwd = _event_ms(fwd_only, steps)
+            f_fwd, f_bwd = flops(b, h, n, d)
+            peak = PEAK_F32_TFLOPS if dtype == torch.float32 else PEAK_BF16_TFLOPS
+            out[name] = {"ms_per_step": round(ms, 4), "frac_of_peak": round((f_fwd + f_bwd) / ms / 1e9 / peak, 4),
+                         "fwd_ms": round(ms_fwd, 4), "fwd_frac_of_peak": round(f_fwd / ms_fwd / 1e9 / peak, 4)}
+            del q, k, v, bias, mask, do
+            torch.cuda.empty_cache()
+    finally:
+        if saved is None:
+            os.environ.pop("TRIFAST_AUTOTUNE", None)
+        else:
+            os.environ["TRIFAST_AUTOTUNE"] = saved
+    return out
+
+
 def _cpu_model() -> str:
     try:
         with open("/proc/cpuinfo") as f:
@@ -275,6 +323,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="M", choices=[w for w in WORKLOADS if w != "C1"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the short fwd+bwd timings of the other configurations that the default run adds")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 256 MiB device copy, the known-size kernel that "
@@ -402,6 +452,12 @@ def main():
         "roofline": roofline,
         "autotune": tuner.autotune_enabled(),
     }
+    if args.workload == "M" and not args.no_other_workloads:
+        del q, k, v, bias, mask, do
+        torch.cuda.empty_cache()
+        line["workloads"] = other_workloads(["C2", "C3", "C4a", "C4b", "C5", "F32"])
+        line["workloads_note"] = "fwd+bwd steps of the other configurations in this run: 5 warm-up + 10 timed steps each, library default tiles"
+        q, k, v, bias, mask, do = make_workload(args.workload, dev)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args.workload, (q, k, v, bias, mask, do), args.cpu_budget)
     print(json.dumps(line))

@@ -231,3 +231,26 @@ def test_equiv_module_matches_the_oracle():
     q, k, v, b = (t.detach() for t in (q, k, v, b))
     torch.testing.assert_close(attention_reference(q, k, v, b, m), orc.attention_reference(q, k, v, b, m), rtol=1e-6, atol=1e-6)
     torch.testing.assert_close(triangle_attention_simple(q, k, v, b, m), orc.triangle_attention_simple(q, k, v, b, m), rtol=1e-6, atol=1e-6)
+
+
+def test_wide_j_strides_are_copied_and_their_gradients_allocated_contiguous():
+    # the kernels address the rows of a tile through 32-bit offsets: a stride between
+    # consecutive j of 2^24 bytes or more is not run in place (the library would refuse it)
+    t = torch.empty_strided((1, 1, 2, 2, 8), (0, 0, 64, 1 << 24, 1), dtype=torch.bfloat16, device="meta")
+    assert tt._vector_ready(t).is_contiguous()
+    assert tt._grad_like(t).is_contiguous()
+    ok = torch.empty_strided((1, 1, 2, 2, 8), (0, 0, 8, 16, 1), dtype=torch.bfloat16, device="meta")  # transposed view
+    assert tt._vector_ready(ok) is ok
+
+
+def test_equiv_simple_takes_any_number_of_batch_dims():
+    from trifast_amd import equiv
+
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(2, 3, 2, 5, 5, 4, generator=g) for _ in range(3))
+    b = torch.randn(2, 3, 2, 5, 5, generator=g)
+    m = torch.rand(2, 3, 5, 5, generator=g) < 0.3
+    whole = equiv.triangle_attention_simple(q, k, v, b, m)
+    parts = torch.stack([equiv.attention_reference(q[x], k[x], v[x], b[x], m[x]) for x in range(2)])
+    assert torch.allclose(whole, parts, atol=1e-6)
+    assert torch.allclose(equiv.triangle_attention_simple(q[0, 0], k[0, 0], v[0, 0], b[0, 0], m[0, 0]), whole[0, 0], atol=1e-6)

@@ -60,6 +60,34 @@ def check_all(kernel, pt, ref, dtype, tag, directions=True):
     print(f"{tag}: " + " ".join(report))
 
 
+# the second output of the operator: log-sum-exp of the logits (natural log, fp32).  The
+# kernel sums the probabilities it feeds to the second product, i.e. rounded to the input
+# dtype, so in 16-bit dtypes lse carries up to half an ulp of that dtype in relative error
+# of the sum: 2^-9 (bf16), 2^-12 (fp16); the bounds below are twice that.  A row whose keys
+# are all masked reports finfo(dtype).min + ln n (reference src/trifast/triton.py:104-109,130-132).
+LSE_ABS_TOL = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -10}
+
+
+def check_lse(low, m, dtype, tag):
+    with torch.no_grad():
+        _, lse = tt._triangle_attention(*low, m)
+    n = m.shape[-1]
+    ref = orc.lse_reference(low[0].float(), low[1].float(), low[3].float(), m)
+    full = m.all(dim=-1)[:, None, :, None].expand_as(lse)  # rows whose keys are all masked
+    assert torch.isfinite(lse).all(), f"{tag} lse: non-finite values"
+    if (~full).any():
+        err = (lse - ref)[~full].abs().max().item()
+        if dtype == torch.float32:
+            bound = 1e-5 * max(ref[~full].abs().max().item(), 1.0)
+        else:
+            bound = LSE_ABS_TOL[dtype]
+        assert err <= bound, f"{tag} lse: max error {err:.3e} > {bound:.3e}"
+    if full.any():
+        want = torch.tensor(torch.finfo(dtype).min, dtype=torch.float32) + float(np.log(n))
+        got = lse[full]
+        assert torch.allclose(got, want.to(got.device).expand_as(got), rtol=1e-6, atol=0), f"{tag} lse of fully masked rows: {got.flatten()[:4].tolist()} != {want.item()}"
+
+
 # ---------------------------------------------------------------------------
 # the reference's own test grid (tests/unit/test_trifast.py:26-38), thinned over n
 # unless TRIFAST_FULL_GRID=1
@@ -84,7 +112,9 @@ def test_values_and_vectors(n, h, d, mask, bs, dtype, std):
     do = torch.ones((), device=DEV, dtype=dtype).expand(q.shape)
     pt = orc.forward_backward(*low, m, do)
     kern = kernel_fwd_bwd(*low, m, do)
-    check_all(kern, pt, ref, dtype, f"n={n} h={h} d={d} bs={bs} std={std} mask={mask} {dtype}")
+    tag = f"n={n} h={h} d={d} bs={bs} std={std} mask={mask} {dtype}"
+    check_all(kern, pt, ref, dtype, tag)
+    check_lse(low, m, dtype, tag)
 
 
 # ---------------------------------------------------------------------------

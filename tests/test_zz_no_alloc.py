@@ -69,6 +69,49 @@ def test_static_forward_matches_workspace_forward_twice():
     assert torch.equal(o_s, o_w) and torch.equal(lse_s, lse_w)
 
 
+def test_static_forward_takes_no_device_memory_and_runs_under_capture():
+    """After one warm-up call (the first call on a device looks up the array's address and
+    may raise a kernel's LDS limit: both happen outside a capture), a call changes the
+    device's free memory by nothing, and the entry point can be recorded into a HIP graph
+    and replayed, with the bits of ``trifast_fwd``."""
+    lib = _lib.load()
+    q, k, v, bias, mask = _inputs(1, 2, 256, 32, torch.bfloat16, 7, 0.2)
+    b, h, n, _, d = q.shape
+    code = tt._DTYPE_CODE[q.dtype]
+    mu8 = mask.view(torch.uint8)
+    S = lambda t: _lib.i64_array(tt._strides(t))
+    o = torch.empty((b, h, n, n, d), dtype=q.dtype, device=DEV)
+    lse = torch.empty((b, h, n, n), dtype=torch.float32, device=DEV)
+
+    def call(stream):
+        return lib.trifast_fwd_static(o.data_ptr(), lse.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), bias.data_ptr(), mu8.data_ptr(),
+                                      b, h, n, d, code, S(q), S(k), S(v), S(bias), S(mu8), -1, stream)
+
+    assert call(torch.cuda.current_stream().cuda_stream) == 0, _lib.last_error()  # warm-up
+    torch.cuda.synchronize()
+    # the driver's own count of free bytes sees any allocation, the library's included
+    free_before = torch.cuda.mem_get_info()[0]
+    assert call(torch.cuda.current_stream().cuda_stream) == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    _, o_w, lse_w = _call(False, q, k, v, bias, mask)
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            assert call(side.cuda_stream) == 0, _lib.last_error()
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        o.fill_(float("nan"))
+        lse.fill_(float("nan"))
+        torch.cuda.synchronize()  # (eager work and a synchronisation between the replays)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(o, o_w) and torch.equal(lse, lse_w), f"replay {rep} differs from trifast_fwd"
+
+
 def test_static_forward_rejects_what_does_not_fit():
     lib = _lib.load()
     # bf16 b=1 h=8 n=1024 needs 16 MiB of packed bias: more than the static array

@@ -71,14 +71,16 @@ hipError_t bwd_row_run_multi(const BwdArgs& a, int bh, hipStream_t st, bool dry)
 template <typename T, int D>
 hipError_t bwd_row_dispatch_kt(const BwdArgs& a, int bh, int tile, hipStream_t st, bool dry) {
   switch (tile) {
+#ifndef TRI_DEV_ONLY_BF16_D32
     case 0: return bwd_row_run<T, D, kRowKT[0]>(a, bh, st, dry);
     case 1: return bwd_row_run<T, D, kRowKT[1]>(a, bh, st, dry);
     case 2: return bwd_row_run<T, D, kRowKT[2]>(a, bh, st, dry);
     case 3: return bwd_row_run<T, D, kRowKT[3]>(a, bh, st, dry);
     case 4: return bwd_row_run<T, D, kRowKT[4]>(a, bh, st, dry);
     case 5: return bwd_row_run<T, D, kRowKT[5]>(a, bh, st, dry);
-    case 6: return bwd_row_run<T, D, kRowKT[6]>(a, bh, st, dry);
     case 7: return bwd_row_run_multi<T, D>(a, bh, st, dry);
+#endif
+    case 6: return bwd_row_run<T, D, kRowKT[6]>(a, bh, st, dry);
   }
   return hipErrorInvalidValue;
 }
@@ -86,9 +88,11 @@ hipError_t bwd_row_dispatch_kt(const BwdArgs& a, int bh, int tile, hipStream_t s
 template <typename T>
 hipError_t bwd_row_dispatch_d(const BwdArgs& a, int bh, int d, int tile, hipStream_t st, bool dry) {
   switch (d) {
+#ifndef TRI_DEV_ONLY_BF16_D32  // (development builds: one instantiation compiles in seconds)
     case 16: return bwd_row_dispatch_kt<T, 16>(a, bh, tile, st, dry);
-    case 32: return bwd_row_dispatch_kt<T, 32>(a, bh, tile, st, dry);
     case 64: return bwd_row_dispatch_kt<T, 64>(a, bh, tile, st, dry);
+#endif
+    case 32: return bwd_row_dispatch_kt<T, 32>(a, bh, tile, st, dry);
   }
   return hipErrorInvalidConfiguration;  // wider rows do not fit the register file
 }

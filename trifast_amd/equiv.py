@@ -19,12 +19,13 @@ def neg_inf(dtype: torch.dtype) -> float:
 def triangle_attention_simple(q, k, v, bias, mask):
     """einsum formulation with a filled mask (reference src/trifast/equiv.py:16-39).
 
-    q, k, v: [b, h, n, n, d]; bias: [b, h, n, n]; mask: [b, n, n] bool, True = masked out.
+    q, k, v: [..., h, n, n, d]; bias: [..., h, n, n]; mask: [..., n, n] bool, True = masked
+    out; any number of leading batch dims, as in the reference.
     """
     scale = q.shape[-1] ** -0.5
-    logits = torch.einsum("bhijd,bhikd->bhijk", q * scale, k) + bias[:, :, None]
-    logits = logits.masked_fill(mask[:, None, :, None, :], neg_inf(q.dtype))
-    return torch.einsum("bhijk,bhikd->bhijd", logits.softmax(dim=-1), v)
+    logits = torch.einsum("...hijd,...hikd->...hijk", q * scale, k) + bias[..., None, :, :]
+    logits = logits.masked_fill(mask[..., None, :, None, :], neg_inf(q.dtype))
+    return torch.einsum("...hijk,...hikd->...hijd", logits.softmax(dim=-1), v)
 
 
 def attention_reference(q, k, v, bias, mask):

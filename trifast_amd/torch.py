@@ -62,9 +62,16 @@ def _vector_ready(t: torch.Tensor) -> torch.Tensor:
     (src/trifast/torch.py:30-34)."""
     vec = 16 // t.element_size()
     st = _strides(t)
-    if st[-1] == 1 and t.data_ptr() % 16 == 0 and all(s % vec == 0 for s in st[:-1]):
+    if st[-1] == 1 and t.data_ptr() % 16 == 0 and all(s % vec == 0 for s in st[:-1]) and _j_stride_ok(t, st):
         return t
     return t.contiguous()
+
+
+def _j_stride_ok(t: torch.Tensor, st: list[int]) -> bool:
+    """The kernels address the rows of a tile through 32-bit offsets from a per-tile base:
+    the stride between consecutive j, in bytes, must lie in [0, 2^24) (the library returns
+    TRIFAST_EUNSUPPORTED otherwise)."""
+    return t.dim() != 5 or 0 <= st[3] * t.element_size() < (1 << 24)
 
 
 def _broadcast_rows(t: torch.Tensor) -> torch.Tensor:
@@ -86,7 +93,7 @@ def _grad_like(t: torch.Tensor) -> torch.Tensor:
     contiguous otherwise."""
     vec = 16 // t.element_size()
     st = _strides(t)
-    if t.dim() == 5 and st[-1] == 1 and all(s % vec == 0 for s in st[:-1]):
+    if t.dim() == 5 and st[-1] == 1 and all(s % vec == 0 for s in st[:-1]) and _j_stride_ok(t, st):
         out = torch.empty_like(t)  # preserves the strides of a dense tensor
         if out.stride() == t.stride():
             return out
@@ -99,6 +106,27 @@ def _grad_like(t: torch.Tensor) -> torch.Tensor:
 
 def _workspace(nbytes: int, device) -> torch.Tensor:
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+# What a call needs besides the pointers, per (operator, shapes and strides of its tensors):
+# the stride arrays the C ABI takes and the workspace size.  At small sizes a step is bound
+# by the host (n = 256: 0.13 ms of kernels), and marshalling ten stride arrays and asking
+# the library for sizes on every call is a good part of that.
+_PLANS: dict = {}
+_MAX_PLANS = 256
+
+
+def _plan(kind: str, tensors, bs: int, h: int, n: int, d: int, code: int):
+    key = (kind, code, tuple((t.shape, t.stride()) for t in tensors))
+    plan = _PLANS.get(key)
+    if plan is None:
+        lib = _lib.load()
+        size = lib.trifast_fwd_workspace_bytes if kind == "fwd" else lib.trifast_bwd_workspace_bytes
+        plan = ([_lib.i64_array(_strides(t)) for t in tensors], size(bs, h, n, d, code))
+        if len(_PLANS) >= _MAX_PLANS:
+            _PLANS.clear()
+        _PLANS[key] = plan
+    return plan
 
 
 def _ptr(t):
@@ -125,16 +153,14 @@ def _triangle_attention(
     mask_u8 = mask.view(torch.uint8)
 
     with torch.cuda.device(q.device):
-        ws_bytes = lib.trifast_fwd_workspace_bytes(bs, h, n, d, code)
+        strides, ws_bytes = _plan("fwd", (q, k, v, b, mask_u8), bs, h, n, d, code)
         ws = _workspace(ws_bytes, q.device)
         stream = torch.cuda.current_stream(q.device).cuda_stream
 
         def launch(tile: int) -> None:
             rc = lib.trifast_fwd(
                 _ptr(o), _ptr(lse), _ptr(q), _ptr(k), _ptr(v), _ptr(b), _ptr(mask_u8),
-                bs, h, n, d, code,
-                _lib.i64_array(_strides(q)), _lib.i64_array(_strides(k)), _lib.i64_array(_strides(v)),
-                _lib.i64_array(_strides(b)), _lib.i64_array(_strides(mask_u8)),
+                bs, h, n, d, code, *strides,
                 tile, _ptr(ws), ws.numel(), stream,
             )
             _lib.check(rc, "trifast_fwd")
@@ -184,12 +210,9 @@ def triangle_attention_bwd(
     # caller's tensors, not of a vector-ready copy)
     dq, dk, dv, db = _grad_like(q_in), _grad_like(k_in), _grad_like(v_in), _grad_like(b)
     with torch.cuda.device(q.device):
-        ws_bytes = lib.trifast_bwd_workspace_bytes(bs, h, n, d, code)
+        strides, ws_bytes = _plan("bwd", (do, q, k, v, b, mask_u8, dq, dk, dv, db), bs, h, n, d, code)
         ws = _workspace(ws_bytes, q.device)
         stream = torch.cuda.current_stream(q.device).cuda_stream
-        strides = [
-            _lib.i64_array(_strides(t)) for t in (do, q, k, v, b, mask_u8, dq, dk, dv, db)
-        ]
 
         def launch_one(kernel: int, tile: int) -> None:
             rc = lib.trifast_bwd_one(
@@ -267,6 +290,40 @@ def setup_context(ctx, inputs, output) -> None:
 _triangle_attention.register_autograd(backwards, setup_context=setup_context)
 
 
+class _EagerTriangleAttention(torch.autograd.Function):
+    """The two operators glued by a plain autograd function: what ``triangle_attention``
+    runs in ordinary eager mode on plain tensors.  Same kernels, same saved tensors, same
+    gradients as the registered operators; it only skips the dispatcher passes of a Python
+    custom operator (forward, autograd wrapper and backward operator: about 50 us of host time
+    per step, which at n = 256 is a third of what the kernels take)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, b, mask):
+        o, l = _triangle_attention._init_fn(q, k, v, b, mask)
+        ctx.save_for_backward(q, k, v, b, mask, o, l)
+        ctx.set_materialize_grads(False)
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, b, mask, o, l = ctx.saved_tensors
+        if do is None:
+            return None, None, None, None, None
+        dq, dk, dv, db, _ = triangle_attention_bwd._init_fn(do, q, k, v, b, o, l, mask)
+        return dq, dk, dv, db, None
+
+
+def _plain_eager(*tensors) -> bool:
+    """Ordinary eager execution on plain tensors: no compilation or tracing, no function
+    transforms, no autocast, no tensor subclasses or dispatch modes; everything else goes
+    through the registered operators."""
+    if torch.compiler.is_compiling() or torch.is_autocast_enabled() or torch._C._are_functorch_transforms_active():
+        return False
+    if torch._C._dispatch_tls_local_include_set().has(torch._C.DispatchKey.Python) or torch._C._len_torch_dispatch_stack() > 0:
+        return False
+    return all(type(t) is torch.Tensor for t in tensors)
+
+
 def triangle_attention(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -286,6 +343,8 @@ def triangle_attention(
     where the layout allows it) and restored on the output.
     """
     if q.dim() == 5:
+        if _plain_eager(q, k, v, b, mask):
+            return _EagerTriangleAttention.apply(q, k, v, b, mask)
         o, _ = _triangle_attention(q, k, v, b, mask)
         return o
     if q.dim() < 4:

@@ -138,6 +138,7 @@ class TileCache:
 
 
 _caches: dict[int, TileCache] = {}
+_defaults: dict[tuple, int] = {}  # (kernel, n, h, d, dtype code) -> the library's heuristic pick
 
 
 def _cache_for(kernel: int) -> TileCache:
@@ -149,6 +150,7 @@ def _cache_for(kernel: int) -> TileCache:
 def reset() -> None:
     """Forget every in-memory cache (the files stay); used by tests."""
     _caches.clear()
+    _defaults.clear()
 
 
 def supported_tiles(kernel: int, n: int, h: int, d: int, dtype: torch.dtype) -> list[int]:
@@ -186,8 +188,13 @@ def pick(kernel: int, n: int, h: int, d: int, dtype: torch.dtype, launch: Callab
     code = _DTYPE_CODE[dtype]
 
     def default() -> int:
-        tile = lib.trifast_default_tile(kernel, n, h, d, code)
-        _lib.check(min(tile, 0), "trifast_default_tile")
+        # (remembered per shape: at small sizes a step is bound by the host)
+        dkey = (kernel, n, h, d, code)
+        tile = _defaults.get(dkey)
+        if tile is None:
+            tile = lib.trifast_default_tile(kernel, n, h, d, code)
+            _lib.check(min(tile, 0), "trifast_default_tile")
+            _defaults[dkey] = tile
         return tile
 
     if not autotune_enabled() and not force_tune():
