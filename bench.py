@@ -37,9 +37,8 @@ PEAK_HBM_GBS = 8000.0
 # as roofline.traffic when the benchmark runs that workload with that tile (keyed by the
 # tile's index in the library's table of the kernel).
 MEASURED_TRAFFIC_MIB = {
-    ("M", "_fwd", 3): 1516.5,
-    ("M", "_bwd_q", 1): 2337.3,
-    ("M", "_bwd_kv", 10): 2676.7,
+    ("M", "_fwd", 7): 1528.3,
+    ("M", "_bwd_kv", 10): 2688.9,
     ("M", "_bwd_b", 4): 1586.0,
 }
 
