@@ -42,6 +42,27 @@ PER_SOURCE_FLAGS = {
 }
 
 
+# The row-resident backward issues some of its MFMAs from asm statements with hand-placed wait
+# states (csrc/tri_common.hpp: mfma_acc).  That schedule was validated, by the parity and
+# bit-equality tests of the row-resident kernel, with the compiler named here; any other one
+# builds those MFMAs through the compiler's own intrinsic instead (slower where the register
+# file is full, but hazard-free by construction) and says so.
+VALIDATED_COMPILER = "roc-7.2.0"
+
+
+def _compiler_flags() -> list[str]:
+    try:
+        out = subprocess.run([_hipcc(), "--version"], capture_output=True, text=True).stdout
+    except OSError:
+        out = ""
+    if VALIDATED_COMPILER in out or os.environ.get("TRIFAST_ASM_MFMA") == "1":
+        return []
+    print(f"trifast_amd.build: hipcc is not {VALIDATED_COMPILER}: building the row-resident backward with "
+          "compiler-placed MFMAs (-DTRI_MFMA_ACC_BUILTIN); set TRIFAST_ASM_MFMA=1 to keep the asm form and "
+          "run the GPU tests of the row-resident kernel before trusting it", file=sys.stderr)
+    return ["-DTRI_MFMA_ACC_BUILTIN"]
+
+
 def _hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -77,6 +98,7 @@ def build(verbose: bool = False, jobs: int | None = None, out: Path | None = Non
     srcs = sources()
     if not srcs:
         raise RuntimeError(f"no .hip sources under {CSRC}")
+    extra = (*extra, *_compiler_flags())
     objs = [build_dir / (s.stem + ".o") for s in srcs]
     jobs = jobs or min(len(srcs), int(os.environ.get("MAX_JOBS", "8")))
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:

@@ -690,8 +690,10 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
       const int key = 32 * (KT0 + NWV * t + wave) + kl;
   #pragma unroll
       for (int mt = 0; mt < DM; ++mt) {
+#ifndef TRI_MFMA_ACC_BUILTIN
         asm volatile("s_nop 15" : "+a"(dkacc[t][mt]));
         asm volatile("s_nop 15" : "+a"(dvacc[t][mt]));
+#endif
       }
       if (key >= N) continue;
       store_rows<T, D, DM>(dkrow + (int64_t)key * a.sdk.j, dkacc[t], a.scale, g);

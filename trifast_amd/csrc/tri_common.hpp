@@ -70,15 +70,27 @@ struct Elem<__bf16> {
   // initialisation and its final read.  The compiler does not know that the statement
   // is an MFMA, so the wait states an MFMA needs after a vector-ALU write of one of its
   // operands (two) are spent inside the statement.
+  // (TRI_MFMA_ACC_BUILTIN: the same through the compiler's own MFMA, for a toolchain the asm
+  // form has not been validated with: the compiler then places the accumulators and the wait
+  // states itself, at the price of register copies where the register file is full)
   static TRI_DEV void mfma_acc(frag a, frag b, f32x16& c) {
+#ifdef TRI_MFMA_ACC_BUILTIN
+    c = mfma(a, b, c);
+#else
 asm("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+#endif
   }
   // Such an accumulator is zeroed by an MFMA too (0 * 0 + 0): a vector-ALU write to it
   // right before the first accumulating MFMA is not ordered against that MFMA's read by
   // anything the compiler knows about an asm statement.
   static TRI_DEV void mfma_acc_zero(f32x16& c) {
+#ifdef TRI_MFMA_ACC_BUILTIN
+#pragma unroll
+    for (int v = 0; v < 16; ++v) c[v] = 0.f;
+#else
     const frag z = zero();
 asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %1, 0" : "=a"(c) : "v"(z));  // volatile: one MFMA per accumulator, no copies
+#endif
   }
   static TRI_DEV frag splat(float x) {
     frag f;
@@ -108,11 +120,20 @@ struct Elem<_Float16> {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
   static TRI_DEV void mfma_acc(frag a, frag b, f32x16& c) {
+#ifdef TRI_MFMA_ACC_BUILTIN
+    c = mfma(a, b, c);
+#else
     asm("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+#endif
   }
   static TRI_DEV void mfma_acc_zero(f32x16& c) {
+#ifdef TRI_MFMA_ACC_BUILTIN
+#pragma unroll
+    for (int v = 0; v < 16; ++v) c[v] = 0.f;
+#else
     const frag z = zero();
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %1, 0" : "=a"(c) : "v"(z));
+#endif
   }
   static TRI_DEV frag splat(float x) {
     frag f;
