@@ -321,15 +321,15 @@ __global__ __launch_bounds__(NW * 64, (bwd_kv_min_waves<T, D, R, BJ>())) void tr
     }
   }
 
-  if (!wave_active || key >= N) return;
+  if (!wave_active) return;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int i = i0 + r;
     if (i >= N) continue;
     T* dkrow = reinterpret_cast<T*>(a.dk) + b * a.sdk.b + h * a.sdk.h + i * a.sdk.i + key * a.sdk.j;
     T* dvrow = reinterpret_cast<T*>(a.dv) + b * a.sdv.b + h * a.sdv.h + i * a.sdv.i + key * a.sdv.j;
-    store_rows<T, D, DM>(dkrow, dkacc[r], a.scale, g);
-    store_rows<T, D, DM>(dvrow, dvacc[r], 1.0f, g);
+    store_rows_any<T, D, DM>(dkrow, dkacc[r], a.scale, g, key < N);
+    store_rows_any<T, D, DM>(dvrow, dvacc[r], 1.0f, g, key < N);
   }
 }
 

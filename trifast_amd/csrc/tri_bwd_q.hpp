@@ -307,13 +307,13 @@ __global__ __launch_bounds__(NW * 64, (R >= 4) ? 1 : 2) void tri_bwd_q_kernel(co
   else if (!any_flagged) stage_loop(std::integral_constant<int, kMasked>{});
   else stage_loop(std::integral_constant<int, kGeneral>{});
 
-  if (!wave_active || j >= N) return;
+  if (!wave_active) return;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int i = i0 + r;
     if (i >= N) continue;
     T* dqrow = reinterpret_cast<T*>(a.dq) + b * a.sdq.b + h * a.sdq.h + i * a.sdq.i + j * a.sdq.j;
-    store_rows<T, D, DM>(dqrow, dqacc[r], a.scale, g);
+    store_rows_any<T, D, DM>(dqrow, dqacc[r], a.scale, g, j < N);
   }
 }
 

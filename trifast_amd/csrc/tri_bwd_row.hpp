@@ -27,7 +27,9 @@
 // query) and the key mask (per key) are rank-1 products of operand words.  That leaves
 // the vector ALU one multiply and one exp2 per score, one multiply per dS and the two
 // conversions.  dq of a query tile is the sum of the four waves' partial tiles: they
-// meet in LDS once per query tile and are added in wave order (deterministic, no atomics).
+// meet in LDS once per query tile (one barrier) and each wave adds a quarter of the tile, its
+// own part first and then the others' in wave order (deterministic, no atomics), behind the
+// MFMAs that start the next query tile.
 // The four waves share the LDS pipe, and an LDS instruction occupies it for four cycles
 // whatever its width (transposing reads move half of what 16-byte reads do): operands
 // that do not change over the key tiles of a query tile (Q^T, dO^T) are read once per
@@ -134,17 +136,26 @@ struct RowSchedOf {
 
 // Key tiles per wave whose V operands live in LDS instead of registers: the longest rows
 // leave the vector registers no room for all of them (the accumulators fill the other file).
-constexpr int bwd_row_v_lds_tiles(int D, int KT) { return KT * (D / 16) < 16 ? 0 : D <= 32 ? KT - 2 : 1; }
-// dq partial buffers: two (one barrier per query tile) unless the longest rows need the room
-constexpr int bwd_row_red_buffers(int D, int KT) { return D <= 32 && KT * (D / 16) < 16 ? 2 : 1; }
-// LDS bytes of the kernel below
-constexpr int bwd_row_base_lds_bytes(int D, int es, int KT, bool multi) {
-  const int rowb = D * es, dm = (D + 31) / 32, keys = kRowWaves * KT * 32;
-  const int nred = bwd_row_red_buffers(D, KT);
-  return keys * rowb + 3 * (2 * 32 * rowb) + kRowWaves * 2048 + nred * kRowWaves * dm * 4096 + (multi ? 0 : 2 * keys * 4) +
-         kRowWaves * bwd_row_v_lds_tiles(D, KT) * (D / 16) * 1024;
+// (one tile more in LDS when the row takes several passes: the words of the queries then leave
+// LDS the room, and the dq carried between the passes takes registers)
+constexpr int bwd_row_v_lds_tiles(int D, int KT, bool multi = false) { return KT * (D / 16) < 16 ? 0 : D <= 32 ? KT - (multi ? 2 : 3) : 1; }
+// LDS bytes of the kernel below.  dq partials: two buffers (one barrier per query tile) of
+// three quarters of a tile per wave (the quarter a wave sums itself waits in its dS tile)
+constexpr int bwd_row_red_bytes(int D) { return kRowWaves * 3 * ((D + 31) / 32) * 1024; }
+constexpr int bwd_row_base_lds_bytes(int D, int es, int KT, bool multi) {  // (without the per-query words)
+  const int rowb = D * es, keys = kRowWaves * KT * 32;
+  return keys * rowb + 3 * (2 * 32 * rowb) + kRowWaves * 2048 + 2 * bwd_row_red_bytes(D) +
+         kRowWaves * bwd_row_v_lds_tiles(D, KT, multi) * (D / 16) * 1024;
 }
-constexpr int bwd_row_lds_bytes(int D, int es, int KT, bool multi = false) { return bwd_row_base_lds_bytes(D, es, KT, multi); }
+// The per-query operand words of the row (two planes of 4 bytes per query) live in LDS where
+// there is room and the row takes one pass; else they come from the global planes that the
+// prologue writes, one query tile ahead.
+constexpr bool bwd_row_words_in_lds(int D, int es, int KT, bool multi) {
+  return !multi && bwd_row_base_lds_bytes(D, es, KT, multi) + 2 * kRowWaves * KT * 32 * 4 <= 160 * 1024;
+}
+constexpr int bwd_row_lds_bytes(int D, int es, int KT, bool multi = false) {
+  return bwd_row_base_lds_bytes(D, es, KT, multi) + (bwd_row_words_in_lds(D, es, KT, multi) ? 2 * kRowWaves * KT * 32 * 4 : 0);
+}
 
 template <typename T, int D, int KT, bool MULTI = false>
 __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const BwdArgs a) {
@@ -160,17 +171,17 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   constexpr int PS = 2;
   constexpr int ROWB = Tile::ROWB;
   constexpr int KEYS = NWV * KT * 32;         // keys (and queries) the workgroup can hold
-  constexpr int NRED = bwd_row_red_buffers(D, KT);  // dq partial buffers
+  constexpr bool WORDS_LDS = bwd_row_words_in_lds(D, (int)sizeof(T), KT, MULTI);  // per-query words of the row in LDS (else from the global planes)
   constexpr int STAGE = 2 * 32 * ROWB;        // Q tile | dO tile
   constexpr int OFF_K = 0;
   constexpr int OFF_ST = KEYS * ROWB;
   constexpr int OFF_DS = OFF_ST + 3 * STAGE;  // three stages: in use, ready, in flight
   constexpr int OFF_RED = OFF_DS + NWV * 2048;
-  constexpr int OFF_NL = OFF_RED + NRED * NWV * DM * 4096;
-  constexpr int PLANE = MULTI ? 0 : KEYS * 4;  // per-query words of the row (single pass only)
+  constexpr int OFF_NL = OFF_RED + 2 * bwd_row_red_bytes(D);
+  constexpr int PLANE = WORDS_LDS ? KEYS * 4 : 0;  // per-query words of the row
   constexpr int OFF_ND = OFF_NL + PLANE;
   constexpr int G2W = (2 * 32 * (ROWB / 16) / 64 + NWV - 1) / NWV;  // global->LDS loads per wave and stage
-  constexpr int VL = bwd_row_v_lds_tiles(D, KT);  // this wave's last VL key tiles keep V in LDS
+  constexpr int VL = bwd_row_v_lds_tiles(D, KT, MULTI);  // this wave's last VL key tiles keep V in LDS
   constexpr int VR = KT - VL;
   constexpr int OFF_V = OFF_ND + PLANE;
   static_assert(OFF_V + NWV * VL * DS * 1024 == bwd_row_lds_bytes(D, (int)sizeof(T), KT, MULTI), "the launcher sizes LDS with bwd_row_lds_bytes");
@@ -251,42 +262,96 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   issue_stage(min(1, NJ - 1), 1);
 
   // a fully masked row drops q.k and the bias from its scores (all logits equal)
-  const bool flagged = __builtin_amdgcn_readfirstlane(a.rowflag[(int64_t)b * N + i]) != 0;
+  // (these words come through the scalar cache, all in flight together and apart from the
+  // vector loads around them)
+  const bool flagged = uniform_word(a.rowflag, b * N + i) != 0;
   // keep words of this wave's key tiles (bit k set = key k of the tile is attended)
   uint32_t kw[KT];
 #pragma unroll
   for (int t = 0; t < KT; ++t) {
     const int kt = KT0 + NWV * t + wave;
-    kw[t] = __builtin_amdgcn_readfirstlane(kt < NJ ? a.keep[((int64_t)b * N + i) * a.nwords + kt] : 0u);
+    kw[t] = uniform_word(a.keep, (b * N + i) * a.nwords + min(kt, NJ - 1));
   }
+#pragma unroll
+  for (int t = 0; t < KT; ++t)
+    if (KT0 + NWV * t + wave >= NJ) kw[t] = 0u;
   const uint32_t lanebit = 1u << kl;
 
   // V rows of this lane's keys as B operands: in registers for the wave's first VR key
   // tiles, in a private piece of LDS (operand by operand, 16 bytes per lane) for the rest
   frag vf[VR > 0 ? VR : 1][DS];
   frag* const v_lds = reinterpret_cast<frag*>(tri_smem + OFF_V + wave * VL * DS * 1024) + lane;
+  // (every load of the prologue is issued before the first one is used: the V rows here, then
+  // the row's o and do for delta (queries past the end read the last one again): one trip to
+  // memory for all of them, while the K row is on its way to LDS)
+  frag vx[KT][DS];
 #pragma unroll
   for (int t = 0; t < KT; ++t) {
     const int key = min(32 * (KT0 + NWV * t + wave) + kl, N - 1);
 #pragma unroll
-    for (int s = 0; s < DS; ++s) {
-      const frag x = *reinterpret_cast<const frag*>(vrow + (int64_t)key * a.sv.j + 2 * KP * s + KP * g);
-      if (t < VR) vf[t][s] = x;
-      else v_lds[((t - VR) * DS + s) * 64] = x;
+    for (int s = 0; s < DS; ++s) vx[t][s] = *reinterpret_cast<const frag*>(vrow + (int64_t)key * a.sv.j + 2 * KP * s + KP * g);
+  }
+  const T* const orow = reinterpret_cast<const T*>(a.o) + ((int64_t)bh * N + i) * N * D;
+  const float* const lserow = a.lse + ((int64_t)bh * N + i) * N;
+  constexpr int NIT = WORDS_LDS ? (KEYS + NWV * 64 - 1) / (NWV * 64) : 1;  // queries per thread (single pass)
+  typename E::vec ov[NIT][D / 8], dv[NIT][D / 8];
+  float lv[NIT];
+  if constexpr (WORDS_LDS) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int jc = min(tid + it * NWV * 64, N - 1);
+#pragma unroll
+      for (int s = 0; s < D / 8; ++s) {
+        ov[it][s] = *reinterpret_cast<const typename E::vec*>(orow + (int64_t)jc * D + 8 * s);
+        dv[it][s] = *reinterpret_cast<const typename E::vec*>(dorow + (int64_t)jc * a.sdo.j + 8 * s);
+      }
+      lv[it] = lserow[jc];
     }
   }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int t = 0; t < KT; ++t)
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+      if (t < VR) vf[t][s] = vx[t][s];
+      else v_lds[((t - VR) * DS + s) * 64] = vx[t][s];
+    }
 
   // per-query terms of the row: -delta and -lse*sqrt(d) (ln n for lse in a fully masked
   // row) as MFMA operand words, kept in LDS for this kernel and written for the db kernel
   uint32_t* const dplane = a.delta + ((int64_t)bh * N + i) * N;
   uint32_t* const lplane = a.lse2 + ((int64_t)bh * N + i) * N;
   if (first_pass) {
-    const T* orow = reinterpret_cast<const T*>(a.o) + ((int64_t)bh * N + i) * N * D;
-    const float* lserow = a.lse + ((int64_t)bh * N + i) * N;
     const float flat = -__builtin_amdgcn_logf((float)N) * (kLn2 * a.sqrt_d);
-    for (int j = tid; j < (MULTI ? N : KEYS); j += NWV * 64) {
+    auto query_words = [&](int j, float dsum, float lse_j) {
       float nlv = E::kMaskElem, ndv = 0.f;  // queries past the end: P = dS = 0
       if (j < N) {
+        ndv = -dsum;
+        nlv = flagged ? flat : -lse_j * a.sqrt_d;
+      }
+      const uint32_t lw = split_word<T>(nlv), dw = split_word<T>(ndv);
+      if (j < N) {
+        dplane[j] = dw;
+        lplane[j] = lw;
+      }
+      if constexpr (WORDS_LDS) {
+        nl[j] = lw;
+        nd[j] = dw;
+      }
+    };
+    if constexpr (WORDS_LDS) {
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const int j = tid + it * NWV * 64;
+        float dsum = 0.f;
+#pragma unroll
+        for (int s = 0; s < D / 8; ++s)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) dsum += (float)ov[it][s][e] * (float)dv[it][s][e];
+        if (KEYS % (NWV * 64) == 0 || j < KEYS) query_words(j, dsum, lv[it]);
+      }
+    } else {
+      for (int j = tid; j < N; j += NWV * 64) {
         float dsum = 0.f;
 #pragma unroll
         for (int s = 0; s < D / 8; ++s) {
@@ -295,21 +360,11 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
 #pragma unroll
           for (int e = 0; e < 8; ++e) dsum += (float)ov[e] * (float)dv[e];
         }
-        ndv = -dsum;
-        nlv = flagged ? flat : -lserow[j] * a.sqrt_d;
-      }
-      const uint32_t lw = split_word<T>(nlv), dw = split_word<T>(ndv);
-      if (j < N) {
-        dplane[j] = dw;
-        lplane[j] = lw;
-      }
-      if constexpr (!MULTI) {
-        nl[j] = lw;
-        nd[j] = dw;
+        query_words(j, dsum, lserow[j]);
       }
     }
   }
-  // (several passes: the words come back from the global planes, which the first pass has just
+  // (words not in LDS: they come back from the global planes, which the first pass has just
   // written: its stores are waited for, with the loads, before the barrier below; the loads
   // are made at device scope so that no stale copy in the first-level cache can serve them)
   auto fetch_words = [&](int jt, uint32_t& lw, uint32_t& dw) {
@@ -384,18 +439,30 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   typename OffsetMask<T>::Keys keys_op;
   keys_op.init(kl, g);
 
-  // dq partial tiles of the four waves: [buffer][wave][mt][quarter][lane] x 16 bytes
-  auto red_slot = [&](int buf, int w, int mt, int q, int ln) -> f32x4* {
-    return reinterpret_cast<f32x4*>(tri_smem + OFF_RED + (((buf * NWV + w) * DM + mt) * 4 + q) * 1024) + ln;
-  };
-  // sum the partials of query tile jt in wave order and store the finished elements; this
-  // wave owns quarter `wave` of every lane's values: head-dim elements 32 mt + 8 wave + 4 g
-  // + 0..3 of query 32 jt + kl, 8 bytes per lane (the four waves' stores complete the rows).
+  // dq partial tiles of the four waves.  Wave q sums quarter q of every lane's values: head-dim
+  // elements 32 mt + 8 q + 4 g + 0..3 of query 32 jt + kl, 8 bytes per lane (the four waves'
+  // stores complete the rows).  The other three waves leave their parts of that quarter in
+  // [buffer][summing wave q][slot][mt][lane] x 16 bytes, the slot being the writer's rank among
+  // those three; the wave's own part waits in its dS tile, which is idle between the last key
+  // tile of a query tile and the first of the next.  Partials are added in wave order
+  // (deterministic, no atomics).
   // The store is written as asm: a store the compiler knows of makes its waits for loads
   // waits for everything in flight (stores and loads retire out of order with each other).
   // Addresses are rebuilt from the lane id at every use: kept in registers across the
   // key-tile steps they would be spilled, and a reload from scratch waits for every load
   // in flight.
+  static_assert(DM * 1024 <= 2048, "the own quarter of a dq tile fits the wave's dS tile");
+  constexpr int RED_BYTES = bwd_row_red_bytes(D);
+  // byte offsets in LDS, all wave-uniform and the same for every query tile: where this wave
+  // leaves quarter q of its tile (per buffer), where its own quarter waits, and where the other
+  // waves leave their parts of its quarter (three slots side by side)
+  int part_wr[2][NWV];
+#pragma unroll
+  for (int q = 0; q < NWV; ++q)
+#pragma unroll
+    for (int bf = 0; bf < 2; ++bf)
+      part_wr[bf][q] = q == wave ? OFF_DS + wave * 2048 : OFF_RED + bf * RED_BYTES + (q * 3 + (wave < q ? wave : wave - 1)) * DM * 1024;
+  const int part_own = OFF_DS + wave * 2048, part_rd = OFF_RED + wave * 3 * DM * 1024;
   T* dqrow = reinterpret_cast<T*>(a.dq) + b * a.sdq.b + h * a.sdq.h + i * a.sdq.i;
   T* lorow = reinterpret_cast<T*>(a.dq_lo) + ((int64_t)bh * N + i) * N * D;  // (several passes only)
   typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
@@ -415,38 +482,102 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
       cy.lo[mt] = *reinterpret_cast<const typename E::vec4*>(lorow + (int64_t)j * D + d0);
     }
   };
-  auto reduce_dq = [&](int jt, int buf, const DqCarry& cy) {
+  // this wave's dq tile of a query tile -> LDS, a quarter for each wave that sums one
+  auto store_partials = [&](int buf, const f32x16 (&acc)[DM]) {
     int ln = lane;
     asm volatile("" : "+v"(ln));
-    const int j = 32 * jt + (ln & 31);
+#pragma unroll
+    for (int q = 0; q < NWV; ++q)
+#pragma unroll
+      for (int mt = 0; mt < DM; ++mt) {
+        f32x4 x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] = acc[mt][4 * q + e];
+        *(reinterpret_cast<f32x4*>(tri_smem + (buf ? part_wr[1][q] : part_wr[0][q]) + mt * 1024) + ln) = x;
+      }
+  };
+  // the four parts of this wave's quarter: its own, then the other waves' in wave order
+  struct DqParts {
+    f32x4 v[NWV][DM];
+  };
+  auto load_partials = [&](int buf, DqParts& pp) {
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const f32x4* own = reinterpret_cast<const f32x4*>(tri_smem + part_own) + ln;
+    const f32x4* others = reinterpret_cast<const f32x4*>(tri_smem + part_rd + (buf ? RED_BYTES : 0)) + ln;
 #pragma unroll
     for (int mt = 0; mt < DM; ++mt) {
-      const int d0 = 32 * mt + 8 * wave + 4 * (ln >> 5);
-      f32x4 acc = *red_slot(buf, 0, mt, wave, ln);
+      pp.v[0][mt] = own[mt * 64];
 #pragma unroll
-      for (int w = 1; w < NWV; ++w) acc += *red_slot(buf, w, mt, wave, ln);
-      float out[4];
+      for (int k = 0; k < 3; ++k) pp.v[1 + k][mt] = others[(k * DM + mt) * 64];
+    }
+  };
+  // Their sum (the own part first, then the others in wave order), scaled, as the stores will write it: dq, what rounding it to the
+  // element type lost (between the passes over a long row), and this lane's byte offset from
+  // the start of the query tile in dq (~0: nothing to store).  The sum is cut into pieces of a
+  // few instructions each (piece 0 .. kSumPieces-1, in this order): they run one per MFMA of a
+  // step that has no vector work of its own, in the shadow of the matrix pipe.
+  struct DqOut {
+    f32x4 sum[DM];
+    u32x2v hi[DM], lo[DM];
+    uint32_t off;
+  };
+  constexpr int kSumPieces = 6;
+  auto sum_dq_piece = [&](int piece, int jt, const DqParts& pp, const DqCarry& cy, DqOut& o) {
+    if (piece == 0) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) out[e] = acc[e] * a.scale;
+      for (int mt = 0; mt < DM; ++mt) o.sum[mt] = pp.v[0][mt] + pp.v[1][mt];
+    } else if (piece == 1 || piece == 2) {
+#pragma unroll
+      for (int mt = 0; mt < DM; ++mt) o.sum[mt] += pp.v[piece + 1][mt];
+    } else if (piece == 3) {
+#pragma unroll
+      for (int mt = 0; mt < DM; ++mt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o.sum[mt][e] *= a.scale;
       if constexpr (MULTI) {
         if (!first_pass) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) out[e] += (float)cy.hi[mt][e] + (float)cy.lo[mt][e];
+          for (int mt = 0; mt < DM; ++mt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o.sum[mt][e] += (float)cy.hi[mt][e] + (float)cy.lo[mt][e];
         }
       }
-      typename E::vec4 ov;
+    } else if (piece == 4) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) ov[e] = (T)out[e];
-      if (d0 < D && j < N) {
-        T* dst = dqrow + (int64_t)j * a.sdq.j + d0;
-        asm volatile("global_store_dwordx2 %0, %1, off" : : "v"(dst), "v"(__builtin_bit_cast(u32x2v, ov)) : "memory");
+      for (int mt = 0; mt < DM; ++mt) {
+        typename E::vec4 ov, lv;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          ov[e] = (T)o.sum[mt][e];
+          lv[e] = MULTI ? (T)(o.sum[mt][e] - (float)ov[e]) : (T)0.f;
+        }
+        o.hi[mt] = __builtin_bit_cast(u32x2v, ov);
+        o.lo[mt] = __builtin_bit_cast(u32x2v, lv);
+      }
+    } else {
+      int ln = lane;
+      asm volatile("" : "+v"(ln));
+      const int jl = ln & 31, d0 = 8 * wave + 4 * (ln >> 5);
+      const bool live = jt >= 0 && jl < N - 32 * jt && d0 < D;
+      // (row strides of the gradients are below 2^24 elements, like those of the inputs)
+      o.off = live ? (__umul24((uint32_t)jl, (uint32_t)a.sdq.j) + (uint32_t)d0) * (uint32_t)sizeof(T) : ~0u;
+    }
+  };
+  // (a 64-bit base per query tile in scalar registers and the 32-bit byte offset of the lane)
+  auto store_dq = [&](int jt, const T* base, const DqOut& o) {
+    const T* base_lo = lorow + (int64_t)(32 * jt) * D;
+    if (o.off != ~0u) {
+#pragma unroll
+      for (int mt = 0; mt < DM; ++mt) {
+        if (32 * mt + 8 * wave >= D) continue;  // (wave-uniform; head dims that are no multiple of 32)
+        asm volatile("global_store_dwordx2 %0, %1, %2 offset:%3" : : "v"(o.off), "v"(o.hi[mt]), "s"(base), "n"(64 * mt) : "memory");
         if constexpr (MULTI) {
           if (!last_pass) {
-            typename E::vec4 lv;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) lv[e] = (T)(out[e] - (float)ov[e]);
-            T* ldst = lorow + (int64_t)j * D + d0;
-            asm volatile("global_store_dwordx2 %0, %1, off" : : "v"(ldst), "v"(__builtin_bit_cast(u32x2v, lv)) : "memory");
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            const uint32_t off_lo = (uint32_t)((ln & 31) * D + 8 * wave + 4 * (ln >> 5)) * (uint32_t)sizeof(T);
+            asm volatile("global_store_dwordx2 %0, %1, %2 offset:%3" : : "v"(off_lo), "v"(o.lo[mt]), "s"(base_lo), "n"(64 * mt) : "memory");
           }
         }
       }
@@ -491,28 +622,28 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
     };
     fetch_bias(0, 0);
     fetch_bias(0, 1);
-    uint32_t lw_next = 0u, dw_next = 0u;  // several passes: the words of the next query tile
-    if constexpr (MULTI) fetch_words(0, lw_next, dw_next);
+    uint32_t lw_next = 0u, dw_next = 0u;  // words from the global planes: those of the next query tile
+    if constexpr (!WORDS_LDS) fetch_words(0, lw_next, dw_next);
     DqCarry carry;
+    const T* dq_base = dqrow;  // dq of the query tile before the current one (from the second on)
+    // dq of a query tile is summed over the waves during the first step of the next query tile
+    // (which has no vector work of its own) and stored near its end, where the next wait for a
+    // load is furthest away: a wait for loads that were issued after a store waits for the store.
     int buf = 0;  // jt % 3: the stage of this query tile
     for (int jt = 0; jt < NJ; ++jt) {
       const int buf_fill = buf == 0 ? 2 : buf - 1;  // (jt + 2) % 3: the stage to refill
-      if (jt > 0) {
-        if constexpr (NRED == 2) reduce_dq(jt - 1, (jt - 1) & 1, carry);
-      }
-      if constexpr (MULTI) {
-        if (!first_pass) fetch_carry(jt, carry);
-      }
+      DqParts parts;  // (of the query tile before this one)
+      DqOut dq_words;
+      f32x16 dqacc[DM];  // (the first dq MFMA of a query tile starts it from zero)
       const unsigned char* qt = tri_smem + OFF_ST + buf * STAGE;
       const unsigned char* dot = qt + 32 * ROWB;
 
       // operand words of this lane's query (lanes 32..63 carry zeros)
       {
         uint32_t lw, dw;
-        if constexpr (MULTI) {
+        if constexpr (!WORDS_LDS) {
           lw = lw_next;
           dw = dw_next;
-          fetch_words(jt + 1, lw_next, dw_next);
         } else {
           lw = nl[32 * jt + perm32(kl)];
           dw = nd[32 * jt + perm32(kl)];
@@ -540,9 +671,6 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
             dotr[mt][s2] = ofq.transposed(dot, s2, mt);
           }
       };
-      f32x16 dqacc[DM];
-#pragma unroll
-      for (int mt = 0; mt < DM; ++mt) dqacc[mt] = zero16();
 
       // ---- the state that moves from step to step --------------------------------------
       f32x16 s_cur, p_cur;   // scores and dP of the tile whose P, dS the step computes
@@ -560,7 +688,6 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
         }
       };
       load_kn(0);
-      if constexpr (QD_ONCE) load_qd_tr();
 
       // Step t (t = -1 .. KT): the vector work of tile t (P, dS, their conversions) between
       // the MFMAs of its neighbours: dv, dk and dq of tile t-1, scores and dP of tile t+1,
@@ -579,6 +706,9 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
         constexpr bool refill = t == KT - 2;
         constexpr int refill_at = FLAGGED ? 0 : Sch::value.last_sb;
         SB();
+        // (words from the global planes: those of the next query tile, fetched before the last
+        // bias tile of this one so that no wait for them is a wait for everything in flight)
+        if constexpr (!WORDS_LDS && t == KT - 1) fetch_words(jt + 1, lw_next, dw_next);
         if constexpr (valu && !refill) fetch_bias(jt, t + 2);
         frag kb = keys_op.plain();
         if constexpr (has_next && MASKED) kb = keys_op.masked(kw[tn]);
@@ -602,9 +732,32 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
             if constexpr (idx % 2 == 0) E::mfma_acc(dotr[mt][s2], pf[s2], dvacc[tp][mt]);
             else E::mfma_acc(qtr[mt][s2], dsf[s2], dkacc[tp][mt]);
           } else {
-            dqacc[idx % DM] = E::mfma(ktr_prev[idx % DM][idx / DM], dst_prev[idx / DM], dqacc[idx % DM]);
+            if constexpr (tp == 0 && idx / DM == 0) dqacc[idx % DM] = E::mfma(ktr_prev[idx % DM][idx / DM], dst_prev[idx / DM], zero16());
+            else dqacc[idx % DM] = E::mfma(ktr_prev[idx % DM][idx / DM], dst_prev[idx / DM], dqacc[idx % DM]);
           }
           SB();
+          // Q^T, dO^T of the query tile are first used by the step after next: their reads go
+          // where the LDS pipe has nothing else to do
+          if constexpr (QD_ONCE && t == -1 && x == 1) load_qd_tr();
+          // dq of the query tile before this one: its parts come from LDS early in this step,
+          // which has no vector work of its own, and are summed and stored piece by piece behind
+          // the MFMAs that follow (before the first query tile the sum is of stale bytes and is
+          // not stored).  No wait for a load that could follow within the time a store takes
+          // allows fewer than two operations in flight, so none of them waits for this store
+          // (a wait for loads issued after a store is a wait for the store as well).
+          if constexpr (t == -1) {
+            if constexpr (x == 0) load_partials((jt + 1) & 1, parts);
+#pragma unroll
+            for (int piece = 0; piece < kSumPieces; ++piece)
+              if ((piece + 3 < NM ? piece + 3 : NM - 1) == x) sum_dq_piece(piece, jt - 1, parts, carry, dq_words);
+            if constexpr (x == NM - 1) {
+              store_dq(jt - 1, dq_base, dq_words);
+              if (jt > 0) dq_base += 32 * a.sdq.j;
+              if constexpr (MULTI) {
+                if (!first_pass) fetch_carry(jt, carry);
+              }
+            }
+          }
           if constexpr (has_prev && x == Sch::value.dq_reads_at) {
             // dS of tile t-1 comes back from LDS with the key index in-lane, with the K
             // rows of that tile transposed beside it
@@ -653,32 +806,24 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
         if constexpr (has_next) { s_cur = s_nxt; p_cur = p_nxt; }
       };
       static_for<KT + 2>(step);
-
-      // this wave's partial dq tile -> LDS
-      const int rbuf = NRED == 2 ? (jt & 1) : 0;
-      int ln = lane;
-      asm volatile("" : "+v"(ln));
-#pragma unroll
-      for (int mt = 0; mt < DM; ++mt)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          f32x4 x;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) x[e] = dqacc[mt][4 * q + e];
-          *red_slot(rbuf, wave, mt, q, ln) = x;
-        }
+      store_partials(jt & 1, dqacc);
       // The stage of the next query tile was requested a whole query tile ago; since then
       // the wave has issued the loads of the stage after it and (unless the row is fully
       // masked) of two bias tiles: everything older than those has landed.  A barrier
-      // without a fence: a fence would wait for the loads in flight.
-      ring_sync<G2W + (FLAGGED ? 0 : 4)>();
+      // without a fence: a fence would wait for the loads in flight.  It is the only one of
+      // the query tile: the partials written before it are read after it, and the buffer they
+      // are in is written again two query tiles on, behind the next barrier.
+      ring_sync<G2W + (FLAGGED ? 0 : 4) + (WORDS_LDS ? 0 : 2)>();
       buf = buf == 2 ? 0 : buf + 1;
-      if constexpr (NRED == 1) {
-        reduce_dq(jt, 0, carry);
-        ring_sync<G2W + (FLAGGED ? 0 : 4)>();
-      }
     }
-    if constexpr (NRED == 2) reduce_dq(NJ - 1, (NJ - 1) & 1, carry);
+    {
+      DqParts parts;
+      DqOut dq_words;
+      load_partials((NJ - 1) & 1, parts);
+#pragma unroll
+      for (int piece = 0; piece < kSumPieces; ++piece) sum_dq_piece(piece, NJ - 1, parts, carry, dq_words);
+      store_dq(NJ - 1, dq_base, dq_words);
+    }
 
     // ---- dk, dv of this wave's keys -------------------------------------------------------
     // (the accumulators were last written by MFMAs inside asm statements, which the compiler
@@ -695,9 +840,8 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
         asm volatile("s_nop 15" : "+a"(dvacc[t][mt]));
 #endif
       }
-      if (key >= N) continue;
-      store_rows<T, D, DM>(dkrow + (int64_t)key * a.sdk.j, dkacc[t], a.scale, g);
-      store_rows<T, D, DM>(dvrow + (int64_t)key * a.sdv.j, dvacc[t], 1.0f, g);
+      store_rows_wide<T, D, DM>(dkrow + (int64_t)key * a.sdk.j, dkacc[t], a.scale, g, key < N);
+      store_rows_wide<T, D, DM>(dvrow + (int64_t)key * a.sdv.j, dvacc[t], 1.0f, g, key < N);
     }
   };
   bool plain = true;

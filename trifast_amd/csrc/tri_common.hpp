@@ -402,6 +402,15 @@ TRI_DEV void static_for(F&& f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
+// A 32-bit word at a wave-uniform index, read through the scalar cache: for words that an
+// earlier kernel wrote (the scalar cache starts every kernel empty).  Several such loads are
+// all in flight before the first of them is waited for, and none of them waits for vector
+// memory operations in flight; a vector load followed by readfirstlane waits for everything.
+TRI_DEV uint32_t uniform_word(const uint32_t* p, int idx) {
+  typedef const uint32_t __attribute__((address_space(4))) * const_ptr;
+  return ((const_ptr)(uintptr_t)p)[__builtin_amdgcn_readfirstlane(idx)];
+}
+
 // acc + the two values of a packed pair (what an MFMA that consumes the pair sees)
 TRI_DEV float pair_sum(bf16x2 w, bf16x2 ones, float acc) { return __builtin_amdgcn_fdot2_f32_bf16(w, ones, acc, false); }
 TRI_DEV float pair_sum(f16x2 w, f16x2 ones, float acc) { return __builtin_amdgcn_fdot2(w, ones, acc, false); }

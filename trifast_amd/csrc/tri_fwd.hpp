@@ -720,10 +720,10 @@ __global__ __launch_bounds__(NW * 64, (R * ((BKF % kFwdFast) / 32) >= 8) ? 1 : 2
   for (int r = 0; r < R; ++r) {
     const int i = i0 + r;
     const float ltot = half_sum(lrun[r]);
-    if (i >= N || j >= N) continue;
+    if (i >= N) continue;  // (wave-uniform; the lanes of queries past the end stay for the exchange inside the store)
     T* orow = reinterpret_cast<T*>(a.o) + (((int64_t)bh * N + i) * N) * D;
-    store_rows<T, D, DM>(orow + (int64_t)j * D, oacc[r], 1.0f / ltot, g);
-    if (g == 0) {
+    store_rows_any<T, D, DM>(orow + (int64_t)j * D, oacc[r], 1.0f / ltot, g, j < N);
+    if (g == 0 && j < N) {
       float lse = kLn2 * (mc[r] + fast_log2(ltot));
       if (flagged[r]) lse = a.neg_inf + lse;
       a.lse[((int64_t)bh * N + i) * N + j] = lse;

@@ -413,4 +413,46 @@ TRI_DEV void store_rows(T* out_row, const f32x16* acc, float mul, int g) {
   }
 }
 
+// The same store for 16-bit outputs with 16 bytes per lane: lane l and lane l ^ 32 own the
+// two halves of every 8 columns of one row; they trade values (v_permlane32_swap) so that
+// the lower lane ends up with columns 32*mt + 8*h + 0..7 and the upper lane with columns
+// 32*mt + 16 + 8*h + 0..7, each whole.  Half as many store instructions, each of them
+// writing whole 16-byte pieces.  Every lane of the wave takes part in the exchange;
+// `active` says whether this lane's row is stored.
+template <typename T, int D, int DM>
+TRI_DEV void store_rows_wide(T* out_row, const f32x16* acc, float mul, int g, bool active) {
+  static_assert(sizeof(T) == 2, "16-bit outputs");
+  using E = Elem<T>;
+  typedef uint32_t u32x2s __attribute__((ext_vector_type(2)));
+  typedef uint32_t u32x4s __attribute__((ext_vector_type(4)));
+#pragma unroll
+  for (int mt = 0; mt < DM; ++mt) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      typename E::vec4 lo4, hi4;  // this lane's columns 8h + 4g + 0..3 and 8(h+2) + 4g + 0..3
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lo4[e] = (T)(acc[mt][4 * h + e] * mul);
+        hi4[e] = (T)(acc[mt][4 * (h + 2) + e] * mul);
+      }
+      const u32x2s x = __builtin_bit_cast(u32x2s, lo4), y = __builtin_bit_cast(u32x2s, hi4);
+      const auto r0 = __builtin_amdgcn_permlane32_swap(x[0], y[0], false, false);
+      const auto r1 = __builtin_amdgcn_permlane32_swap(x[1], y[1], false, false);
+      const u32x4s out = {(uint32_t)r0[0], (uint32_t)r1[0], (uint32_t)r0[1], (uint32_t)r1[1]};
+      const int d0 = 32 * mt + 16 * g + 8 * h;
+      if (active && d0 < D) *reinterpret_cast<u32x4s*>(out_row + d0) = out;
+    }
+  }
+}
+
+// either of the two, by the element type
+template <typename T, int D, int DM>
+TRI_DEV void store_rows_any(T* out_row, const f32x16* acc, float mul, int g, bool active) {
+  if constexpr (sizeof(T) == 2) {
+    store_rows_wide<T, D, DM>(out_row, acc, mul, g, active);
+  } else {
+    if (active) store_rows<T, D, DM>(out_row, acc, mul, g);
+  }
+}
+
 }  // namespace tri
