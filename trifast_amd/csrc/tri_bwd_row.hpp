@@ -54,6 +54,28 @@
 #include "tri_common.hpp"
 #include "tri_tile.hpp"
 
+// -DTRI_ROW_TIMING builds the kernel as a probe of itself (benchmark/microbench/row_timeline.py):
+// wave 0 of every workgroup reads the 100 MHz counter at the marks below and the shader clock
+// between the steps of the query-tile loop, and leaves the readings where the db argument
+// points (a buffer of the caller's; db itself is not computed by this kernel).
+#ifdef TRI_ROW_TIMING
+#define TRI_ROW_MARK(var)               \
+  __builtin_amdgcn_sched_barrier(0);    \
+  const uint64_t var = __builtin_amdgcn_s_memrealtime(); \
+  __builtin_amdgcn_sched_barrier(0)
+#define TRI_ROW_TICK(k)                                      \
+  do {                                                       \
+    __builtin_amdgcn_sched_barrier(0);                       \
+    const uint64_t now_ = __builtin_amdgcn_s_memtime();      \
+    tacc[k] += now_ - tprev;                                 \
+    tprev = now_;                                            \
+    __builtin_amdgcn_sched_barrier(0);                       \
+  } while (0)
+#else
+#define TRI_ROW_MARK(var) (void)0
+#define TRI_ROW_TICK(k) (void)0
+#endif
+
 namespace tri {
 
 constexpr int kRowWaves = 4;
@@ -189,6 +211,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   static_assert((KT - 1) * NWV * 32 * ROWB + 32 * ROWB <= 65536, "key tile offsets are LDS immediates");
   extern __shared__ __attribute__((aligned(16))) unsigned char tri_smem[];
 
+  TRI_ROW_MARK(t_entry);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -275,6 +298,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
 #pragma unroll
   for (int t = 0; t < KT; ++t)
     if (KT0 + NWV * t + wave >= NJ) kw[t] = 0u;
+  TRI_ROW_MARK(t_p1);
   const uint32_t lanebit = 1u << kl;
 
   // V rows of this lane's keys as B operands: in registers for the wave's first VR key
@@ -317,6 +341,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
       else v_lds[((t - VR) * DS + s) * 64] = vx[t][s];
     }
 
+  TRI_ROW_MARK(t_p2);
   // per-query terms of the row: -delta and -lse*sqrt(d) (ln n for lse in a fully masked
   // row) as MFMA operand words, kept in LDS for this kernel and written for the db kernel
   uint32_t* const dplane = a.delta + ((int64_t)bh * N + i) * N;
@@ -364,6 +389,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
       }
     }
   }
+  TRI_ROW_MARK(t_p3);
   // (words not in LDS: they come back from the global planes, which the first pass has just
   // written: its stores are waited for, with the loads, before the barrier below; the loads
   // are made at device scope so that no stale copy in the first-level cache can serve them)
@@ -584,6 +610,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
     }
   };
 
+  TRI_ROW_MARK(t_p4);
   wait_dma_known();
   __syncthreads();
 
@@ -630,6 +657,11 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
     // (which has no vector work of its own) and stored near its end, where the next wait for a
     // load is furthest away: a wait for loads that were issued after a store waits for the store.
     int buf = 0;  // jt % 3: the stage of this query tile
+#ifdef TRI_ROW_TIMING
+    uint64_t tacc[KT + 5] = {};  // shader clocks per step, summed over the query tiles
+    const uint64_t t_clk0 = __builtin_amdgcn_s_memtime(), t_loop0 = __builtin_amdgcn_s_memrealtime();
+    uint64_t tprev = t_clk0;
+#endif
     for (int jt = 0; jt < NJ; ++jt) {
       const int buf_fill = buf == 0 ? 2 : buf - 1;  // (jt + 2) % 3: the stage to refill
       DqParts parts;  // (of the query tile before this one)
@@ -706,6 +738,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
         constexpr bool refill = t == KT - 2;
         constexpr int refill_at = FLAGGED ? 0 : Sch::value.last_sb;
         SB();
+        TRI_ROW_TICK(t + 1);  // (slot 0: from the loop head to step -1; slot k: step k-2)
         // (words from the global planes: those of the next query tile, fetched before the last
         // bias tile of this one so that no wait for them is a wait for everything in flight)
         if constexpr (!WORDS_LDS && t == KT - 1) fetch_words(jt + 1, lw_next, dw_next);
@@ -806,7 +839,9 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
         if constexpr (has_next) { s_cur = s_nxt; p_cur = p_nxt; }
       };
       static_for<KT + 2>(step);
+      TRI_ROW_TICK(KT + 2);
       store_partials(jt & 1, dqacc);
+      TRI_ROW_TICK(KT + 3);
       // The stage of the next query tile was requested a whole query tile ago; since then
       // the wave has issued the loads of the stage after it and (unless the row is fully
       // masked) of two bias tiles: everything older than those has landed.  A barrier
@@ -814,6 +849,7 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
       // the query tile: the partials written before it are read after it, and the buffer they
       // are in is written again two query tiles on, behind the next barrier.
       ring_sync<G2W + (FLAGGED ? 0 : 4) + (WORDS_LDS ? 0 : 2)>();
+      TRI_ROW_TICK(KT + 4);
       buf = buf == 2 ? 0 : buf + 1;
     }
     {
@@ -824,6 +860,9 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
       for (int piece = 0; piece < kSumPieces; ++piece) sum_dq_piece(piece, NJ - 1, parts, carry, dq_words);
       store_dq(NJ - 1, dq_base, dq_words);
     }
+#ifdef TRI_ROW_TIMING
+    const uint64_t t_clk1 = __builtin_amdgcn_s_memtime(), t_loop1 = __builtin_amdgcn_s_memrealtime();
+#endif
 
     // ---- dk, dv of this wave's keys -------------------------------------------------------
     // (the accumulators were last written by MFMAs inside asm statements, which the compiler
@@ -843,6 +882,19 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
       store_rows_wide<T, D, DM>(dkrow + (int64_t)key * a.sdk.j, dkacc[t], a.scale, g, key < N);
       store_rows_wide<T, D, DM>(dvrow + (int64_t)key * a.sdv.j, dvacc[t], 1.0f, g, key < N);
     }
+#ifdef TRI_ROW_TIMING
+    // one record of 32 words per workgroup (wave 0), at the start of what db points to
+    if (wave == 0 && lane == 0) {
+      uint64_t* rec = reinterpret_cast<uint64_t*>(a.db) + (int64_t)L * 32;
+      const uint64_t t_end = __builtin_amdgcn_s_memrealtime();
+      const uint64_t marks[8] = {t_entry, t_p1, t_p2, t_p3, t_p4, t_loop0, t_loop1, t_end};  // 100 MHz
+      for (int x = 0; x < 8; ++x) rec[x] = marks[x];
+      rec[8] = __builtin_amdgcn_s_getreg(4 | (0 << 6) | (31 << 11));   // HW_ID
+      rec[9] = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (31 << 11));  // XCC_ID
+      rec[10] = t_clk1 - t_clk0;                                        // shader clocks of the loop
+      for (int x = 0; x < KT + 5; ++x) rec[11 + x] = tacc[x];
+    }
+#endif
   };
   bool plain = true;
 #pragma unroll
