@@ -171,7 +171,7 @@ def kernel_breakdown(q, k, v, bias, mask, do, reps):
     for kernel in (_lib.KERNEL_FWD, _lib.KERNEL_BWD_Q, _lib.KERNEL_BWD_KV, _lib.KERNEL_BWD_B):
         launch = fwd if kernel == _lib.KERNEL_FWD else (lambda t, kern=kernel: bwd_one(kern, t))
         tile = tuner.pick(kernel, n, h, d, q.dtype, launch)
-        for _ in range(3):  # (the first launches after a change of kernel run at other clocks)
+        for _ in range(20):  # (after a pause the clocks take some twenty milliseconds to come back up)
             launch(tile)
         torch.cuda.synchronize()
         out[_lib.KERNEL_NAMES[kernel]] = {"ms": _event_ms(lambda: launch(tile), reps), "tile": dict(_lib.tile_info(kernel, tile), id=tile)}
