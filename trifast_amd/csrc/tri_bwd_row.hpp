@@ -470,8 +470,8 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
   // stores complete the rows).  The other three waves leave their parts of that quarter in
   // [buffer][summing wave q][slot][mt][lane] x 16 bytes, the slot being the writer's rank among
   // those three; the wave's own part waits in its dS tile, which is idle between the last key
-  // tile of a query tile and the first of the next.  Partials are added in wave order
-  // (deterministic, no atomics).
+  // tile of a query tile and the first of the next.  A wave adds its own part first, then the
+  // others' in wave order (deterministic, no atomics).
   // The store is written as asm: a store the compiler knows of makes its waits for loads
   // waits for everything in flight (stores and loads retire out of order with each other).
   // Addresses are rebuilt from the lane id at every use: kept in registers across the
@@ -653,9 +653,8 @@ __global__ __launch_bounds__(kRowWaves * 64, 1) void tri_bwd_row_kernel(const Bw
     if constexpr (!WORDS_LDS) fetch_words(0, lw_next, dw_next);
     DqCarry carry;
     const T* dq_base = dqrow;  // dq of the query tile before the current one (from the second on)
-    // dq of a query tile is summed over the waves during the first step of the next query tile
-    // (which has no vector work of its own) and stored near its end, where the next wait for a
-    // load is furthest away: a wait for loads that were issued after a store waits for the store.
+    // dq of a query tile is summed over the waves, and stored, during the first step of the
+    // next query tile, which has no vector work of its own.
     int buf = 0;  // jt % 3: the stage of this query tile
 #ifdef TRI_ROW_TIMING
     uint64_t tacc[KT + 5] = {};  // shader clocks per step, summed over the query tiles
