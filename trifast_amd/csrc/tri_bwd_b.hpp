@@ -190,6 +190,20 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
       item_base[x] += advance & item_step[x];
     }
   };
+  // the same, one item at a time (for loops that deal the loads of a row between other work);
+  // next_row_advance() once per row, before its items
+  auto next_row_advance = [&]() __attribute__((always_inline)) -> int64_t {
+    const int64_t advance = ones_while_positive(nrows - 1 - rows_issued);
+    ++rows_issued;
+    return advance;
+  };
+  auto issue_item = [&](int buf, auto x_tag, int64_t advance) __attribute__((always_inline)) {
+    constexpr int x = decltype(x_tag)::value;
+    const uint32_t dst = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(TRI_L3 unsigned char*)(tri_smem + buf * STAGE) + (uint32_t)item_lds[x]);
+    if constexpr (x < XW) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(item_voff[x]), "s"(item_base[x]) : "memory", "m0");
+    else asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(dst), "v"(item_voff[x]), "s"(item_base[x]) : "memory", "m0");
+    item_base[x] += advance & item_step[x];
+  };
   // wait until at most the newest `K` rows of this wave's loads are in flight and
   // every LDS read has returned, then meet the other waves
   auto sync_rows = [&](auto k_tag) {
@@ -371,6 +385,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     }
   };
 
+  auto walk_rows = [&]() __attribute__((always_inline)) {
   if constexpr (NBUF >= 2) {
     // Ring of NBUF row buffers: the loads run NBUF-1 rows ahead of the compute, which
     // hides the memory latency behind several rows of work.  Row q lives in buffer
@@ -402,6 +417,156 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
       if (wave_live != 0) compute_row(0, meta);
       sync_rows(std::integral_constant<int, 0>{});
     }
+  }
+  };
+  // Workgroups of the 8-wave block whose rows are all plain (no flagged row, no masked key in
+  // any of the block's key tiles: the common case) walk the rows software-pipelined: a wave's
+  // matrix instructions of one tile are issued between the exponentials and multiply-adds of
+  // the tile before it (the second tile of a row overlaps the first, the first tile of the
+  // next row overlaps the second), so neither pipe waits for the other although only two
+  // waves share a SIMD.  The next row's operands are read from LDS a whole row ahead.
+  constexpr bool kPipelined = WJ == 1 && WK == 2 && NBUF == 4 && sizeof(T) == 2 && D <= 32;
+  if constexpr (kPipelined) {
+    bool mine = nrows > 0;
+    {
+      const int w0 = k_blk / 32;
+      for (int i = i_begin + tid; i < i_end; i += NW * 64) {
+        mine = mine && a.rowflag[(int64_t)b * N + i] == 0;
+        const uint32_t* kw = a.keep + ((int64_t)b * N + i) * a.nwords;
+#pragma unroll
+        for (int w = 0; w < BKB / 32; ++w) mine = mine && (w0 + w < a.nwords ? kw[w0 + w] : 0u) == 0xffffffffu;
+      }
+    }
+    // all lanes of all waves agree: one word per wave through LDS (not yet in use)
+    uint32_t* votes = reinterpret_cast<uint32_t*>(tri_smem);
+    const bool wave_ok = __builtin_amdgcn_readfirstlane((int)(__ballot(mine) == ~0ull)) != 0;
+    if (lane == 0) votes[wave] = wave_ok ? 1u : 0u;
+    __syncthreads();
+    bool plain = true;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) plain = plain && votes[w] != 0;
+    plain = __builtin_amdgcn_readfirstlane((int)plain) != 0;
+    __syncthreads();
+    if (plain) {
+      struct RowOps {
+        frag q[WJ][DS], dout[WJ][DS], k[WK][DS], v[WK][DS];
+        frag df[WJ];    // -delta of the lane's query as a rank-1 operand
+        float nl2[WJ];  // -lse of the lane's query in the exponent's unit
+        uint32_t lw[WJ], dw[WJ];
+      };
+      auto read_ops = [&](int buf, RowOps& o) __attribute__((always_inline)) {
+        const bool high = kHighSet && buf >= 2;
+        const int sl = buf * STAGE - (high ? HIGH : 0);
+        const OperandOffsets<T, D>& oq = high ? ofq_hi : ofq;
+        const OperandOffsets<T, D>& ok = high ? ofk_hi : ofk;
+        const int soff = high ? scalar_off_hi : scalar_off;
+#pragma unroll
+        for (int tj = 0; tj < WJ; ++tj) {
+#pragma unroll
+          for (int s = 0; s < DS; ++s) {
+            o.q[tj][s] = oq.natural_at(sl + OFF_Q + tj * 32 * ROWB, s);
+            o.dout[tj][s] = oq.natural_at(sl + OFF_DO + tj * 32 * ROWB, s);
+          }
+          o.lw[tj] = *reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_LSE + tj * 128 + soff));
+          o.dw[tj] = *reinterpret_cast<TRI_L3 const uint32_t*>((uintptr_t)(uint32_t)(sl + OFF_DELTA + tj * 128 + soff));
+        }
+#pragma unroll
+        for (int tk = 0; tk < WK; ++tk)
+#pragma unroll
+          for (int s = 0; s < DS; ++s) {
+            o.k[tk][s] = ok.natural_at(sl + OFF_K + tk * 32 * ROWB, s);
+            o.v[tk][s] = ok.natural_at(sl + OFF_V + tk * 32 * ROWB, s);
+          }
+      };
+      auto finish_ops = [&](RowOps& o) __attribute__((always_inline)) {
+#pragma unroll
+        for (int tj = 0; tj < WJ; ++tj) {
+          o.nl2[tj] = split_value<T>(o.lw[tj]) * c;
+          o.df[tj] = drank[tj].set(g ? 0u : o.dw[tj]);
+        }
+      };
+      // The tiles of a wave in the order they are walked: tile t is (t / WK, t % WK).  The
+      // matrix instructions of tile `tn` of row `on` (scores from the bias tile, dP from
+      // -delta) go into sn / dpn, dealt between the elementwise work of tile `tc` of row
+      // `oc`, whose scores s and dP are complete: db += exp2(c s - lse) dP.
+      constexpr int NT = WJ * WK;
+      constexpr int NM = 2 * DS + 1;
+      auto phase = [&](const RowOps& on, auto tn_tag, f32x16& sn, f32x16& dpn, const RowOps& oc, auto tc_tag, const f32x16& s,
+                       const f32x16& dp, auto&& between) __attribute__((always_inline)) {
+        constexpr int TN = decltype(tn_tag)::value, TC = decltype(tc_tag)::value;
+        constexpr int nj = TN / WK, nk = TN % WK, cj = TC / WK, ck = TC % WK;
+        static_for<NM>([&](auto xc) __attribute__((always_inline)) {
+          constexpr int X = decltype(xc)::value;
+          // the two chains alternate, so that an instruction seldom waits for the one before it
+          constexpr bool IS_S = X == 0 || (X >= 2 && X % 2 == 0 && X / 2 < DS);
+          constexpr int before = (X - 1) / 2 < DS - 1 ? (X - 1) / 2 : DS - 1;  // score steps among slots 1 .. X-1
+          constexpr int DI = X - 2 - before;                                    // dP steps among them, less the -delta one
+          if constexpr (X == 0) sn = E::mfma(on.k[nk][0], on.q[nj][0], biasr[nj][nk]);
+          else if constexpr (X == 1) dpn = E::mfma(ones, on.df[nj], zero16());
+          else if constexpr (IS_S) sn = E::mfma(on.k[nk][X / 2], on.q[nj][X / 2], sn);
+          else dpn = E::mfma(on.v[nk][DI], on.dout[nj][DI], dpn);
+          between(std::integral_constant<int, TC * NM + X>{});
+#pragma unroll
+          for (int v = 16 * X / NM; v < 16 * (X + 1) / NM; ++v) {
+            const float p = fast_exp2(__builtin_fmaf(s[v], c, oc.nl2[cj]));
+            dbacc[cj][ck][v] = __builtin_fmaf(p, dp[v], dbacc[cj][ck][v]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      };
+      constexpr int AHEAD = NBUF;  // rows between the loads and the compute
+#pragma unroll
+      for (int u = 0; u < AHEAD; ++u) issue_row(u);
+      sync_rows(std::integral_constant<int, AHEAD - 2>{});  // rows 0 and 1 have landed
+      // (two sets of operand registers that swap roles from row to row: no copies)
+      RowOps ops[2];
+      f32x16 sc[2], dpc[2];  // scores and dP of the tile in flight and the tile being consumed
+      read_ops(0, ops[0]);
+      finish_ops(ops[0]);
+      sc[0] = E::mfma(ops[0].k[0][0], ops[0].q[0][0], biasr[0][0]);
+#pragma unroll
+      for (int sd = 1; sd < DS; ++sd) sc[0] = E::mfma(ops[0].k[0][sd], ops[0].q[0][sd], sc[0]);
+      dpc[0] = E::mfma(ones, ops[0].df[0], zero16());
+#pragma unroll
+      for (int sd = 0; sd < DS; ++sd) dpc[0] = E::mfma(ops[0].v[0][sd], ops[0].dout[0][sd], dpc[0]);
+      sc[1] = zero16();
+      dpc[1] = zero16();
+      sync_rows(std::integral_constant<int, AHEAD - 2>{});  // every wave has read row 0: its buffer is free
+      static_assert(NT % 2 == 0, "the two accumulator sets swap once per tile");
+      for (int r = 0; r < nrows; r += NBUF) {
+#pragma unroll
+        for (int u = 0; u < NBUF; ++u) {
+          if (r + u < nrows) {
+            RowOps& cur = ops[u & 1];
+            RowOps& next = ops[(u + 1) & 1];
+            // row r + u + NBUF goes into the buffer whose row is in registers already; its
+            // loads are dealt over the row (a burst of them would hold up the wave's other
+            // instructions until the memory pipeline has taken them all)
+            const int64_t advance = next_row_advance();
+            auto deal_loads = [&](auto slot_tag) __attribute__((always_inline)) {
+              constexpr int slot = decltype(slot_tag)::value;
+              static_for<XN>([&](auto xt) __attribute__((always_inline)) {
+                constexpr int x = decltype(xt)::value;
+                if constexpr (slot == (x * NT * NM) / XN) issue_item(u, xt, advance);
+              });
+            };
+            read_ops((u + 1) % NBUF, next);
+            __builtin_amdgcn_sched_barrier(0);
+            static_for<NT - 1>([&](auto tc) __attribute__((always_inline)) {
+              constexpr int t = decltype(tc)::value;
+              phase(cur, std::integral_constant<int, t + 1>{}, sc[(t + 1) & 1], dpc[(t + 1) & 1], cur, tc, sc[t & 1], dpc[t & 1], deal_loads);
+            });
+            finish_ops(next);
+            phase(next, std::integral_constant<int, 0>{}, sc[0], dpc[0], cur, std::integral_constant<int, NT - 1>{}, sc[(NT - 1) & 1], dpc[(NT - 1) & 1], deal_loads);
+            sync_rows(std::integral_constant<int, AHEAD - 2>{});  // rows up to r + u + 2 have landed
+          }
+        }
+      }
+    } else {
+      walk_rows();
+    }
+  } else {
+    walk_rows();
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the spare rows loaded past the end
   if (wave_live == 0) return;
