@@ -147,6 +147,59 @@ def test_every_tile(n, h, d, dtype, monkeypatch):
 
 
 # ---------------------------------------------------------------------------
+# the db kernel's pipelined walk of plain rows (blocks whose waves own two key tiles) and
+# its hand-over to the general loop at the first row that is not plain: no mask at all,
+# padding (keys and rows past a valid length), one masked row in the middle, a masked row
+# near the start (nothing is pipelined then).  Several row chunks at these sizes.
+# Each such tile must give db within the reference's bound of the oracle, and bit-identical
+# to the 16-wave tile where every block is plain (same order of the sum over the rows, same
+# arithmetic per element).
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("pattern", ["none", "padding", "middle", "early"])
+@pytest.mark.parametrize("n,h,d", [(300, 2, 32), (256, 1, 16), (200, 1, 32)])
+def test_db_pipelined_rows(n, h, d, pattern, dtype, monkeypatch):
+    lib = _lib.load()
+    code = tt._DTYPE_CODE[dtype]
+    g = torch.Generator().manual_seed(n + d)
+    q, k, v, b, m = orc.gen_tensors(n, d, h, False, "cpu", torch.float32, 1, 1.0, generator=g)
+    if pattern == "padding":
+        valid = n - 37
+        m[:, valid:, :] = True
+        m[:, :, valid:] = True
+    elif pattern == "middle":
+        m[:, n // 2, :] = torch.rand(n, generator=g) < 0.3
+        m[:, n // 2 + 9, :] = True
+    elif pattern == "early":
+        m[:, 5, 1::2] = True
+    do = torch.randn(q.shape, generator=g)
+    q, k, v, b, m, do = (t.detach().to(DEV) for t in (q, k, v, b, m, do))
+    low = [t.to(dtype) for t in (q, k, v, b)]
+    ref = orc.forward_backward(*(t.float() for t in low), m, do.to(dtype).float())
+    pt = orc.forward_backward(*low, m, do.to(dtype))
+    infos = {t: _lib.tile_info(_lib.KERNEL_BWD_B, t) for t in range(lib.trifast_num_tiles(_lib.KERNEL_BWD_B))}
+    two_key_tiles = [t for t, i in infos.items() if i["BLOCK_K"] // 32 == 2 * (i["num_waves"] // (i["BLOCK_J"] // 32))
+                     and lib.trifast_supports(_lib.KERNEL_BWD_B, t, n, h, d, code)]
+    plain_tile = max(t for t, i in infos.items() if i["num_waves"] == 16)
+    assert len(two_key_tiles) >= 2, infos
+    results = {}
+    for tile in [plain_tile] + two_key_tiles:
+        monkeypatch.setattr(tuner, "pick", lambda kern, n_, h_, d_, dt, launch, extra_cost=None, tile=tile:
+                            tile if kern == _lib.KERNEL_BWD_B else lib.trifast_default_tile(kern, n_, h_, d_, code))
+        out = kernel_fwd_bwd(*low, m, do.to(dtype))
+        check_all(out, pt, ref, dtype, f"db tile {tile} n={n} d={d} {pattern} {dtype}", directions=False)
+        results[tile] = out[NAMES.index("db")] if "db" in NAMES else out[-1]
+    for tile in two_key_tiles:
+        if pattern == "none" and n % 128 == 0:
+            # every block plain: the same arithmetic in the same order
+            assert torch.equal(results[tile], results[plain_tile]), f"db of tile {tile} differs from tile {plain_tile} ({pattern}, n={n})"
+        else:
+            # (-lse enters through a matrix instruction where the other tile adds it in the exponent)
+            err = (results[tile].float() - results[plain_tile].float()).abs().max().item()
+            assert err <= 2.0 ** -6 * results[plain_tile].float().abs().max().item(), f"db of tile {tile} vs tile {plain_tile}: {err} ({pattern}, n={n})"
+
+
+# ---------------------------------------------------------------------------
 # the row-resident backward (dq, dk, dv in one pass) at every size class it has:
 # 2 to 8 key tiles per wave, ragged sizes, masked keys, fully masked rows
 # ---------------------------------------------------------------------------

@@ -385,7 +385,8 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     }
   };
 
-  auto walk_rows = [&]() __attribute__((always_inline)) {
+  // the rows from `first_row` on (the loads and the row words stand at that row)
+  auto walk_rows = [&](int first_row) __attribute__((always_inline)) {
   if constexpr (NBUF >= 2) {
     // Ring of NBUF row buffers: the loads run NBUF-1 rows ahead of the compute, which
     // hides the memory latency behind several rows of work.  Row q lives in buffer
@@ -396,7 +397,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     for (int u = 0; u < P; ++u) issue_row(u);
     RowMeta meta = load_meta();
     sync_rows(std::integral_constant<int, P - 1>{});  // row 0 has landed
-    for (int r = 0; r < nrows; r += NBUF) {
+    for (int r = first_row; r < nrows; r += NBUF) {
 #pragma unroll
       for (int u = 0; u < NBUF; ++u) {
         if (r + u < nrows) {
@@ -410,7 +411,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     }
   } else {
     // one stage only (two do not fit in LDS): load, then compute
-    for (int ir = 0; ir < nrows; ++ir) {
+    for (int ir = first_row; ir < nrows; ++ir) {
       issue_row(0);
       const RowMeta meta = load_meta();
       sync_rows(std::integral_constant<int, 0>{});
@@ -419,35 +420,40 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
     }
   }
   };
-  // Workgroups of the 8-wave block whose rows are all plain (no flagged row, no masked key in
-  // any of the block's key tiles: the common case) walk the rows software-pipelined: a wave's
-  // matrix instructions of one tile are issued between the exponentials and multiply-adds of
-  // the tile before it (the second tile of a row overlaps the first, the first tile of the
-  // next row overlaps the second), so neither pipe waits for the other although only two
-  // waves share a SIMD.  The next row's operands are read from LDS a whole row ahead.
+  // Waves that own two key tiles (16-bit types, d <= 32) walk the plain rows at the start of
+  // the chunk (not flagged, no masked key in any of the block's key tiles: the common case)
+  // software-pipelined: a wave's matrix instructions of one tile are issued between the
+  // exponentials and multiply-adds of the tile before it (the second tile of a row overlaps
+  // the first, the first tile of the next row overlaps the second), so neither pipe waits
+  // for the other although only one or two waves share a SIMD.  The next row's operands are
+  // read from LDS a whole row ahead.  From the first row that is not plain on (padding: the
+  // rows past the valid length) the loop above takes over.  (The same walk with the masked
+  // form of the score needs about 290 registers per lane: it does not fit 8 waves.)
   constexpr bool kPipelined = WJ == 1 && WK == 2 && NBUF == 4 && sizeof(T) == 2 && D <= 32;
   if constexpr (kPipelined) {
-    bool mine = nrows > 0;
+    // the first row that is not plain: every thread looks at its share of the rows, the
+    // smallest index wins (through a word of LDS, which is not yet in use)
+    uint32_t* first_word = reinterpret_cast<uint32_t*>(tri_smem);
+    if (tid == 0) *first_word = (uint32_t)nrows;
+    __syncthreads();
     {
       const int w0 = k_blk / 32;
-      for (int i = i_begin + tid; i < i_end; i += NW * 64) {
-        mine = mine && a.rowflag[(int64_t)b * N + i] == 0;
-        const uint32_t* kw = a.keep + ((int64_t)b * N + i) * a.nwords;
+      for (int ir = tid; ir < nrows; ir += NW * 64) {
+        bool ok = a.rowflag[(int64_t)b * N + i_begin + ir] == 0;
+        const uint32_t* kw = a.keep + ((int64_t)b * N + i_begin + ir) * a.nwords;
 #pragma unroll
-        for (int w = 0; w < BKB / 32; ++w) mine = mine && (w0 + w < a.nwords ? kw[w0 + w] : 0u) == 0xffffffffu;
+        for (int w = 0; w < BKB / 32; ++w) ok = ok && (w0 + w < a.nwords ? kw[w0 + w] : 0u) == 0xffffffffu;
+        if (!ok) {
+          atomicMin(first_word, (uint32_t)ir);
+          break;
+        }
       }
     }
-    // all lanes of all waves agree: one word per wave through LDS (not yet in use)
-    uint32_t* votes = reinterpret_cast<uint32_t*>(tri_smem);
-    const bool wave_ok = __builtin_amdgcn_readfirstlane((int)(__ballot(mine) == ~0ull)) != 0;
-    if (lane == 0) votes[wave] = wave_ok ? 1u : 0u;
     __syncthreads();
-    bool plain = true;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) plain = plain && votes[w] != 0;
-    plain = __builtin_amdgcn_readfirstlane((int)plain) != 0;
+    int nplain = __builtin_amdgcn_readfirstlane((int)*first_word);
     __syncthreads();
-    if (plain) {
+    if (nplain < 2 * NBUF) nplain = 0;  // too few to fill the pipeline
+    if (nplain > 0) {
       struct RowOps {
         frag q[WJ][DS], dout[WJ][DS], k[WK][DS], v[WK][DS];
         frag df[WJ];    // -delta of the lane's query as a rank-1 operand
@@ -486,11 +492,12 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
         }
       };
       // The tiles of a wave in the order they are walked: tile t is (t / WK, t % WK).  The
-      // matrix instructions of tile `tn` of row `on` (scores from the bias tile, dP from
-      // -delta) go into sn / dpn, dealt between the elementwise work of tile `tc` of row
+      // matrix instructions of tile TN of row `on` (scores from the bias tile, dP from
+      // -delta) go into sn / dpn, dealt between the elementwise work of tile TC of row
       // `oc`, whose scores s and dP are complete: db += exp2(c s - lse) dP.
       constexpr int NT = WJ * WK;
-      constexpr int NM = 2 * DS + 1;
+      constexpr int NM = 2 * DS + 1;  // matrix instructions of a tile
+      static_assert(NT % 2 == 0, "the two accumulator sets swap once per tile");
       auto phase = [&](const RowOps& on, auto tn_tag, f32x16& sn, f32x16& dpn, const RowOps& oc, auto tc_tag, const f32x16& s,
                        const f32x16& dp, auto&& between) __attribute__((always_inline)) {
         constexpr int TN = decltype(tn_tag)::value, TC = decltype(tc_tag)::value;
@@ -523,6 +530,7 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
       f32x16 sc[2], dpc[2];  // scores and dP of the tile in flight and the tile being consumed
       read_ops(0, ops[0]);
       finish_ops(ops[0]);
+      // (the first tile of the first row has nothing to overlap with)
       sc[0] = E::mfma(ops[0].k[0][0], ops[0].q[0][0], biasr[0][0]);
 #pragma unroll
       for (int sd = 1; sd < DS; ++sd) sc[0] = E::mfma(ops[0].k[0][sd], ops[0].q[0][sd], sc[0]);
@@ -532,11 +540,10 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
       sc[1] = zero16();
       dpc[1] = zero16();
       sync_rows(std::integral_constant<int, AHEAD - 2>{});  // every wave has read row 0: its buffer is free
-      static_assert(NT % 2 == 0, "the two accumulator sets swap once per tile");
-      for (int r = 0; r < nrows; r += NBUF) {
+      for (int r = 0; r < nplain; r += NBUF) {
 #pragma unroll
         for (int u = 0; u < NBUF; ++u) {
-          if (r + u < nrows) {
+          if (r + u < nplain) {
             RowOps& cur = ops[u & 1];
             RowOps& next = ops[(u + 1) & 1];
             // row r + u + NBUF goes into the buffer whose row is in registers already; its
@@ -562,11 +569,22 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
           }
         }
       }
-    } else {
-      walk_rows();
+      if (nplain < nrows) {
+        // hand over: nothing in flight, the loads and the row words moved to row nplain
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const int at = min(rows_issued, nrows - 1);  // the row the loads stand at
+#pragma unroll
+        for (int x = 0; x < XN; ++x) item_base[x] += (int64_t)(nplain - at) * item_step[x];
+        rows_issued = nplain;
+        flag_word = (const_words)((uintptr_t)flag_word + (uintptr_t)((int64_t)nplain * 4));
+        keep_word = (const_words)((uintptr_t)keep_word + (uintptr_t)((int64_t)nplain * keep_step));
+        meta_rows = nplain;
+      }
     }
+    if (nplain < nrows) walk_rows(nplain);
   } else {
-    walk_rows();
+    walk_rows(0);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the spare rows loaded past the end
   if (wave_live == 0) return;
