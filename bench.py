@@ -40,6 +40,7 @@ MEASURED_TRAFFIC_MIB = {
     ("M", "_fwd", 7): 1537.0,
     ("M", "_bwd_kv", 10): 2563.8,
     ("M", "_bwd_b", 4): 1586.0,
+    ("M", "_bwd_b", 3): 1585.0,
 }
 
 # name -> (dtype, b, n, h, d, description)
