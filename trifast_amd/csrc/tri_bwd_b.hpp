@@ -32,6 +32,17 @@
 #include "tri_common.hpp"
 #include "tri_tile.hpp"
 
+// -DTRI_DB_TIMING builds the kernel as a probe of its pipelined walk
+// (benchmark/microbench/db_timeline.py): every wave reads the shader clock around the counted
+// wait and the barrier that end a row, and leaves per wave {clocks of the walk, clocks in the
+// wait, clocks in the barrier, 100 MHz ticks of the walk} where the db argument points; db
+// itself is not written.  -DTRI_DB_TIMING_LOADS=0 also takes the walk's global loads out (the
+// rows in LDS are then stale), =2 makes them read one row over and over (the same traffic from
+// L2 to LDS, none from memory): what the loads cost the arithmetic beside them.
+#if defined(TRI_DB_TIMING) && !defined(TRI_DB_TIMING_LOADS)
+#define TRI_DB_TIMING_LOADS 1
+#endif
+
 namespace tri {
 
 // LDS bytes of one stage (one pair row) of the kernel below
@@ -193,7 +204,11 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
   // the same, one item at a time (for loops that deal the loads of a row between other work);
   // next_row_advance() once per row, before its items
   auto next_row_advance = [&]() __attribute__((always_inline)) -> int64_t {
+#if defined(TRI_DB_TIMING) && TRI_DB_TIMING_LOADS == 2
+    const int64_t advance = ones_while_positive(0);
+#else
     const int64_t advance = ones_while_positive(nrows - 1 - rows_issued);
+#endif
     ++rows_issued;
     return advance;
   };
@@ -540,6 +555,10 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
       sc[1] = zero16();
       dpc[1] = zero16();
       sync_rows(std::integral_constant<int, AHEAD - 2>{});  // every wave has read row 0: its buffer is free
+#ifdef TRI_DB_TIMING
+      uint64_t t_wait = 0, t_barrier = 0;
+      const uint64_t t_clk0 = __builtin_amdgcn_s_memtime(), t_real0 = __builtin_amdgcn_s_memrealtime();
+#endif
       for (int r = 0; r < nplain; r += NBUF) {
 #pragma unroll
         for (int u = 0; u < NBUF; ++u) {
@@ -554,7 +573,9 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
               constexpr int slot = decltype(slot_tag)::value;
               static_for<XN>([&](auto xt) __attribute__((always_inline)) {
                 constexpr int x = decltype(xt)::value;
+#if !defined(TRI_DB_TIMING) || TRI_DB_TIMING_LOADS != 0
                 if constexpr (slot == (x * NT * NM) / XN) issue_item(u, xt, advance);
+#endif
               });
             };
             read_ops((u + 1) % NBUF, next);
@@ -565,10 +586,37 @@ __global__ __launch_bounds__(GJ * GK * 64) void tri_bwd_b_kernel(const BwdArgs a
             });
             finish_ops(next);
             phase(next, std::integral_constant<int, 0>{}, sc[0], dpc[0], cur, std::integral_constant<int, NT - 1>{}, sc[(NT - 1) & 1], dpc[(NT - 1) & 1], deal_loads);
+#ifdef TRI_DB_TIMING
+            {
+              const uint64_t m0 = __builtin_amdgcn_s_memtime();
+              asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"((AHEAD - 2) * XN) : "memory");
+              const uint64_t m1 = __builtin_amdgcn_s_memtime();
+              asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+              const uint64_t m2 = __builtin_amdgcn_s_memtime();
+              asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+              t_wait += m1 - m0;
+              t_barrier += m2 - m1;
+            }
+#else
             sync_rows(std::integral_constant<int, AHEAD - 2>{});  // rows up to r + u + 2 have landed
+#endif
           }
         }
       }
+#ifdef TRI_DB_TIMING
+      {
+        const uint64_t t_clk1 = __builtin_amdgcn_s_memtime(), t_real1 = __builtin_amdgcn_s_memrealtime();
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        if (lane == 0) {
+          uint64_t* rec = reinterpret_cast<uint64_t*>(a.db) + ((int64_t)L * NW + wave) * 4;
+          rec[0] = t_clk1 - t_clk0;
+          rec[1] = t_wait;
+          rec[2] = t_barrier;
+          rec[3] = t_real1 - t_real0;
+        }
+        return;
+      }
+#endif
       if (nplain < nrows) {
         // hand over: nothing in flight, the loads and the row words moved to row nplain
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
