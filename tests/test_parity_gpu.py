@@ -147,6 +147,84 @@ def test_every_tile(n, h, d, dtype, monkeypatch):
 
 
 # ---------------------------------------------------------------------------
+# the forward's scheduled loop with masked keys (tiles of two and four pair rows, n a multiple
+# of 32, no fully masked row in the workgroup): a random mask, padding (the workgroups with
+# rows past the valid length take the general loop, the others stop at the last attended key
+# tile), key tiles without an attended key at the start (the softmax reference starts on
+# masked scores) and in the middle, rows that attend to a single key.
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("pattern", ["random", "padding", "first_dead", "middle_dead", "one_key"])
+@pytest.mark.parametrize("n,h,d", [(256, 2, 32), (128, 1, 16), (160, 1, 32)])
+def test_forward_scheduled_loop_masked(n, h, d, pattern, dtype, monkeypatch):
+    lib = _lib.load()
+    code = tt._DTYPE_CODE[dtype]
+    g = torch.Generator().manual_seed(3 * n + d)
+    q, k, v, b, m = orc.gen_tensors(n, d, h, pattern == "random", "cpu", torch.float32, 1, 1.0, generator=g)
+    if pattern == "random":
+        m[:, :, 0] &= ~m.all(dim=-1)  # (no fully masked row)
+    elif pattern == "padding":
+        valid = n - 37
+        m[:, valid:, :] = True
+        m[:, :, valid:] = True
+    elif pattern == "first_dead":
+        m[:, :, :64] = True
+        m[:, 7, 70:] = True  # a row whose attended keys end early
+    elif pattern == "middle_dead":
+        m[:, :, 64:96] = True
+    elif pattern == "one_key":
+        m[:] = True
+        m[0, torch.arange(n), torch.randint(0, n, (n,), generator=g)] = False
+    do = torch.randn(q.shape, generator=g)
+    q, k, v, b, m, do = (t.detach().to(DEV) for t in (q, k, v, b, m, do))
+    low = [t.to(dtype) for t in (q, k, v, b)]
+    ref = orc.forward_backward(*(t.float() for t in low), m, do.to(dtype).float())
+    pt = orc.forward_backward(*low, m, do.to(dtype))
+    scheduled = [t for t in range(lib.trifast_num_tiles(_lib.KERNEL_FWD)) if t >= 6 and lib.trifast_supports(_lib.KERNEL_FWD, t, n, h, d, code)]
+    assert len(scheduled) == 2, "tiles 6 and 7 are the forward's scheduled loop"
+    for tile in scheduled:
+        monkeypatch.setattr(tuner, "pick", lambda kern, n_, h_, d_, dt, launch, extra_cost=None, tile=tile:
+                            tile if kern == _lib.KERNEL_FWD else lib.trifast_default_tile(kern, n_, h_, d_, code))
+        out = kernel_fwd_bwd(*low, m, do.to(dtype))
+        tag = f"fwd tile {tile} n={n} d={d} {pattern} {dtype}"
+        check_all(out, pt, ref, dtype, tag, directions=False)
+        check_lse(low, m, dtype, tag)
+
+
+# ---------------------------------------------------------------------------
+# more than 32 key tiles with the first 32 of them plain: the bitmaps over the key tiles are
+# 64-bit words put together from two 32-bit halves, and a low half with its top bit set once
+# spilled into the high half (tiles 32.. then passed for plain and live).  Padding at n = 1088:
+# tile 31 has no masked key, tile 33 has; the forward and the dq kernel (three-kernel backward
+# forced in the second pass) read those bitmaps.
+# ---------------------------------------------------------------------------
+def test_key_tile_bitmaps_past_32_tiles(monkeypatch):
+    lib = _lib.load()
+    n, h, d, dtype = 1088, 1, 32, torch.bfloat16
+    code = tt._DTYPE_CODE[dtype]
+    g = torch.Generator().manual_seed(n)
+    q, k, v, b, m = orc.gen_tensors(n, d, h, False, "cpu", torch.float32, 1, 1.0, generator=g)
+    valid = 1060
+    m[:, valid:, :] = True
+    m[:, :, valid:] = True
+    do = torch.randn(q.shape, generator=g)
+    q, k, v, b, m, do = (t.detach().to(DEV) for t in (q, k, v, b, m, do))
+    low = [t.to(dtype) for t in (q, k, v, b)]
+    ref = oracle_fwd_bwd(*(t.float() for t in low), m, do.to(dtype).float(), 64)
+    pt = oracle_fwd_bwd(*low, m, do.to(dtype), 64)
+    out = kernel_fwd_bwd(*low, m, do.to(dtype))
+    check_all(out, pt, ref, dtype, f"n={n} padding to {valid}, default tiles", directions=False)
+    check_lse(low, m, dtype, f"n={n} padding to {valid}")
+    # the same with the dq and dk/dv kernels instead of the row-resident one
+    kv = next(t for t in range(lib.trifast_num_tiles(_lib.KERNEL_BWD_KV))
+              if not lib.trifast_bwd_kv_tile_writes_dq(t) and lib.trifast_supports(_lib.KERNEL_BWD_KV, t, n, h, d, code))
+    real_pick = tuner.pick
+    monkeypatch.setattr(tuner, "pick", lambda kern, *a, **kw: kv if kern == _lib.KERNEL_BWD_KV else real_pick(kern, *a, **kw))
+    out = kernel_fwd_bwd(*low, m, do.to(dtype))
+    check_all(out, pt, ref, dtype, f"n={n} padding to {valid}, three-kernel backward", directions=False)
+
+
+# ---------------------------------------------------------------------------
 # the db kernel's pipelined walk of plain rows (blocks whose waves own two key tiles) and
 # its hand-over to the general loop at the first row that is not plain: no mask at all,
 # padding (keys and rows past a valid length), one masked row in the middle, a masked row

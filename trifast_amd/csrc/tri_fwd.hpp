@@ -375,9 +375,13 @@ __global__ __launch_bounds__(NW * 64, (R * ((BKF % kFwdFast) / 32) >= 8) ? 1 : 2
   //     stage: its packed words are the B operand against a constant A operand that holds
   //     sqrt(d) where the contraction slot is the row's key (sqrt(32) as hi + lo parts), and
   //     the product is the accumulator init of the score MFMAs of the R rows.
-  auto fast_loop = [&]() __attribute__((always_inline)) {
+  // masked_tag: the rows have masked keys (none of them is fully masked): every tile takes one
+  // more MFMA, which gives the masked keys a large negative score, and the stages after the
+  // last one with an attended key are left out
+  auto fast_loop = [&](auto masked_tag) __attribute__((always_inline)) {
     static_assert(!FAST || (sizeof(T) == 2 && BK == 32 && R >= 2), "16-bit types, 32-key stages, two or more pair rows");
     if constexpr (FAST) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
     typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
     typedef T pair_t __attribute__((ext_vector_type(2)));
     constexpr int NS = fwd_fast_stages(R);
@@ -388,7 +392,22 @@ __global__ __launch_bounds__(NW * 64, (R * ((BKF % kFwdFast) / 32) >= 8) ? 1 : 2
     constexpr int XN = G / NW;
     constexpr int NLD = XN + 2;  // loads per wave and stage: its share of K and V, its bias tile
     auto SB = [] { __builtin_amdgcn_sched_barrier(0); };
-    const int ns = N >> 5;
+    const int ns = MASKED ? masks.last_live() : N >> 5;
+    // the keep words of the stage in use and of the next one, one per pair row (wave-uniform:
+    // scalar loads, issued a stage ahead of their use)
+    uint32_t kwc[R], kwn[R];
+    auto fetch_keep_words = [&](int stage, uint32_t* kw) __attribute__((always_inline)) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) kw[r] = MASKED ? uniform_word(keep_row[r], min(stage, a.nwords - 1)) : 0xffffffffu;
+    };
+    if constexpr (MASKED) {
+      kop.init(perm32(jl), g);
+      typename OffsetMask<T>::Queries qz;
+      qz.init(split_word<T>(0.f), g);
+      qzero = qz.get();
+      fetch_keep_words(0, kwc);
+      fetch_keep_words(1, kwn);
+    }
 
     // this wave's loads of a stage: a 32-bit byte offset per lane from the stage's first K / V row
     uint32_t lofs[XN];
@@ -498,11 +517,12 @@ __global__ __launch_bounds__(NW * 64, (R * ((BKF % kFwdFast) / 32) >= 8) ? 1 : 2
       for (int x = 0; x < NB; ++x)
         bias_s = E::mfma(bsel[x / NPART][x % NPART], lds_frag(ab + (x / NPART) * 1024), bias_s);
       sc_cur = bias_s;
+      if constexpr (MASKED) sc_cur = E::mfma(kop.masked(kwc[0]), qzero, sc_cur);
 #pragma unroll
       for (int sd = 0; sd < DS; ++sd) sc_cur = E::mfma(lds_frag(ak[sd]), qf[0][sd], sc_cur);
     }
 
-    enum { F_B, F_PV, F_S };
+    enum { F_B, F_PV, F_S, F_M };
     // (the loop exists twice: for waves with queries, and for the waves past the end of the pair
     // row, which only take part in the loads and barriers; one loop with the test inside would
     // make the compiler copy the state where the two cases meet)
@@ -519,15 +539,16 @@ __global__ __launch_bounds__(NW * 64, (R * ((BKF % kFwdFast) / 32) >= 8) ? 1 : 2
         constexpr bool last_r = r == R - 1;
         constexpr int rn = (r + 1) % R, rp = (r + R - 1) % R;
         constexpr int NPV = PS * DM;
-        constexpr int NM = DS + NPV + (last_r ? NB : 0);
+        constexpr int NM = DS + NPV + (last_r ? NB : 0) + (MASKED ? 1 : 0);
         constexpr int NU = 8;
-        // MFMA order: the P.V products of the last tile, (the bias products,) the score products
+        // MFMA order: the P.V products of the last tile, (the bias products,) (the key mask,) the score products
         struct Order { int kind[NM], idx[NM]; };
         constexpr Order ord = [] {
           Order o{};
           int n = 0;
           for (int i = 0; i < NPV; ++i) { o.kind[n] = F_PV; o.idx[n++] = i; }
           if (last_r) for (int i = 0; i < NB; ++i) { o.kind[n] = F_B; o.idx[n++] = i; }
+          if (MASKED) { o.kind[n] = F_M; o.idx[n++] = 0; }
           for (int i = 0; i < DS; ++i) { o.kind[n] = F_S; o.idx[n++] = i; }
           return o;
         }();
@@ -549,6 +570,11 @@ __global__ __launch_bounds__(NW * 64, (R * ((BKF % kFwdFast) / 32) >= 8) ? 1 : 2
           }
           SB();
           f32x16 sc_next, bias_next = zero16();
+          frag mk;
+          if constexpr (MASKED) {
+            // keys operand of the next tile's mask product (the next row of this stage, or the first row of the next)
+            mk = kop.masked(last_r ? kwn[0] : kwc[rn]);
+          }
           uint32_t pw[NU];
           const float mcr = mc[r], l_old = lrun[r];
           float l_new = l_old;  // the running row sum with this tile's probabilities on top
@@ -582,8 +608,10 @@ __global__ __launch_bounds__(NW * 64, (R * ((BKF % kFwdFast) / 32) >= 8) ? 1 : 2
             } else if constexpr (kind == F_PV) {
               constexpr int s2 = idx / DM, mt = idx % DM;
               oacc[rp][mt] = E::mfma(vf_prev[mt][s2], pf_prev[s2], oacc[rp][mt]);
+            } else if constexpr (kind == F_M) {
+              sc_next = E::mfma(mk, qzero, last_r ? bias_next : bias_s);
             } else {
-              if constexpr (idx == 0) sc_next = E::mfma(kf[0], qf[rn][0], last_r ? bias_next : bias_s);
+              if constexpr (idx == 0 && !MASKED) sc_next = E::mfma(kf[0], qf[rn][0], last_r ? bias_next : bias_s);
               else sc_next = E::mfma(kf[idx], qf[rn][idx], sc_next);
             }
             SB();
@@ -610,7 +638,13 @@ __global__ __launch_bounds__(NW * 64, (R * ((BKF % kFwdFast) / 32) >= 8) ? 1 : 2
 #pragma unroll
             for (int v = 2; v < 16; ++v) mx = fmaxf(mx, sc_cur[v]);
             mx = half_max(mx);
-            const float mcn = fmaxf(mc[r], mx * c);
+            // A row that attends to no key of this tile (the same for all its queries): every
+            // score is the mask value alone.  The tile then adds nothing and must not become
+            // the reference: exp2(c * score - reference) would be exp2 of the rounding error of
+            // two numbers of the mask value's size.  (With a reference from real scores such a
+            // tile's probabilities are exactly zero and it never gets here.)
+            const bool no_key = MASKED && mx < 2.0f * E::kMaskElem;
+            const float mcn = no_key ? mc[r] : fmaxf(mc[r], mx * c);
             const float alpha = fast_exp2(mc[r] - mcn);
 #pragma unroll
             for (int mt = 0; mt < DM; ++mt)
@@ -620,8 +654,9 @@ __global__ __launch_bounds__(NW * 64, (R * ((BKF % kFwdFast) / 32) >= 8) ? 1 : 2
             l_new = l_old * alpha;
 #pragma unroll
             for (int u = 0; u < NU; ++u) {
-              const float p0 = fast_exp2(__builtin_fmaf(sc_cur[2 * u], c, -mcn));
-              const float p1 = fast_exp2(__builtin_fmaf(sc_cur[2 * u + 1], c, -mcn));
+              const float e0 = fast_exp2(__builtin_fmaf(sc_cur[2 * u], c, -mcn));
+              const float e1 = fast_exp2(__builtin_fmaf(sc_cur[2 * u + 1], c, -mcn));
+              const float p0 = no_key ? 0.f : e0, p1 = no_key ? 0.f : e1;
               const pair_t w = {(T)p0, (T)p1};
               pw[u] = __builtin_bit_cast(uint32_t, w);
               l_new = pair_sum(w, ones, l_new);
@@ -636,6 +671,11 @@ __global__ __launch_bounds__(NW * 64, (R * ((BKF % kFwdFast) / 32) >= 8) ? 1 : 2
           }
           sc_cur = sc_next;
           if constexpr (last_r) bias_s = bias_next;
+        }
+        if constexpr (MASKED && last_r) {
+#pragma unroll
+          for (int r2 = 0; r2 < R; ++r2) kwc[r2] = kwn[r2];
+          fetch_keep_words(stage + 2, kwn);
         }
         // The next slot reads stage s+1: every wave's loads of it have landed (a ring of four
         // leaves one younger stage in flight), and nobody reads stage s-1 any more: the buffer
@@ -698,16 +738,21 @@ __global__ __launch_bounds__(NW * 64, (R * ((BKF % kFwdFast) / 32) >= 8) ? 1 : 2
     }
   };
   // (a last stage with fewer than KU key tiles is not plain: its missing tiles are masked)
-  bool fast = false;
+  bool fast = false, fast_masked = false;
   if constexpr (FAST) {
     // (the per-lane offsets of the stage loads are 32-bit: rows and keys of a stage must lie within 4 GiB)
     const auto fits = [&](const Str5& st) {
       return st.i >= 0 && st.j >= 0 && (uint64_t)(R - 1) * st.i + 31ull * st.j + D < (1ull << 31) / sizeof(T);
     };
-    fast = masks.all_plain() && (N & 31) == 0 && fits(a.sk) && fits(a.sv);
+    const bool shape_fits = (N & 31) == 0 && fits(a.sk) && fits(a.sv);
+    fast = shape_fits && masks.all_plain();
+    // (a fully masked row drops its bias and q.k: such workgroups take the general loop)
+    fast_masked = shape_fits && !fast && !any_flagged && masks.last_live() > 0;
   }
   if (fast) {
-    if constexpr (FAST) fast_loop();
+    if constexpr (FAST) fast_loop(std::false_type{});
+  } else if (fast_masked) {
+    if constexpr (FAST) fast_loop(std::true_type{});
   } else {
     setup_general();
     if (masks.all_plain() && ntiles % KU == 0) stage_loop(std::integral_constant<int, kPlain>{});

@@ -314,6 +314,14 @@ TRI_DEV f32x16 bias_tile(const T* pack_bh, int NP, int jt, int kt, int lane, flo
 //   plain = every row attends to every key of the tile (no mask work at all).
 // The words of the 64-tile chunk in use are cached in scalar registers, so the
 // per-stage queries are scalar bit operations.
+// A 64-bit word that every lane holds, as a wave-uniform value (the two halves go through
+// readfirstlane, whose result is a signed int: each half is widened as unsigned).
+TRI_DEV uint64_t uniform_u64(uint64_t x) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)x);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(x >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
 struct KeyTileMasks {
   const uint64_t* words;  // LDS: [nchunks] live, then [nchunks] plain
   int nchunks, ntiles, cur;
@@ -351,8 +359,8 @@ struct KeyTileMasks {
     if (ch == cur) return;
     cur = ch;
     const uint64_t lv = words[ch], pl = words[nchunks + ch];
-    live = ((uint64_t)__builtin_amdgcn_readfirstlane((uint32_t)(lv >> 32)) << 32) | __builtin_amdgcn_readfirstlane((uint32_t)lv);
-    plain = ((uint64_t)__builtin_amdgcn_readfirstlane((uint32_t)(pl >> 32)) << 32) | __builtin_amdgcn_readfirstlane((uint32_t)pl);
+    live = uniform_u64(lv);
+    plain = uniform_u64(pl);
   }
   // first stage of KU tiles at or after tile t (t % KU == 0) with a live tile; ntiles if none
   template <int KU>
@@ -368,6 +376,17 @@ struct KeyTileMasks {
     }
     return ntiles;
   }
+  // one past the last key tile with an attended key, 0 if there is none (wave-uniform; reads
+  // the bitmaps from LDS)
+  TRI_DEV int last_live() const {
+    int last = 0;
+    for (int ch = 0; ch < nchunks; ++ch) {
+      const uint64_t lv = words[ch];
+      const uint64_t u = uniform_u64(lv);
+      if (u != 0) last = 64 * ch + 64 - __builtin_clzll(u);
+    }
+    return last;
+  }
   // every key tile is plain (wave-uniform; reads the bitmaps from LDS)
   TRI_DEV bool all_plain() const {
     bool all = true;
@@ -375,7 +394,7 @@ struct KeyTileMasks {
       const int nt = min(64, ntiles - 64 * ch);
       const uint64_t want = nt == 64 ? ~0ull : ((1ull << nt) - 1);
       const uint64_t pl = words[nchunks + ch];
-      const uint64_t u = ((uint64_t)__builtin_amdgcn_readfirstlane((uint32_t)(pl >> 32)) << 32) | __builtin_amdgcn_readfirstlane((uint32_t)pl);
+      const uint64_t u = uniform_u64(pl);
       all = all && (u & want) == want;
     }
     return all;
