@@ -196,17 +196,22 @@ def test_forward_scheduled_loop_masked(n, h, d, pattern, dtype, monkeypatch):
 # 64-bit words put together from two 32-bit halves, and a low half with its top bit set once
 # spilled into the high half (tiles 32.. then passed for plain and live).  Padding at n = 1088:
 # tile 31 has no masked key, tile 33 has; the forward and the dq kernel (three-kernel backward
-# forced in the second pass) read those bitmaps.
+# forced in the second pass) read those bitmaps.  At n = 2112 a bitmap is two words.
 # ---------------------------------------------------------------------------
-def test_key_tile_bitmaps_past_32_tiles(monkeypatch):
+@pytest.mark.parametrize("n,valid", [(1088, 1060), (2112, 2090)], ids=["34_tiles", "66_tiles"])
+def test_key_tile_bitmaps_past_32_tiles(n, valid, monkeypatch):
     lib = _lib.load()
-    n, h, d, dtype = 1088, 1, 32, torch.bfloat16
+    h, d, dtype = 1, 32, torch.bfloat16
     code = tt._DTYPE_CODE[dtype]
     g = torch.Generator().manual_seed(n)
     q, k, v, b, m = orc.gen_tensors(n, d, h, False, "cpu", torch.float32, 1, 1.0, generator=g)
-    valid = 1060
     m[:, valid:, :] = True
     m[:, :, valid:] = True
+    if n > 2048:
+        # (two 64-bit words per bitmap) a row without an attended key in the first word's tiles,
+        # and one whose attended keys end in the first word
+        m[:, 9, :2050] = True
+        m[:, 70, 1000:] = True
     do = torch.randn(q.shape, generator=g)
     q, k, v, b, m, do = (t.detach().to(DEV) for t in (q, k, v, b, m, do))
     low = [t.to(dtype) for t in (q, k, v, b)]
