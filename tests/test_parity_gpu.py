@@ -231,6 +231,69 @@ def test_structured_masks(n, h, d, pattern, dtype):
 
 
 # ---------------------------------------------------------------------------
+# seeded mixtures: shape, dtype, batch, layout (contiguous, i<->j transposed views, the
+# heads-interleaved [b, n, n, h, d] storage of a projection seen as [b, h, n, n, d]) and a
+# structured mask per batch element (padding to its own length, a band, blocks on the
+# diagonal, dead key ranges, dead leading keys per row), through the default tiles.
+# ---------------------------------------------------------------------------
+def _structured_mask(kind, bs, n, g):
+    m = torch.zeros(bs, n, n, dtype=torch.bool)
+    idx = torch.arange(n)
+    for bi in range(bs):
+        if kind == "padding":
+            valid = int(torch.randint(max(1, n // 2), n + 1, (1,), generator=g))
+            m[bi, valid:, :] = True
+            m[bi, :, valid:] = True
+        elif kind == "band":
+            w = int(torch.randint(1, max(2, n // 3), (1,), generator=g))
+            m[bi] = (idx[:, None] - idx[None, :]).abs() > w
+        elif kind == "blocks":
+            size = int(torch.randint(8, max(9, n // 2), (1,), generator=g))
+            m[bi] = (idx[:, None] // size) != (idx[None, :] // size)
+        elif kind == "dead_ranges":
+            for _ in range(3):
+                lo = int(torch.randint(0, n, (1,), generator=g))
+                m[bi, :, lo:lo + int(torch.randint(1, 80, (1,), generator=g))] = True
+            m[bi, :, int(torch.randint(0, n, (1,), generator=g))] = False  # (every row keeps a key)
+        elif kind == "leading":
+            first = torch.randint(0, n, (n,), generator=g)
+            m[bi] = idx[None, :] < first[:, None]
+    return m
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_seeded_mixtures(seed):
+    g = torch.Generator().manual_seed(9000 + seed)
+    pick = lambda xs: xs[int(torch.randint(0, len(xs), (1,), generator=g))]
+    n = int(torch.randint(33, 420, (1,), generator=g))
+    if pick([0, 1]):
+        n = n // 32 * 32  # (whole key tiles: the scheduled loops)
+    h, d, bs = pick([1, 2, 3]), pick([16, 32, 64]), pick([1, 2])
+    dtype = pick([torch.bfloat16, torch.float16, torch.float32])
+    kind = pick(["padding", "band", "blocks", "dead_ranges", "leading"])
+    layout = pick(["contiguous", "transposed", "heads_interleaved"])
+    q, k, v, b, _ = orc.gen_tensors(n, d, h, False, "cpu", torch.float32, bs, 1.0, generator=g)
+    m = _structured_mask(kind, bs, n, g)
+    do = torch.randn(q.shape, generator=g)
+    q, k, v, b, m, do = (t.detach().to(DEV) for t in (q, k, v, b, m, do))
+    low = [t.to(dtype) for t in (q, k, v, b)]
+    do = do.to(dtype)
+    if layout == "transposed":
+        # the same values behind views whose i and j strides are swapped
+        low = [t.transpose(2, 3).contiguous().transpose(2, 3) for t in low[:3]] + [low[3].transpose(-1, -2).contiguous().transpose(-1, -2)]
+    elif layout == "heads_interleaved":
+        low = [t.permute(0, 2, 3, 1, 4).contiguous().permute(0, 3, 1, 2, 4) for t in low[:3]] + [low[3].permute(0, 2, 3, 1).contiguous().permute(0, 3, 1, 2)]
+    chunk = 64 if n > 300 else None
+    ref = oracle_fwd_bwd(*(t.float() for t in low), m, do.float(), chunk)
+    pt = oracle_fwd_bwd(*low, m, do, chunk)
+    out = kernel_fwd_bwd(*low, m, do)
+    tag = f"seed {seed}: n={n} h={h} d={d} bs={bs} {dtype} {kind} {layout}"
+    # (rows with one attended key give gradients that are zero by cancellation: see test_structured_masks)
+    check_all(out, pt, ref, dtype, tag, directions=False, rel_floor=16.0 if kind in ("band", "blocks", "leading") else 1e-30)
+    check_lse(low, m, dtype, tag)
+
+
+# ---------------------------------------------------------------------------
 # more than 32 key tiles with the first 32 of them plain: the bitmaps over the key tiles are
 # 64-bit words put together from two 32-bit halves, and a low half with its top bit set once
 # spilled into the high half (tiles 32.. then passed for plain and live).  Padding at n = 1088:
