@@ -19,6 +19,10 @@
 // with masked keys -lse moves to an extra MFMA that it shares with the key mask (see
 // OffsetMask): masked keys get a large negative score there.
 //
+// Waves that own two key tiles walk the plain rows at the start of a chunk as a hand-made
+// software pipeline (matrix instructions of one tile between the vector instructions of the
+// tile before it, operands a row ahead); see kPipelined below.
+//
 // All workgroups of one (batch*head, chunk) read the same rows at about the same
 // time; the block index is remapped so that they run on one XCD and share its L2.
 // When the rows are split into several chunks (to fill the GPU), each chunk writes

@@ -27,7 +27,8 @@
 // skipped) and whether all of them are plain (every row attends to every key:
 // the workgroup then runs a loop with no mask work and no per-tile branch).
 // Otherwise a masked key gets a large negative score through one extra MFMA
-// (see OffsetMask).
+// (see OffsetMask).  The scheduled loop further down exists in both forms; workgroups with
+// a fully masked row, ragged n and fp32 take the general stage loop.
 //
 // Replaces _fwd of reference src/trifast/triton.py:19-132.
 #pragma once
@@ -359,7 +360,7 @@ __global__ __launch_bounds__(NW * 64, (R * ((BKF % kFwdFast) / 32) >= 8) ? 1 : 2
       if (t + 1 < TS) sc = sn;
     }
   };
-  // ---- the scheduled loop: workgroups whose rows attend to every key ------------------------
+  // ---- the scheduled loop: workgroups without a fully masked row, n a multiple of 32 ----------
   // Same work as the plain stage loop above, laid out as the schedule it should run in.  A
   // wave issues in order, so everything a tile needs is asked for a whole tile ahead:
   //   * a ring of three or four 32-key stages (K rows, V rows and the waves' packed bias
